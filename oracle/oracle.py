@@ -1,0 +1,206 @@
+"""ctypes binding of the CPU oracle (oracle/libnvfp4_oracle.so).  TEST INFRASTRUCTURE ONLY.
+
+Only tests, ``__graft_entry__.smoke()`` and the ``cpu_baseline`` leg of ``bench.py`` import this
+module; the product package never does.  ``build()`` compiles the C restatement with the
+Makefile beside this file; ``lib()`` loads what is built (and builds it if nothing is).
+"""
+from __future__ import annotations
+
+import ctypes as C
+import os
+import subprocess
+
+import numpy as np
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+_SO = os.path.join(_HERE, "libnvfp4_oracle.so")
+_lib = None
+
+u8p = np.ctypeslib.ndpointer(np.uint8, flags="C_CONTIGUOUS")
+f32p = np.ctypeslib.ndpointer(np.float32, flags="C_CONTIGUOUS")
+f64p = np.ctypeslib.ndpointer(np.float64, flags="C_CONTIGUOUS")
+i32p = np.ctypeslib.ndpointer(np.int32, flags="C_CONTIGUOUS")
+
+
+def build() -> None:
+    subprocess.run(["make", "-C", _HERE, "-B", "libnvfp4_oracle.so"], check=True, capture_output=True)
+
+
+def lib():
+    global _lib
+    if _lib is not None:
+        return _lib
+    if not os.path.exists(_SO):
+        build()
+    L = C.CDLL(_SO)
+    sz, f, i = C.c_size_t, C.c_float, C.c_int
+    L.orc_e2m1.restype = f
+    L.orc_e2m1.argtypes = [C.c_uint32]
+    L.orc_ue4m3.restype = f
+    L.orc_ue4m3.argtypes = [C.c_uint32]
+    L.orc_scale_rule.restype = C.c_uint8
+    L.orc_scale_rule.argtypes = [C.c_uint8]
+    L.orc_scale_lut.argtypes = [f, f32p]
+    L.orc_dequant_raw.argtypes = [u8p, sz, f, f32p]
+    L.orc_dequant.argtypes = [u8p, sz, f, f32p]
+    L.orc_byte_len.restype = sz
+    L.orc_byte_len.argtypes = [sz, sz]
+    L.orc_encode_ue4m3_ceil.restype = C.c_uint32
+    L.orc_encode_ue4m3_ceil.argtypes = [f]
+    L.orc_quantize_ceil.restype = f
+    L.orc_quantize_ceil.argtypes = [f32p, sz, u8p]
+    L.orc_gemv.restype = i
+    L.orc_gemv.argtypes = [u8p, sz, sz, f, f32p, sz, f32p, i, i]
+    L.orc_expert_ffn.restype = i
+    L.orc_expert_ffn.argtypes = [u8p, f, u8p, f, u8p, f, sz, sz, f32p, sz, f32p, i, i]
+    L.orc_ffn_clamped.restype = i
+    L.orc_ffn_clamped.argtypes = [u8p, f, u8p, f, u8p, f, sz, sz, f, f32p, sz, f32p, i, i]
+    L.orc_gemv_f64.argtypes = [u8p, sz, sz, f, f32p, sz, i, f64p, f64p]
+    L.orc_gamma.restype = C.c_double
+    L.orc_gamma.argtypes = [sz]
+    L.orc_silu_mul.restype = f
+    L.orc_silu_mul.argtypes = [f, f]
+    L.orc_silu_mul_combo.argtypes = [f32p, sz, sz, f32p]
+    L.orc_acc_combo.argtypes = [f32p, f32p, sz, sz, sz, f32p]
+    L.orc_router_topk.argtypes = [f32p, sz, sz, sz, i32p, f32p]
+    L.orc_argmax_ref.restype = C.c_int32
+    L.orc_argmax_ref.argtypes = [f32p, sz]
+    L.orc_moe_layer.restype = i
+    L.orc_moe_layer.argtypes = [u8p, f, u8p, f, sz, sz, sz, f32p, f32p, sz, sz, i32p, f32p, f32p, i, i]
+    L.orc_f32_to_bf16.restype = C.c_uint16
+    L.orc_f32_to_bf16.argtypes = [f]
+    _lib = L
+    return L
+
+
+def _u8(a):
+    return np.ascontiguousarray(a, dtype=np.uint8).reshape(-1)
+
+
+def _f32(a):
+    return np.ascontiguousarray(a, dtype=np.float32)
+
+
+def byte_len(rows: int, cols: int) -> int:
+    return rows * (cols // 64) * 36
+
+
+def e2m1(n: int) -> float:
+    return lib().orc_e2m1(n)
+
+
+def ue4m3(b: int) -> float:
+    return lib().orc_ue4m3(b)
+
+
+def scale_lut(gs: float) -> np.ndarray:
+    out = np.zeros(256, np.float32)
+    lib().orc_scale_lut(gs, out)
+    return out
+
+
+def dequant(blocks, gs: float, rule: bool = True) -> np.ndarray:
+    b = _u8(blocks)
+    assert b.size % 36 == 0
+    out = np.empty(b.size // 36 * 64, np.float32)
+    (lib().orc_dequant if rule else lib().orc_dequant_raw)(b, b.size // 36, gs, out)
+    return out
+
+
+def quantize_ceil(values) -> tuple[np.ndarray, float]:
+    v = _f32(values).reshape(-1)
+    assert v.size % 64 == 0
+    out = np.empty(v.size // 64 * 36, np.uint8)
+    gs = lib().orc_quantize_ceil(v, v.size, out)
+    return out, float(np.float32(gs))
+
+
+def gemv(w, rows: int, cols: int, gs: float, x, threads: int = 1, path: int = 1) -> np.ndarray:
+    wb = _u8(w)
+    if cols == 0 or cols % 64 != 0:
+        raise ValueError(f"cpu_nvfp4: {cols} columns are not whole 64-value NVFP4 blocks")
+    if wb.size != byte_len(rows, cols):
+        raise ValueError(f"cpu_nvfp4: [{rows}, {cols}] needs {byte_len(rows, cols)} B, got {wb.size}")
+    xv = _f32(x).reshape(-1, cols)
+    y = np.empty((xv.shape[0], rows), np.float32)
+    rc = lib().orc_gemv(wb, rows, cols, gs, xv, xv.shape[0], y, threads, path)
+    assert rc == 0
+    return y
+
+
+def gemv_f64(w, rows: int, cols: int, gs: float, x, rule: bool = True):
+    wb = _u8(w)
+    xv = _f32(x).reshape(-1, cols)
+    y = np.empty((xv.shape[0], rows), np.float64)
+    a = np.empty((xv.shape[0], rows), np.float64)
+    lib().orc_gemv_f64(wb, rows, cols, gs, xv, xv.shape[0], int(rule), y, a)
+    return y, a
+
+
+def gamma(cols: int) -> float:
+    return lib().orc_gamma(cols)
+
+
+def ffn(gate, gs_g, up, gs_u, down, gs_d, hidden, inter, x, limit: float = 0.0, threads: int = 1, path: int = 1):
+    xv = _f32(x).reshape(-1, hidden)
+    y = np.empty_like(xv)
+    rc = lib().orc_ffn_clamped(_u8(gate), gs_g, _u8(up), gs_u, _u8(down), gs_d, hidden, inter, limit, xv,
+                               xv.shape[0], y, threads, path)
+    assert rc == 0
+    return y
+
+
+def silu_mul(g, u) -> np.ndarray:
+    g, u = _f32(g), _f32(u)
+    L = lib()
+    return np.array([L.orc_silu_mul(float(a), float(b)) for a, b in zip(g.reshape(-1), u.reshape(-1))],
+                    np.float32).reshape(g.shape)
+
+
+def silu_mul_combo(h1, inter: int) -> np.ndarray:
+    h = _f32(h1).reshape(-1, 2 * inter)
+    out = np.empty((h.shape[0], inter), np.float32)
+    lib().orc_silu_mul_combo(h, h.shape[0], inter, out)
+    return out
+
+
+def acc_combo(x, rw, tokens: int, topk: int, hidden: int, y0=None) -> np.ndarray:
+    y = np.zeros((tokens, hidden), np.float32) if y0 is None else _f32(y0).copy()
+    lib().orc_acc_combo(_f32(x), _f32(rw), tokens, topk, hidden, y)
+    return y
+
+
+def router_topk(logits, topk: int):
+    l = _f32(logits)
+    t, e = l.shape
+    assert e & (e - 1) == 0, "the reference's tree reductions need a power-of-two expert count"
+    ids = np.empty((t, topk), np.int32)
+    w = np.empty((t, topk), np.float32)
+    lib().orc_router_topk(l, t, e, topk, ids, w)
+    return ids, w
+
+
+def argmax_ref(logits) -> int:
+    l = _f32(logits).reshape(-1)
+    return int(lib().orc_argmax_ref(l, l.size))
+
+
+def moe_layer(gate_up, gs_gu, down, gs_dn, experts, hidden, inter, x, logits, topk, threads: int = 1, path: int = 1):
+    xv = _f32(x).reshape(-1, hidden)
+    t = xv.shape[0]
+    ids = np.empty((t, topk), np.int32)
+    w = np.empty((t, topk), np.float32)
+    y = np.empty((t, hidden), np.float32)
+    rc = lib().orc_moe_layer(_u8(gate_up), gs_gu, _u8(down), gs_dn, experts, hidden, inter, xv, _f32(logits), t, topk,
+                             ids, w, y, threads, path)
+    assert rc == 0
+    return ids, w, y
+
+
+def f32_to_bf16_bits(v) -> np.ndarray:
+    x = _f32(v).view(np.uint32).astype(np.uint64)
+    return (((x + 0x7FFF + ((x >> 16) & 1)) >> 16) & 0xFFFF).astype(np.uint16)
+
+
+def bf16_bits_to_f32(b) -> np.ndarray:
+    return (np.asarray(b, np.uint16).astype(np.uint32) << 16).view(np.float32)
