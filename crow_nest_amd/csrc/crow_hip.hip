@@ -1,0 +1,364 @@
+// libcrow_hip.so: gfx950 code objects (built ahead of time from the headers below) and the C ABI
+// declared in include/crow_hip.h.  One translation unit, so the device globals are shared.
+#include <hip/hip_runtime.h>
+#include <cstdio>
+#include <cstdlib>
+#include <cstring>
+
+#include "../../include/crow_hip.h"
+#include "kernels.h"
+#include "misc_kernels.h"
+#include "gemm.h"
+
+namespace {
+
+struct FnEntry {
+    const char* name;
+    const void* stub;
+    int nargs;
+};
+
+#define CROW_FN(name, nargs) {#name, (const void*)&name, nargs}
+const FnEntry g_table[] = {
+    CROW_FN(gemv_nvfp4_w, 6),      CROW_FN(gemv_nvfp4_w_bf16, 6),   CROW_FN(gemv_nvfp4_w_argmax, 7),
+    CROW_FN(gemv_nvfp4_gu, 8),     CROW_FN(gemv_nvfp4_wm, 7),       CROW_FN(gemv_nvfp4_gum, 9),
+    CROW_FN(gemv_nvfp4_wm_bf16, 7), CROW_FN(gemv_nvfp4_gum_bf16, 9), CROW_FN(gemv_fp4, 6),
+    CROW_FN(gemv_fp4_b, 7),        CROW_FN(gemv_fp4_b1k, 7),        CROW_FN(gemv_fp4_bs, 8),
+    CROW_FN(gemv_fp4_ptrb, 8),     CROW_FN(moe_gate_up_silu, 8),    CROW_FN(moe_down_combine, 7),
+    CROW_FN(router_top10, 10),     CROW_FN(silu_mul_combo, 3),      CROW_FN(acc_combo, 3),
+    CROW_FN(argmax_k, 3),          CROW_FN(dequant_fp4_flat, 4),    CROW_FN(repack_nvfp4, 4),
+    CROW_FN(unpack_nvfp4, 4),      CROW_FN(dequant_nvfp4_tiled, 5),
+};
+const int g_table_n = (int)(sizeof(g_table) / sizeof(g_table[0]));
+
+struct State {
+    bool ready = false;
+    int device = -1;
+    int cus = 256;
+    hipStream_t stream = nullptr;
+    crow::Workspace ws{};
+    int* scalars = nullptr;  // two device words for the library's own launches (rows, k_dim)
+    char name[256] = {0};
+} g;
+
+const unsigned long long PARTIAL_FLOATS = 16ull << 20;  // 64 MiB of split-K partial sums
+const unsigned COUNTER_SLOTS = 1u << 16;
+const unsigned AM_SLOTS = 1u << 16;
+
+int hip_rc(hipError_t e) { return e == hipSuccess ? CROW_OK : (int)e; }
+
+long env_long(const char* key, long dflt) {
+    const char* v = getenv(key);
+    if (!v || !*v) return dflt;
+    char* end = nullptr;
+    long r = strtol(v, &end, 10);
+    return end && *end == 0 ? r : dflt;
+}
+
+const FnEntry* find(const char* name) {
+    if (!name) return nullptr;
+    for (int i = 0; i < g_table_n; i++)
+        if (strcmp(g_table[i].name, name) == 0) return &g_table[i];
+    return nullptr;
+}
+
+int launch_entry(const FnEntry* e, dim3 grid, dim3 block, const uint64_t* vals, uint32_t n, hipStream_t s) {
+    if (!g.ready) return CROW_ERR_NOT_INITIALIZED;
+    if (!e || !vals) return CROW_ERR_BAD_ARGUMENT;
+    if ((int)n != e->nargs) return CROW_ERR_ARG_COUNT;
+    if (grid.x == 0 || grid.y == 0 || grid.z == 0 || block.x == 0 || block.x > 1024) return CROW_ERR_BAD_ARGUMENT;
+    void* args[16];
+    for (uint32_t i = 0; i < n; i++) args[i] = (void*)&vals[i];
+    return hip_rc(hipLaunchKernel(e->stub, grid, block, args, 0, s));
+}
+
+}  // namespace
+
+extern "C" {
+
+int crow_hip_init(int device) {
+    if (g.ready) return g.device == device ? CROW_OK : CROW_ERR_BAD_ARGUMENT;
+    hipError_t e = hipSetDevice(device);
+    if (e != hipSuccess) return (int)e;
+    hipDeviceProp_t pr;
+    if ((e = hipGetDeviceProperties(&pr, device)) != hipSuccess) return (int)e;
+    snprintf(g.name, sizeof g.name, "%s (%s), %d CUs", pr.name, pr.gcnArchName, pr.multiProcessorCount);
+    if (strncmp(pr.gcnArchName, "gfx950", 6) != 0) {
+        fprintf(stderr, "crow_hip: this library holds gfx950 code objects only; device %d is %s\n", device, pr.gcnArchName);
+        return CROW_ERR_BAD_ARGUMENT;
+    }
+    g.cus = pr.multiProcessorCount;
+    crow::Workspace ws{};
+    ws.partial_floats = PARTIAL_FLOATS;
+    ws.counter_slots = COUNTER_SLOTS;
+    ws.am_slots = AM_SLOTS;
+    if ((e = hipMalloc((void**)&ws.partials, PARTIAL_FLOATS * sizeof(float))) != hipSuccess) return (int)e;
+    if ((e = hipMalloc((void**)&ws.counters, (COUNTER_SLOTS + 2) * sizeof(unsigned))) != hipSuccess) return (int)e;
+    if ((e = hipMalloc((void**)&ws.am_val, AM_SLOTS * sizeof(float))) != hipSuccess) return (int)e;
+    if ((e = hipMalloc((void**)&ws.am_idx, AM_SLOTS * sizeof(int))) != hipSuccess) return (int)e;
+    if ((e = hipMalloc((void**)&g.scalars, 16 * sizeof(int))) != hipSuccess) return (int)e;
+    if ((e = hipMemset(ws.counters, 0, (COUNTER_SLOTS + 2) * sizeof(unsigned))) != hipSuccess) return (int)e;
+    ws.status = ws.counters + COUNTER_SLOTS;
+    ws.am_counter = ws.counters + COUNTER_SLOTS + 1;
+    if ((e = hipMemcpyToSymbol(HIP_SYMBOL(crow::g_ws), &ws, sizeof ws)) != hipSuccess) return (int)e;
+    crow::Geo geo{0, 0, 0, 0};
+    if ((e = hipMemcpyToSymbol(HIP_SYMBOL(crow::g_geo), &geo, sizeof geo)) != hipSuccess) return (int)e;
+    if ((e = hipDeviceSynchronize()) != hipSuccess) return (int)e;
+    g.ws = ws;
+    g.device = device;
+    g.stream = nullptr;
+    g.ready = true;
+    return CROW_OK;
+}
+
+int crow_hip_shutdown(void) {
+    if (!g.ready) return CROW_OK;
+    (void)hipDeviceSynchronize();
+    (void)hipFree(g.ws.partials);
+    (void)hipFree(g.ws.counters);
+    (void)hipFree(g.ws.am_val);
+    (void)hipFree(g.ws.am_idx);
+    (void)hipFree(g.scalars);
+    g = State{};
+    return CROW_OK;
+}
+
+const char* crow_hip_error_string(int code) {
+    switch (code) {
+        case CROW_OK: return "ok";
+        case CROW_ERR_NOT_INITIALIZED: return "crow_hip_init has not been called";
+        case CROW_ERR_KERNEL_MISSING: return "kernel missing";
+        case CROW_ERR_BAD_ARGUMENT: return "bad argument";
+        case CROW_ERR_ARG_COUNT: return "wrong number of kernel arguments";
+        case CROW_ERR_WORKSPACE: return "launch does not fit the split-K workspace";
+        case CROW_ERR_SCALE_BYTE: return "scale byte 0xFF in an NVFP4 tensor (no encoder emits it; E4M3 cannot hold 480)";
+        case CROW_ERR_SHAPE: return "shape not supported by this kernel";
+        case CROW_ERR_GEO: return "geometry not set or out of range (crow_hip_set_geo)";
+        default: return code > 0 ? hipGetErrorString((hipError_t)code) : "unknown crow_hip error";
+    }
+}
+
+int crow_hip_device_name(char* out, size_t n) {
+    if (!g.ready) return CROW_ERR_NOT_INITIALIZED;
+    if (!out || n == 0) return CROW_ERR_BAD_ARGUMENT;
+    snprintf(out, n, "%s", g.name);
+    return CROW_OK;
+}
+
+// The module is the library itself: load/unload exist so that the reference's
+// compile -> Module -> get -> unload sequence keeps its shape.
+int crow_hip_module_load(crow_module_t* out) {
+    if (!g.ready) return CROW_ERR_NOT_INITIALIZED;
+    if (!out) return CROW_ERR_BAD_ARGUMENT;
+    *out = (crow_module_t)(void*)g_table;
+    return CROW_OK;
+}
+int crow_hip_module_unload(crow_module_t m) { return m == (crow_module_t)(void*)g_table ? CROW_OK : CROW_ERR_BAD_ARGUMENT; }
+int crow_hip_module_get(crow_module_t m, const char* name, crow_fn_t* out) {
+    if (m != (crow_module_t)(void*)g_table) return CROW_ERR_BAD_ARGUMENT;
+    return crow_hip_get_function(name, out);
+}
+int crow_hip_get_function(const char* name, crow_fn_t* out) {
+    if (!out || !name) return CROW_ERR_BAD_ARGUMENT;
+    const FnEntry* e = find(name);
+    if (!e) {
+        *out = nullptr;
+        return CROW_ERR_KERNEL_MISSING;
+    }
+    *out = (crow_fn_t)(void*)e;
+    return CROW_OK;
+}
+int crow_hip_function_count(void) { return g_table_n; }
+const char* crow_hip_function_name(int index) { return index >= 0 && index < g_table_n ? g_table[index].name : nullptr; }
+int crow_hip_function_arg_count(crow_fn_t f) {
+    const FnEntry* e = (const FnEntry*)(void*)f;
+    if (e < g_table || e >= g_table + g_table_n) return CROW_ERR_BAD_ARGUMENT;
+    return e->nargs;
+}
+
+int crow_hip_set_geo(int experts, int topk, int hidden, int inter) {
+    if (!g.ready) return CROW_ERR_NOT_INITIALIZED;
+    if (experts < 0 || topk < 0 || hidden < 0 || inter < 0) return CROW_ERR_BAD_ARGUMENT;
+    crow::Geo geo{experts, topk, hidden, inter};
+    hipError_t e = hipMemcpyToSymbolAsync(HIP_SYMBOL(crow::g_geo), &geo, sizeof geo, 0, hipMemcpyHostToDevice, g.stream);
+    if (e != hipSuccess) return (int)e;
+    return hip_rc(hipStreamSynchronize(g.stream));
+}
+
+int crow_hip_launch(crow_fn_t f, uint32_t gx, uint32_t gy, uint32_t gz, uint32_t bx, const uint64_t* vals, uint32_t n_vals,
+                    void* stream) {
+    const FnEntry* e = (const FnEntry*)(void*)f;
+    if (e < g_table || e >= g_table + g_table_n) return CROW_ERR_KERNEL_MISSING;
+    return launch_entry(e, dim3(gx, gy, gz), dim3(bx, 1, 1), vals, n_vals, stream ? (hipStream_t)stream : g.stream);
+}
+
+// Split of a [rows, k_dim] product over the chip.  Every wave owns one 64-row tile; a tile's
+// 256-column panels are dealt to W waves of a block (combined in LDS) and S blocks (combined
+// through the workspace).  Aim: about `target` waves in total, so that every CU holds enough
+// 16-byte loads in flight to cover HBM latency, and far more units than CUs so that the
+// hardware dispatcher balances them.  The result depends on (rows, k_dim) only.
+int crow_hip_launch_dims(const char* name, uint32_t rows, uint32_t k_dim, uint32_t z, crow_dims* out) {
+    if (!out || !name || rows == 0 || z == 0) return CROW_ERR_BAD_ARGUMENT;
+    const FnEntry* e = find(name);
+    if (!e) return CROW_ERR_KERNEL_MISSING;
+    const uint32_t rt = (rows + CROW_TILE_ROWS - 1) / CROW_TILE_ROWS;
+    const uint32_t panels = (k_dim + CROW_PANEL_COLS - 1) / CROW_PANEL_COLS;
+    if (strncmp(name, "gemv_", 5) == 0 || strncmp(name, "moe_gate_up", 11) == 0) {
+        if (k_dim == 0 || k_dim % CROW_BLOCK_VALUES != 0) return CROW_ERR_SHAPE;
+        const bool moe = strcmp(name, "gemv_fp4_ptrb") == 0 || strncmp(name, "moe_", 4) == 0;
+        const bool tokens = strcmp(name, "gemv_fp4_b") == 0 || strcmp(name, "gemv_fp4_b1k") == 0 || strcmp(name, "gemv_fp4_bs") == 0;
+        const bool two = strstr(name, "_gu") != nullptr || strncmp(name, "moe_gate_up", 11) == 0;
+        uint32_t tiles = two && !strncmp(name, "moe_", 4) ? rt : rt;  // rows = output rows for every kernel
+        const uint32_t gz = moe ? z : (tokens ? (z + 3) / 4 : 1);
+        long target = env_long("CROW_GEMV_TARGET_WAVES", 20L * g.cus);
+        long max_w = env_long("CROW_GEMV_MAX_W", 1);
+        long force_s = env_long("CROW_GEMV_S", 0), force_w = env_long("CROW_GEMV_W", 0);
+        // routed / batched launches multiply the tile count by gz, but the split must not depend on z
+        // for the dense kernels (bit-identity across M); routed kernels have their own fixed z per model.
+        long per_tile = (target + (long)tiles * (moe ? gz : 1) - 1) / ((long)tiles * (moe ? gz : 1));
+        if (per_tile < 1) per_tile = 1;
+        if (per_tile > (long)panels) per_tile = panels;
+        long w = per_tile < max_w ? per_tile : max_w;
+        long s = (per_tile + w - 1) / w;
+        if (force_w > 0) w = force_w;
+        if (force_s > 0) s = force_s;
+        if (w > 16) w = 16;
+        const int nrm = (two ? 2 : 1) * 4;
+        while (w > 1 && (w - 1) * nrm * 64 > CROW_RED_FLOATS) w--;
+        if (s * w > (long)panels) s = (panels + w - 1) / w;
+        if (s < 1) s = 1;
+        out->gx = (uint32_t)s;
+        out->gy = tiles;
+        out->gz = gz;
+        out->bx = (uint32_t)(64 * w);
+        const unsigned long long need = (unsigned long long)tiles * gz * s * nrm * 64;
+        if (s > 1 && (need > PARTIAL_FLOATS || (unsigned long long)tiles * gz > COUNTER_SLOTS)) return CROW_ERR_WORKSPACE;
+        if (strcmp(name, "gemv_nvfp4_w_argmax") == 0 && tiles > AM_SLOTS) return CROW_ERR_WORKSPACE;
+        return CROW_OK;
+    }
+    if (strcmp(name, "moe_down_combine") == 0) {
+        out->gx = 1; out->gy = rt; out->gz = z; out->bx = 64 * (g.ready ? 1 : 1);
+        return CROW_OK;
+    }
+    if (strcmp(name, "repack_nvfp4") == 0 || strcmp(name, "unpack_nvfp4") == 0 || strcmp(name, "dequant_nvfp4_tiled") == 0) {
+        *out = crow_dims{panels, rt, 1, 64};
+        return CROW_OK;
+    }
+    if (strcmp(name, "router_top10") == 0) { *out = crow_dims{z, 1, 1, 64}; return CROW_OK; }
+    if (strcmp(name, "argmax_k") == 0) { *out = crow_dims{1, 1, 1, 1024}; return CROW_OK; }
+    if (strcmp(name, "acc_combo") == 0) { *out = crow_dims{(rows + 255) / 256, z, 1, 256}; return CROW_OK; }  // rows = hidden
+    if (strcmp(name, "silu_mul_combo") == 0 || strcmp(name, "dequant_fp4_flat") == 0) {  // rows = element count
+        *out = crow_dims{(rows + 255) / 256, 1, 1, 256};
+        return CROW_OK;
+    }
+    return CROW_ERR_KERNEL_MISSING;
+}
+
+int crow_hip_status(void) {
+    if (!g.ready) return CROW_ERR_NOT_INITIALIZED;
+    hipError_t e = hipStreamSynchronize(g.stream);
+    if (e != hipSuccess) return (int)e;
+    unsigned st = 0;
+    if ((e = hipMemcpy(&st, g.ws.status, sizeof st, hipMemcpyDeviceToHost)) != hipSuccess) return (int)e;
+    if (st == 0) return CROW_OK;
+    (void)hipMemset(g.ws.status, 0, sizeof st);
+    // a launch that bailed out may have left arrival counters behind
+    (void)hipMemset(g.ws.counters, 0, (COUNTER_SLOTS + 2) * sizeof(unsigned));
+    if (st & CROW_STATUS_BAD_SCALE_BYTE) return CROW_ERR_SCALE_BYTE;
+    if (st & crow::STATUS_WORKSPACE_TOO_SMALL) return CROW_ERR_WORKSPACE;
+    if (st & crow::STATUS_BAD_GEO) return CROW_ERR_GEO;
+    return CROW_ERR_SHAPE;
+}
+
+int crow_hip_reset_workspace(void) {
+    if (!g.ready) return CROW_ERR_NOT_INITIALIZED;
+    hipError_t e = hipDeviceSynchronize();
+    if (e != hipSuccess) return (int)e;
+    return hip_rc(hipMemset(g.ws.counters, 0, (COUNTER_SLOTS + 2) * sizeof(unsigned)));
+}
+
+void crow_hip_set_stream(void* stream) { g.stream = (hipStream_t)stream; }
+void* crow_hip_cur_stream(void) { return (void*)g.stream; }
+int crow_hip_sync(void) { return g.ready ? hip_rc(hipStreamSynchronize(g.stream)) : CROW_ERR_NOT_INITIALIZED; }
+
+int crow_hip_alloc(size_t bytes, void** out) {
+    if (!g.ready) return CROW_ERR_NOT_INITIALIZED;
+    if (!out || bytes == 0) return CROW_ERR_BAD_ARGUMENT;
+    hipError_t e = hipMalloc(out, bytes);
+    if (e != hipSuccess) {
+        *out = nullptr;
+        return (int)e;
+    }
+    return hip_rc(hipMemset(*out, 0, bytes));
+}
+int crow_hip_free(void* p) { return p ? hip_rc(hipFree(p)) : CROW_OK; }
+int crow_hip_upload(void* dst, const void* src, size_t bytes) {
+    if (!g.ready) return CROW_ERR_NOT_INITIALIZED;
+    if (!dst || !src) return CROW_ERR_BAD_ARGUMENT;
+    hipError_t e = hipMemcpyAsync(dst, src, bytes, hipMemcpyHostToDevice, g.stream);
+    if (e != hipSuccess) return (int)e;
+    return g.stream == nullptr ? hip_rc(hipStreamSynchronize(nullptr)) : CROW_OK;
+}
+int crow_hip_download(void* dst, const void* src, size_t bytes) {
+    if (!g.ready) return CROW_ERR_NOT_INITIALIZED;
+    if (!dst || !src) return CROW_ERR_BAD_ARGUMENT;
+    hipError_t e = hipStreamSynchronize(g.stream);
+    if (e != hipSuccess) return (int)e;
+    return hip_rc(hipMemcpy(dst, src, bytes, hipMemcpyDeviceToHost));
+}
+
+int crow_hip_event_create(void** out) {
+    if (!out) return CROW_ERR_BAD_ARGUMENT;
+    hipEvent_t e;
+    hipError_t rc = hipEventCreate(&e);
+    *out = rc == hipSuccess ? (void*)e : nullptr;
+    return hip_rc(rc);
+}
+int crow_hip_event_record(void* ev) { return ev ? hip_rc(hipEventRecord((hipEvent_t)ev, g.stream)) : CROW_ERR_BAD_ARGUMENT; }
+int crow_hip_event_elapsed_ms(void* start, void* stop, float* ms) {
+    if (!start || !stop || !ms) return CROW_ERR_BAD_ARGUMENT;
+    hipError_t rc = hipEventSynchronize((hipEvent_t)stop);
+    if (rc != hipSuccess) return (int)rc;
+    return hip_rc(hipEventElapsedTime(ms, (hipEvent_t)start, (hipEvent_t)stop));
+}
+int crow_hip_event_destroy(void* ev) { return ev ? hip_rc(hipEventDestroy((hipEvent_t)ev)) : CROW_OK; }
+
+size_t crow_hip_container_bytes(uint32_t rows, uint32_t cols) { return crow_container_bytes(rows, cols); }
+size_t crow_hip_tiled_bytes(uint32_t rows, uint32_t cols) { return crow_tiled_bytes(rows, cols); }
+
+static int layout_launch(const char* name, const void* a, const void* b, const void* c, uint32_t rows, uint32_t cols) {
+    if (!g.ready) return CROW_ERR_NOT_INITIALIZED;
+    if (!a || !b || rows == 0 || cols == 0 || cols % CROW_BLOCK_VALUES != 0) return a && b ? CROW_ERR_SHAPE : CROW_ERR_BAD_ARGUMENT;
+    // the two scalars ride in a small ring of device words so that back-to-back calls do not race
+    static int slot = 0;
+    int* sc = g.scalars + 2 * (slot++ & 7);
+    int host[2] = {(int)rows, (int)cols};
+    hipError_t e = hipMemcpyAsync(sc, host, sizeof host, hipMemcpyHostToDevice, g.stream);
+    if (e != hipSuccess) return (int)e;
+    if ((e = hipStreamSynchronize(g.stream)) != hipSuccess) return (int)e;  // `host` is a stack buffer
+    crow_dims d;
+    int rc = crow_hip_launch_dims(name, rows, cols, 1, &d);
+    if (rc != CROW_OK) return rc;
+    uint64_t vals[5];
+    uint32_t n = 0;
+    vals[n++] = (uint64_t)a;
+    vals[n++] = (uint64_t)b;
+    if (c) vals[n++] = (uint64_t)c;
+    vals[n++] = (uint64_t)sc;
+    vals[n++] = (uint64_t)(sc + 1);
+    rc = launch_entry(find(name), dim3(d.gx, d.gy, d.gz), dim3(d.bx), vals, n, g.stream);
+    if (rc != CROW_OK) return rc;
+    return crow_hip_status();
+}
+
+int crow_hip_repack_nvfp4(const void* src_dev, uint32_t rows, uint32_t cols, void* dst_dev) {
+    return layout_launch("repack_nvfp4", src_dev, dst_dev, nullptr, rows, cols);
+}
+int crow_hip_unpack_nvfp4(const void* src_dev, uint32_t rows, uint32_t cols, void* dst_dev) {
+    return layout_launch("unpack_nvfp4", src_dev, dst_dev, nullptr, rows, cols);
+}
+int crow_hip_dequant_tiled(const void* w_dev, const float* gs_dev, uint32_t rows, uint32_t cols, float* out_dev) {
+    return layout_launch("dequant_nvfp4_tiled", w_dev, gs_dev, out_dev, rows, cols);
+}
+
+}  // extern "C"

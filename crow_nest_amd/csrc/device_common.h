@@ -1,0 +1,85 @@
+// Device-side state and helpers shared by every kernel of the library (one translation unit).
+#pragma once
+#include <hip/hip_runtime.h>
+#include "layout.h"
+
+namespace crow {
+
+typedef float f32x2 __attribute__((ext_vector_type(2)));
+typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+
+// Library-owned scratch for kernels that split one output tile over several workgroups:
+// per-slice partial sums and one arrival counter per output tile.  Set once by crow_hip_init.
+struct Workspace {
+    float* partials;
+    unsigned* counters;
+    unsigned long long partial_floats;  // capacity of `partials`
+    unsigned counter_slots;             // capacity of `counters`
+    unsigned* status;                   // device word: non-zero = a launch did not fit the workspace
+    float* am_val;                      // fused lm_head argmax: one (value, index) candidate per row tile
+    int* am_idx;
+    unsigned* am_counter;
+    unsigned am_slots;
+};
+__device__ Workspace g_ws;
+
+// Model geometry the reference bakes into its kernel text as CN_* defines
+// (engine/src/kernels.rs:5040-5125); here it is a device struct written by crow_hip_set_geo.
+struct Geo {
+    int experts, topk, hidden, inter;
+};
+__device__ Geo g_geo;
+
+enum StatusBits : unsigned { STATUS_WORKSPACE_TOO_SMALL = 1u, STATUS_BAD_SHAPE = 2u, STATUS_BAD_GEO = 4u };
+
+__device__ __forceinline__ int lane_id() { return (int)(threadIdx.x & 63u); }
+
+// E2M1 pair decode: byte `SEL` of `word` holds two codes (low nibble first); the gfx950
+// conversion instruction returns them as two exact f32 values (scale operand 1.0).
+template <int SEL>
+__device__ __forceinline__ f32x2 fp4x2_to_f32(unsigned word) {
+    return __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(word, 1.0f, SEL);
+}
+template <int SEL>
+__device__ __forceinline__ bf16x2 fp4x2_to_bf16(unsigned word) {
+    return __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(word, 1.0f, SEL);
+}
+// UE4M3 scale decode of byte `SEL` (canonical bytes 0x00..0x7E only: OCP E4M3, exact)
+template <int SEL>
+__device__ __forceinline__ float e4m3_to_f32(unsigned word) {
+    return __builtin_amdgcn_cvt_f32_fp8((int)word, SEL);
+}
+
+__device__ __forceinline__ unsigned u4_get(const uint4& v, int i) { return i == 0 ? v.x : (i == 1 ? v.y : (i == 2 ? v.z : v.w)); }
+
+// silu(g) * u exactly as the reference kernels write it (kernels_p2.rs:386-387)
+__device__ __forceinline__ float silu_mul(float g, float u) { return (g / (1.0f + expf(-g))) * u; }
+
+// Greedy argmax order.  The reference (engine/src/kernels.rs:4238-4260) scans with 1024 strided
+// threads (strict >, so a thread keeps its smallest index) and then halves a 1024-slot tree with
+// strides 512 .. 1 in which slot t takes slot t + stride only when strictly greater.  Among equal
+// maxima that tournament prefers bit 0 of t clear (the last round), then bit 1, ... : the winner is
+// the position with the smallest BIT-REVERSED (i mod 1024), then the smallest i.  That is a total
+// order, so any reduction shape gives the same index.  Start value -3.0e38 with index 0, as the
+// reference.
+struct Best {
+    float v;
+    int i;
+};
+__device__ __forceinline__ bool better(float v, int i, float bv, int bi) {
+    const unsigned ki = __brev((unsigned)i & 1023u), kb = __brev((unsigned)bi & 1023u);
+    return v > bv || (v == bv && (ki < kb || (ki == kb && i < bi)));
+}
+__device__ __forceinline__ Best wave_best(Best b) {
+    for (int o = 32; o > 0; o >>= 1) {
+        const float ov = __shfl_xor(b.v, o);
+        const int oi = __shfl_xor(b.i, o);
+        if (better(ov, oi, b.v, b.i)) {
+            b.v = ov;
+            b.i = oi;
+        }
+    }
+    return b;
+}
+
+}  // namespace crow

@@ -1,0 +1,372 @@
+// NVFP4 GEMV family for gfx950: y[m][row] = gs * sum_k W[row][k] * x[m][k], M <= 4 activation rows.
+//
+// Mapping.  One wavefront owns one 64-row tile: lane l computes row l.  All lanes of a wave walk
+// the same columns, so the activation is wave-uniform and is read through scalar loads into
+// SGPRs; the FMA takes it as its scalar operand and nothing is ever shuffled between lanes.
+// Weights are read exactly once, as 16-byte-per-lane loads that cover 1024 contiguous bytes per
+// instruction (layout.h).  E2M1 pairs decode with v_cvt_scalef32_pk_f32_fp4 (exact), UE4M3 scales
+// with v_cvt_f32_fp8 (exact on canonical bytes).
+//
+// FP32 accumulation order (per output row and activation row), documented because it differs
+// from the reference CPU path's 8-lane order (cpu_nvfp4.rs:22-31) and from its GPU kernel of
+// record (kernels_p2.rs:304-347); all three are within the same gamma bound of the exact sum:
+//   for each 16-value sub-block, in column order:
+//       part = fma(w15, x15, ... fma(w1, x1, w0 * x0))        (w exact, 16 fused steps)
+//       acc  = fma(part, ue4m3(scale), acc)
+//   a row split over several waves / workgroups: the per-slice `acc` values are added in slice
+//   order (slice 0 first), each slice covering whole 256-column panels p = slice, slice + S, ...
+//   y = acc * gs                                               (gs last, as kernels_p2.rs:367)
+// The order depends only on (K, slices), never on M: row m of an M-row launch is bit-identical to
+// a one-row launch with the same slicing (the verify contract of kernels_p2.rs:391-396).
+//
+// Launch geometry: grid (S, row_tiles, Z), block 64 * W.  blockIdx.x = column slice, blockIdx.y =
+// row tile, blockIdx.z = token group / expert combo.  The W waves of a block and the S blocks of
+// a row tile split the panels round-robin: unit u = slice * W + wave takes panels u, u + S W, ...
+// Waves combine through LDS, blocks through the library workspace: every block stores its
+// partial sums, bumps the tile's arrival counter, and the block that arrives last adds all
+// partials in slice order and writes y (deterministic whatever the arrival order).
+#pragma once
+#include "device_common.h"
+
+namespace crow {
+
+enum Epilogue { EPI_SCALE = 0, EPI_SILU_GU = 1 };
+
+struct GemvArgs {
+    const unsigned char* w[2];  // tiled tensors (w[1] only for EPI_SILU_GU: the `up` matrix)
+    const float* gs[2];
+    const void* x;       // [M][x_stride] f32 (or bf16 when XBF16)
+    size_t x_stride;     // elements between activation rows
+    float* y;            // [M][y_stride]
+    size_t y_stride;
+    int k_dim, rows, m;  // m <= MMAX of the instantiation
+    int* argmax_out;     // not null: also write the greedy argmax of y row 0 (fused lm_head head)
+};
+
+// LDS floats for the wave -> wave 0 hand-over: (waves - 1) * NR * M * 64 must fit
+#define CROW_RED_FLOATS 4096
+
+// 16 consecutive activation values of row m, wave-uniform (scalar loads)
+template <bool XBF16>
+struct XChunk;
+template <>
+struct XChunk<false> {
+    float v[16];
+    __device__ __forceinline__ void load(const void* x, size_t off) {
+        const float* p = (const float*)x + off;
+#pragma unroll
+        for (int j = 0; j < 16; j++) v[j] = p[j];
+    }
+};
+template <>
+struct XChunk<true> {
+    unsigned v[8];  // bf16 pairs
+    __device__ __forceinline__ void load(const void* x, size_t off) {
+        const unsigned* p = (const unsigned*)((const unsigned short*)x + off);
+#pragma unroll
+        for (int j = 0; j < 8; j++) v[j] = p[j];
+    }
+};
+
+// one 16-value sub-block: two code words (w0: values 0..7, w1: values 8..15).  The chain is split
+// into its first link and the rest so that a caller can place other work between them.
+template <bool XBF16>
+__device__ __forceinline__ float dot_head(unsigned w0, const XChunk<XBF16>& x);
+template <bool XBF16>
+__device__ __forceinline__ float dot_tail(float part, unsigned w0, unsigned w1, const XChunk<XBF16>& x);
+
+template <>
+__device__ __forceinline__ float dot_head<false>(unsigned w0, const XChunk<false>& x) {
+    return fp4x2_to_f32<0>(w0).x * x.v[0];
+}
+template <>
+__device__ __forceinline__ float dot_tail<false>(float part, unsigned w0, unsigned w1, const XChunk<false>& x) {
+    f32x2 a = fp4x2_to_f32<0>(w0), b = fp4x2_to_f32<1>(w0), c = fp4x2_to_f32<2>(w0), d = fp4x2_to_f32<3>(w0);
+    part = __builtin_fmaf(a.y, x.v[1], part);
+    part = __builtin_fmaf(b.x, x.v[2], part);
+    part = __builtin_fmaf(b.y, x.v[3], part);
+    part = __builtin_fmaf(c.x, x.v[4], part);
+    part = __builtin_fmaf(c.y, x.v[5], part);
+    part = __builtin_fmaf(d.x, x.v[6], part);
+    part = __builtin_fmaf(d.y, x.v[7], part);
+    a = fp4x2_to_f32<0>(w1), b = fp4x2_to_f32<1>(w1), c = fp4x2_to_f32<2>(w1), d = fp4x2_to_f32<3>(w1);
+    part = __builtin_fmaf(a.x, x.v[8], part);
+    part = __builtin_fmaf(a.y, x.v[9], part);
+    part = __builtin_fmaf(b.x, x.v[10], part);
+    part = __builtin_fmaf(b.y, x.v[11], part);
+    part = __builtin_fmaf(c.x, x.v[12], part);
+    part = __builtin_fmaf(c.y, x.v[13], part);
+    part = __builtin_fmaf(d.x, x.v[14], part);
+    part = __builtin_fmaf(d.y, x.v[15], part);
+    return part;
+}
+
+// bf16 activations: both factors are bf16, every product is exact in f32 and the dot
+// instruction adds two of them per step (v_dot2c_f32_bf16)
+template <>
+__device__ __forceinline__ float dot_head<true>(unsigned w0, const XChunk<true>& x) {
+    return __builtin_amdgcn_fdot2_f32_bf16(fp4x2_to_bf16<0>(w0), __builtin_bit_cast(bf16x2, x.v[0]), 0.0f, false);
+}
+template <>
+__device__ __forceinline__ float dot_tail<true>(float part, unsigned w0, unsigned w1, const XChunk<true>& x) {
+    part = __builtin_amdgcn_fdot2_f32_bf16(fp4x2_to_bf16<1>(w0), __builtin_bit_cast(bf16x2, x.v[1]), part, false);
+    part = __builtin_amdgcn_fdot2_f32_bf16(fp4x2_to_bf16<2>(w0), __builtin_bit_cast(bf16x2, x.v[2]), part, false);
+    part = __builtin_amdgcn_fdot2_f32_bf16(fp4x2_to_bf16<3>(w0), __builtin_bit_cast(bf16x2, x.v[3]), part, false);
+    part = __builtin_amdgcn_fdot2_f32_bf16(fp4x2_to_bf16<0>(w1), __builtin_bit_cast(bf16x2, x.v[4]), part, false);
+    part = __builtin_amdgcn_fdot2_f32_bf16(fp4x2_to_bf16<1>(w1), __builtin_bit_cast(bf16x2, x.v[5]), part, false);
+    part = __builtin_amdgcn_fdot2_f32_bf16(fp4x2_to_bf16<2>(w1), __builtin_bit_cast(bf16x2, x.v[6]), part, false);
+    part = __builtin_amdgcn_fdot2_f32_bf16(fp4x2_to_bf16<3>(w1), __builtin_bit_cast(bf16x2, x.v[7]), part, false);
+    return part;
+}
+template <bool XBF16>
+__device__ __forceinline__ float subblock_dot(unsigned w0, unsigned w1, const XChunk<XBF16>& x) {
+    return dot_tail<XBF16>(dot_head<XBF16>(w0, x), w0, w1, x);
+}
+
+template <int I>
+__device__ __forceinline__ float scale_of(const uint4& sc) {  // sub-block I (0..15) of the panel
+    return e4m3_to_f32<I & 3>(u4_get(sc, I >> 2));
+}
+
+// One 32-column step S of a panel for NR tensors and M activation rows.
+template <int NR, int M, bool XBF16, int S>
+__device__ __forceinline__ void step(const uint4 (&sc)[NR], const uint4 (&cd)[NR], const void* x, size_t x_off,
+                                     size_t x_stride, int m_rows, float (&acc)[NR][M]) {
+#pragma unroll
+    for (int half = 0; half < 2; half++) {
+        XChunk<XBF16> xc[M];
+#pragma unroll
+        for (int m = 0; m < M; m++)
+            if (m < m_rows) xc[m].load(x, (size_t)m * x_stride + x_off + half * 16);
+#pragma unroll
+        for (int r = 0; r < NR; r++) {
+            const unsigned w0 = half ? cd[r].z : cd[r].x, w1 = half ? cd[r].w : cd[r].y;
+            const float sf = half ? scale_of<2 * S + 1>(sc[r]) : scale_of<2 * S>(sc[r]);
+#pragma unroll
+            for (int m = 0; m < M; m++)
+                if (m < m_rows) acc[r][m] = __builtin_fmaf(subblock_dot<XBF16>(w0, w1, xc[m]), sf, acc[r][m]);
+        }
+    }
+}
+
+template <int NR, int M, bool XBF16, int S>
+struct Steps {
+    __device__ __forceinline__ static void run(const uint4 (&sc)[NR], const uint4 (&cd)[NR][CROW_STEPS], const void* x,
+                                               size_t x_off, size_t x_stride, int m_rows, int nsteps,
+                                               float (&acc)[NR][M]) {
+        if (S < nsteps) {
+            uint4 c[NR];
+#pragma unroll
+            for (int r = 0; r < NR; r++) c[r] = cd[r][S];
+            step<NR, M, XBF16, S>(sc, c, x, x_off + S * CROW_STEP_COLS, x_stride, m_rows, acc);
+        }
+        Steps<NR, M, XBF16, S + 1>::run(sc, cd, x, x_off, x_stride, m_rows, nsteps, acc);
+    }
+    // a whole panel: no per-step test (see panel_full below)
+};
+template <int NR, int M, bool XBF16>
+struct Steps<NR, M, XBF16, CROW_STEPS> {
+    __device__ __forceinline__ static void run(const uint4 (&)[NR], const uint4 (&)[NR][CROW_STEPS], const void*, size_t,
+                                               size_t, int, int, float (&)[NR][M]) {}
+};
+
+// A whole 256-column panel with the activation chunks software-pipelined: the scalar loads of
+// sub-block H + 1 are issued before the arithmetic of sub-block H, so their latency is covered by
+// 16 * M fused multiply-adds instead of being waited for.
+template <int NR, int M, bool XBF16, int H>
+struct PanelFull {
+    __device__ __forceinline__ static void run(const uint4 (&sc)[NR], const uint4 (&cd)[NR][CROW_STEPS], const void* x, size_t x_off,
+                                               size_t x_stride, int m_rows, XChunk<XBF16> (&cur)[M], float (&acc)[NR][M]) {
+        // first link of every chain: this is where the wave waits for `cur`; only then are the
+        // next sub-block's scalar loads issued (scalar loads return out of order, so a wait covers
+        // everything outstanding - issued any earlier they would be waited for here as well)
+        float part[NR][M];
+#pragma unroll
+        for (int r = 0; r < NR; r++) {
+            const uint4& c = cd[r][H >> 1];
+#pragma unroll
+            for (int m = 0; m < M; m++)
+                if (m < m_rows) part[r][m] = dot_head<XBF16>((H & 1) ? c.z : c.x, cur[m]);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+        XChunk<XBF16> nxt[M];
+        if (H + 1 < 2 * CROW_STEPS) {
+#pragma unroll
+            for (int m = 0; m < M; m++)
+                if (m < m_rows) nxt[m].load(x, (size_t)m * x_stride + x_off + (H + 1) * 16);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int r = 0; r < NR; r++) {
+            const uint4& c = cd[r][H >> 1];
+            const unsigned w0 = (H & 1) ? c.z : c.x, w1 = (H & 1) ? c.w : c.y;
+            const float sf = scale_of<H>(sc[r]);
+#pragma unroll
+            for (int m = 0; m < M; m++)
+                if (m < m_rows) acc[r][m] = __builtin_fmaf(dot_tail<XBF16>(part[r][m], w0, w1, cur[m]), sf, acc[r][m]);
+        }
+        PanelFull<NR, M, XBF16, H + 1>::run(sc, cd, x, x_off, x_stride, m_rows, nxt, acc);
+    }
+};
+template <int NR, int M, bool XBF16>
+struct PanelFull<NR, M, XBF16, 2 * CROW_STEPS> {
+    __device__ __forceinline__ static void run(const uint4 (&)[NR], const uint4 (&)[NR][CROW_STEPS], const void*, size_t, size_t, int,
+                                               XChunk<XBF16> (&)[M], float (&)[NR][M]) {}
+};
+
+// acc[r][m] = sum over panels p = p0, p0 + stride, ... of the 64-row tile `rt` of tensor r against
+// activation row m: the per-lane (= per-row) partial dot product of one wave.
+template <int NR, int M, bool XBF16>
+__device__ __forceinline__ void tile_accumulate(const unsigned char* const (&w)[2], int rt, int panels, int p0, int stride,
+                                                int k_dim, const void* x, size_t x_stride, int m_rows, float (&acc)[NR][M]) {
+    const int lane = lane_id();
+#pragma unroll
+    for (int r = 0; r < NR; r++)
+#pragma unroll
+        for (int m = 0; m < M; m++) acc[r][m] = 0.0f;
+    for (int p = p0; p < panels; p += stride) {
+        uint4 sc[NR], cd[NR][CROW_STEPS];
+#pragma unroll
+        for (int r = 0; r < NR; r++) {
+            const uint4* t = (const uint4*)(w[r] + ((size_t)rt * panels + p) * CROW_TILE_BYTES) + lane;
+            sc[r] = t[0];
+#pragma unroll
+            for (int s = 0; s < CROW_STEPS; s++) cd[r][s] = t[64 * (s + 1)];
+        }
+        const int left = (k_dim - p * CROW_PANEL_COLS) / CROW_STEP_COLS;
+        if (left >= CROW_STEPS) {
+            XChunk<XBF16> first[M];
+#pragma unroll
+            for (int m = 0; m < M; m++)
+                if (m < m_rows) first[m].load(x, (size_t)m * x_stride + (size_t)p * CROW_PANEL_COLS);
+            PanelFull<NR, M, XBF16, 0>::run(sc, cd, x, (size_t)p * CROW_PANEL_COLS, x_stride, m_rows, first, acc);
+        } else Steps<NR, M, XBF16, 0>::run(sc, cd, x, (size_t)p * CROW_PANEL_COLS, x_stride, m_rows, left, acc);
+    }
+}
+
+// The body every GEMV entry point runs.  `z` selects nothing here: the caller has already
+// offset the pointers in `a` for its token group / combo; `tile_id` indexes the workspace.
+template <int NR, int M, bool XBF16, int EPI>
+__device__ __forceinline__ void gemv_body(const GemvArgs& a, unsigned tile_id, float* red) {
+    const int lane = lane_id();
+    const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6)), waves = (int)(blockDim.x >> 6);  // wave-uniform on purpose
+    const int slice = (int)blockIdx.x, slices = (int)gridDim.x;
+    const int rt = (int)blockIdx.y;
+    const int panels = (a.k_dim + CROW_PANEL_COLS - 1) / CROW_PANEL_COLS;
+    const int m_rows = a.m < M ? a.m : M;
+
+    float acc[NR][M];
+    tile_accumulate<NR, M, XBF16>(a.w, rt, panels, slice * waves + wave, slices * waves, a.k_dim, a.x, a.x_stride, m_rows, acc);
+
+    // waves of the block -> wave 0, in wave order
+    if (waves > 1) {
+        if ((waves - 1) * NR * M * 64 > CROW_RED_FLOATS) {  // uniform: the launch does not fit this kernel
+            if (threadIdx.x == 0) atomicOr(g_ws.status, STATUS_BAD_SHAPE);
+            return;
+        }
+        if (wave > 0) {
+#pragma unroll
+            for (int r = 0; r < NR; r++)
+#pragma unroll
+                for (int m = 0; m < M; m++) red[((wave - 1) * NR * M + r * M + m) * 64 + lane] = acc[r][m];
+        }
+        __syncthreads();
+        if (wave > 0) return;
+        for (int w = 1; w < waves; w++) {
+#pragma unroll
+            for (int r = 0; r < NR; r++)
+#pragma unroll
+                for (int m = 0; m < M; m++) acc[r][m] += red[((w - 1) * NR * M + r * M + m) * 64 + lane];
+        }
+    }
+
+    // blocks of the row tile -> the last one to arrive, in slice order
+    if (slices > 1) {
+        const Workspace ws = g_ws;
+        const size_t need = ((size_t)tile_id + 1) * slices * (NR * M) * 64;
+        if (need > ws.partial_floats || tile_id >= ws.counter_slots) {
+            if (lane == 0) atomicOr(ws.status, STATUS_WORKSPACE_TOO_SMALL);
+            return;
+        }
+        float* base = ws.partials + (size_t)tile_id * slices * (NR * M) * 64;
+        float* mine = base + (size_t)slice * (NR * M) * 64;
+#pragma unroll
+        for (int r = 0; r < NR; r++)
+#pragma unroll
+            for (int m = 0; m < M; m++)
+                if (m < m_rows) __hip_atomic_store(mine + (r * M + m) * 64 + lane, acc[r][m], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "agent");
+        unsigned arrived = 0;
+        if (lane == 0) arrived = __hip_atomic_fetch_add(ws.counters + tile_id, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        arrived = __builtin_amdgcn_readfirstlane(arrived);
+        if (arrived != (unsigned)slices - 1) return;
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
+#pragma unroll
+        for (int r = 0; r < NR; r++)
+#pragma unroll
+            for (int m = 0; m < M; m++) acc[r][m] = 0.0f;
+        for (int s = 0; s < slices; s++) {
+            const float* q = base + (size_t)s * (NR * M) * 64;
+#pragma unroll
+            for (int r = 0; r < NR; r++)
+#pragma unroll
+                for (int m = 0; m < M; m++)
+                    if (m < m_rows) acc[r][m] += __hip_atomic_load(q + (r * M + m) * 64 + lane, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
+        if (lane == 0) __hip_atomic_store(ws.counters + tile_id, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+
+    const int row = rt * CROW_TILE_ROWS + lane;
+    if (EPI == EPI_SCALE && a.argmax_out != nullptr) {
+        // fused head: logits out, then one (value, index) candidate per row tile; the tile that
+        // arrives last scans all candidates.  The order is total, so arrival order cannot matter.
+        const float v = acc[0][0] * a.gs[0][0];
+        if (row < a.rows) a.y[row] = v;
+        Best b = wave_best(Best{row < a.rows ? v : -3.0e38f, row < a.rows ? row : 0});
+        const Workspace ws = g_ws;
+        const unsigned tiles = gridDim.y;
+        if (tiles > ws.am_slots) {
+            if (lane == 0) atomicOr(ws.status, STATUS_WORKSPACE_TOO_SMALL);
+            return;
+        }
+        unsigned arrived = 0;
+        if (lane == 0) {
+            __hip_atomic_store(ws.am_val + rt, b.v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            __hip_atomic_store(ws.am_idx + rt, b.i, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "agent");
+            arrived = __hip_atomic_fetch_add(ws.am_counter, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
+        arrived = __builtin_amdgcn_readfirstlane(arrived);
+        if (arrived != tiles - 1) return;
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
+        Best g{-3.0e38f, 0};
+        for (unsigned t = lane; t < tiles; t += 64) {
+            const float tv = __hip_atomic_load(ws.am_val + t, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            const int ti = __hip_atomic_load(ws.am_idx + t, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            if (better(tv, ti, g.v, g.i)) {
+                g.v = tv;
+                g.i = ti;
+            }
+        }
+        g = wave_best(g);
+        if (lane == 0) {
+            a.argmax_out[0] = g.i;
+            __hip_atomic_store(ws.am_counter, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
+        return;
+    }
+    if (row >= a.rows) return;
+    if (EPI == EPI_SCALE) {
+        const float gs = a.gs[0][0];
+#pragma unroll
+        for (int m = 0; m < M; m++)
+            if (m < m_rows) a.y[(size_t)m * a.y_stride + row] = acc[0][m] * gs;
+    } else {
+        const float gg = a.gs[0][0], gu = a.gs[NR - 1][0];
+#pragma unroll
+        for (int m = 0; m < M; m++)
+            if (m < m_rows) a.y[(size_t)m * a.y_stride + row] = silu_mul(acc[0][m] * gg, acc[NR - 1][m] * gu);
+    }
+}
+
+}  // namespace crow

@@ -1,0 +1,269 @@
+// Load-time repack, dequant, and the small kernels around the GEMVs (router, SwiGLU, combine, argmax).
+#pragma once
+#include "device_common.h"
+
+using namespace crow;
+
+#define CROW_STATUS_BAD_SCALE_BYTE 8u
+
+// ------------------------------------------------------------------ container <-> tiled
+// One 64-thread block per tile (blockIdx.x = panel, blockIdx.y = row tile); lane l moves row l.
+// Load-time work: the strided 36-byte reads are not coalesced and need not be.
+extern "C" __global__ void __launch_bounds__(64) repack_nvfp4(const unsigned char* __restrict__ src, unsigned char* __restrict__ dst,
+                                                              const int* __restrict__ rows_p, const int* __restrict__ k_dim_p) {
+    const int rows = *rows_p, k = *k_dim_p;
+    const int panels = (k + CROW_PANEL_COLS - 1) / CROW_PANEL_COLS, bpr = k / CROW_BLOCK_VALUES;
+    const int p = (int)blockIdx.x, rt = (int)blockIdx.y, lane = lane_id();
+    const int row = rt * CROW_TILE_ROWS + lane;
+    unsigned sc[4] = {0, 0, 0, 0};
+    unsigned cd[CROW_STEPS][4];
+#pragma unroll
+    for (int s = 0; s < CROW_STEPS; s++) cd[s][0] = cd[s][1] = cd[s][2] = cd[s][3] = 0;
+    bool bad = false;
+    if (row < rows) {
+#pragma unroll
+        for (int b = 0; b < 4; b++) {
+            const int blk = p * 4 + b;
+            if (blk < bpr) {
+                const unsigned* q = (const unsigned*)(src + ((size_t)row * bpr + blk) * CROW_BLOCK_BYTES);
+                unsigned s4 = q[0], canon = 0;
+#pragma unroll
+                for (int i = 0; i < 4; i++) {
+                    unsigned v = (s4 >> (8 * i)) & 0xFFu;
+                    if (v == 0xFFu) bad = true;
+                    v &= 0x7Fu;
+                    if (v == 0x7Fu) v = 0x7Eu;
+                    canon |= v << (8 * i);
+                }
+                sc[b] = canon;
+#pragma unroll
+                for (int j = 0; j < 4; j++) {
+                    cd[2 * b][j] = q[1 + j];
+                    cd[2 * b + 1][j] = q[5 + j];
+                }
+            }
+        }
+    }
+    uint4* t = (uint4*)(dst + ((size_t)rt * panels + p) * CROW_TILE_BYTES) + lane;
+    t[0] = make_uint4(sc[0], sc[1], sc[2], sc[3]);
+#pragma unroll
+    for (int s = 0; s < CROW_STEPS; s++) t[64 * (s + 1)] = make_uint4(cd[s][0], cd[s][1], cd[s][2], cd[s][3]);
+    if (bad) atomicOr(g_ws.status, CROW_STATUS_BAD_SCALE_BYTE);
+}
+
+// The inverse: tiled -> container bytes (scale bytes come back canonical: 0x7F has become 0x7E and
+// bit 7 is cleared; everything else is byte-identical to what was repacked).
+extern "C" __global__ void __launch_bounds__(64) unpack_nvfp4(const unsigned char* __restrict__ src, unsigned char* __restrict__ dst,
+                                                              const int* __restrict__ rows_p, const int* __restrict__ k_dim_p) {
+    const int rows = *rows_p, k = *k_dim_p;
+    const int panels = (k + CROW_PANEL_COLS - 1) / CROW_PANEL_COLS, bpr = k / CROW_BLOCK_VALUES;
+    const int p = (int)blockIdx.x, rt = (int)blockIdx.y, lane = lane_id();
+    const int row = rt * CROW_TILE_ROWS + lane;
+    if (row >= rows) return;
+    const uint4* t = (const uint4*)(src + ((size_t)rt * panels + p) * CROW_TILE_BYTES) + lane;
+    const uint4 sc = t[0];
+#pragma unroll
+    for (int b = 0; b < 4; b++) {
+        const int blk = p * 4 + b;
+        if (blk < bpr) {
+            unsigned* q = (unsigned*)(dst + ((size_t)row * bpr + blk) * CROW_BLOCK_BYTES);
+            q[0] = u4_get(sc, b);
+            const uint4 c0 = t[64 * (2 * b + 1)], c1 = t[64 * (2 * b + 2)];
+            q[1] = c0.x; q[2] = c0.y; q[3] = c0.z; q[4] = c0.w;
+            q[5] = c1.x; q[6] = c1.y; q[7] = c1.z; q[8] = c1.w;
+        }
+    }
+}
+
+// Dequantise a tiled tensor to f32 [rows][k_dim]: w = e2m1(code) * f32(ue4m3(scale) * gs), the two
+// roundings of the reference decode in that order (engine/src/cnq.rs:1298-1308 with the scale rule of
+// cpu_nvfp4.rs:98-105 already applied by the repacker).  Same grid as repack_nvfp4.
+extern "C" __global__ void __launch_bounds__(64) dequant_nvfp4_tiled(const unsigned char* __restrict__ w, const float* __restrict__ gs_ptr,
+                                                                     float* __restrict__ out, const int* __restrict__ rows_p,
+                                                                     const int* __restrict__ k_dim_p) {
+    const int rows = *rows_p, k = *k_dim_p;
+    const int panels = (k + CROW_PANEL_COLS - 1) / CROW_PANEL_COLS;
+    const int p = (int)blockIdx.x, rt = (int)blockIdx.y, lane = lane_id();
+    const int row = rt * CROW_TILE_ROWS + lane;
+    if (row >= rows) return;
+    const float gs = gs_ptr[0];
+    const uint4* t = (const uint4*)(w + ((size_t)rt * panels + p) * CROW_TILE_BYTES) + lane;
+    const uint4 sc = t[0];
+    for (int s = 0; s < CROW_STEPS; s++) {
+        const int col0 = p * CROW_PANEL_COLS + s * CROW_STEP_COLS;
+        if (col0 >= k) break;
+        const uint4 c = t[64 * (s + 1)];
+        float* o = out + (size_t)row * k + col0;
+        for (int h = 0; h < 2; h++) {
+            const int sb = 2 * s + h;
+            const unsigned byte = (u4_get(sc, sb >> 2) >> (8 * (sb & 3))) & 0xFFu;
+            const float sf = __builtin_amdgcn_cvt_f32_fp8((int)byte, 0) * gs;
+            for (int d = 0; d < 2; d++) {
+                const unsigned wd = u4_get(c, 2 * h + d);
+                for (int j = 0; j < 8; j++) {
+                    const unsigned nib = (wd >> (4 * j)) & 0xFu;
+                    const f32x2 v = __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(nib, 1.0f, 0);
+                    o[h * 16 + d * 8 + j] = v.x * sf;
+                }
+            }
+        }
+    }
+}
+
+// reference: dequant_fp4_flat, engine/src/kernels.rs:1460-1471 - CONTAINER layout, raw decode
+// (no scale rule: 0x7F reads 480, bit 7 ignored), one thread per value.
+extern "C" __global__ void dequant_fp4_flat(const unsigned char* __restrict__ w, const float* __restrict__ gs_ptr,
+                                            float* __restrict__ out, const int* __restrict__ n_p) {
+    const int i = (int)(blockIdx.x * blockDim.x + threadIdx.x);
+    if (i >= *n_p) return;
+    const int b = i >> 6, idx = i & 63;
+    const unsigned char* blk = w + (size_t)b * CROW_BLOCK_BYTES;
+    // (byte & 0x7F) << 20 is the f32 whose value is ue4m3(byte) * 2^-120, subnormal ladder included
+    const float u = __uint_as_float(((unsigned)blk[idx >> 4] & 0x7Fu) << 20) * 0x1p120f;
+    const float s = u * gs_ptr[0];
+    const unsigned byte = blk[4 + (idx >> 1)];
+    const unsigned nib = (idx & 1) ? (byte >> 4) : (byte & 0xFu);
+    const f32x2 v = __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(nib, 1.0f, 0);
+    out[i] = v.x * s;
+}
+
+// ------------------------------------------------------------------ router
+// reference: router_top10, engine/src/kernels.rs:3109-3184.  grid (T), block 64: one wavefront per
+// token, expert e lives in lane e % 64, slot e / 64.  The softmax denominator is added in the
+// reference's halving-tree order (slots first, then lanes), so weights match an E-thread tree.
+// Ties go to the lowest expert id.  E = g_geo.experts (power of two, 64..1024), K = g_geo.topk <= 16.
+// bitmap / cold_mask / counters / sel_counts / table / *_ptrs may be null (skipped).
+extern "C" __global__ void __launch_bounds__(64) router_top10(const float* __restrict__ logits, const unsigned int* __restrict__ bitmap,
+                                                              int* __restrict__ ids, float* __restrict__ wts,
+                                                              unsigned long long* __restrict__ gu_ptrs, unsigned long long* __restrict__ dn_ptrs,
+                                                              const unsigned long long* __restrict__ table, unsigned int* __restrict__ cold_mask,
+                                                              unsigned long long* __restrict__ counters, unsigned long long* __restrict__ sel_counts) {
+    const int E = g_geo.experts, K = g_geo.topk;
+    if (E < 64 || E > 1024 || (E & (E - 1)) != 0 || K < 1 || K > 16 || K > E) {
+        if (threadIdx.x == 0) atomicOr(g_ws.status, STATUS_BAD_GEO);
+        return;
+    }
+    const int t = (int)blockIdx.x, lane = lane_id(), slots = E >> 6;
+    float l[16], p[16];
+    float mx = -INFINITY;
+    for (int j = 0; j < 16; j++) {
+        l[j] = j < slots ? logits[(size_t)t * E + j * 64 + lane] : -INFINITY;
+        mx = fmaxf(mx, l[j]);
+    }
+    for (int o = 32; o > 0; o >>= 1) mx = fmaxf(mx, __shfl_xor(mx, o));
+    float red[16];
+    for (int j = 0; j < 16; j++) red[j] = p[j] = j < slots ? expf(l[j] - mx) : 0.0f;
+    // tree over E slots: strides E/2 .. 64 pair slots inside a lane, strides 32 .. 1 pair lanes
+#pragma unroll
+    for (int st = 8; st > 0; st >>= 1) {
+        if (st <= (slots >> 1)) {
+#pragma unroll
+            for (int j = 0; j < st; j++) red[j] += red[j + st];
+        }
+    }
+    float den = red[0];
+    for (int o = 32; o > 0; o >>= 1) den += __shfl_down(den, o);
+    den = __shfl(den, 0);
+    for (int j = 0; j < 16; j++) p[j] = j < slots ? p[j] / den : -2.0f;
+    float sum = 0.0f, my_w = 0.0f;
+    int my_id = 0;
+    for (int k = 0; k < K; k++) {
+        // key = (probability bits, inverted expert id): the maximum is the best probability, lowest id on ties
+        unsigned long long best = 0;
+        for (int j = 0; j < 16; j++) {
+            if (j < slots && p[j] >= 0.0f) {
+                const unsigned long long key = ((unsigned long long)__float_as_uint(p[j]) << 32) | (unsigned)(0xFFFFFFFFu - (unsigned)(j * 64 + lane));
+                best = key > best ? key : best;
+            }
+        }
+        for (int o = 32; o > 0; o >>= 1) {
+            const unsigned long long other = __shfl_xor(best, o);
+            best = other > best ? other : best;
+        }
+        const int pick = (int)(0xFFFFFFFFu - (unsigned)(best & 0xFFFFFFFFull));
+        const float pw = __uint_as_float((unsigned)(best >> 32));
+        sum += pw;
+        if (lane == k) {
+            my_w = pw;
+            my_id = pick;
+        }
+        if ((pick & 63) == lane) {
+            for (int j = 0; j < 16; j++)
+                if (j == (pick >> 6)) p[j] = -1.0f;
+        }
+    }
+    unsigned cold = 0;
+    if (lane < K) {
+        wts[(size_t)t * K + lane] = my_w / sum;
+        ids[(size_t)t * K + lane] = my_id;
+        if (table) {
+            if (gu_ptrs) gu_ptrs[(size_t)t * K + lane] = table[my_id * 2];
+            if (dn_ptrs) dn_ptrs[(size_t)t * K + lane] = table[my_id * 2 + 1];
+        }
+        if (sel_counts) atomicAdd(&sel_counts[my_id], 1ull);
+        if (bitmap && !((bitmap[my_id >> 5] >> (my_id & 31)) & 1u)) cold = 1u << lane;
+    }
+    for (int o = 32; o > 0; o >>= 1) cold |= __shfl_xor(cold, o);
+    if (lane == 0) {
+        if (cold_mask) cold_mask[t] = cold;
+        if (counters) {
+            atomicAdd(&counters[0], (unsigned long long)K);
+            atomicAdd(&counters[1], (unsigned long long)__popc(cold));
+        }
+    }
+}
+
+// reference: silu_mul_combo, engine/src/kernels.rs:1562-1570: [C][2 I] -> [C][I], I = g_geo.inter
+extern "C" __global__ void silu_mul_combo(const float* __restrict__ h1, float* __restrict__ h2, const int* __restrict__ n_p) {
+    const int i = (int)(blockIdx.x * blockDim.x + threadIdx.x);
+    if (i >= *n_p) return;
+    const int inter = g_geo.inter;
+    const int c = i / inter, j = i % inter;
+    h2[i] = silu_mul(h1[(size_t)c * 2 * inter + j], h1[(size_t)c * 2 * inter + inter + j]);
+}
+
+// reference: acc_combo, engine/src/kernels.rs:1583-1592: y[t][c] += sum_j rw[t][j] * x[t K + j][c],
+// j ascending, one rounding per multiply and per add.  grid (ceil(H / 256), T), block 256.
+extern "C" __global__ void acc_combo(const float* __restrict__ x, const float* __restrict__ rw, float* __restrict__ y) {
+    const int H = g_geo.hidden, K = g_geo.topk;
+    const int c = (int)(blockIdx.x * blockDim.x + threadIdx.x), t = (int)blockIdx.y;
+    if (c >= H) return;
+    float acc = 0.0f;
+    for (int j = 0; j < K; j++) {
+        const float prod = rw[t * K + j] * x[((size_t)t * K + j) * H + c];
+        acc = __fadd_rn(acc, prod);
+    }
+    y[(size_t)t * H + c] += acc;
+}
+
+// ------------------------------------------------------------------ greedy argmax
+// (the order itself: device_common.h)
+// grid (1), block up to 1024
+extern "C" __global__ void __launch_bounds__(1024) argmax_k(const float* __restrict__ logits, int* __restrict__ out, const int* __restrict__ n_p) {
+    __shared__ float sv[16];
+    __shared__ int si[16];
+    const int n = *n_p;
+    Best b{-3.0e38f, 0};
+    for (int i = (int)threadIdx.x; i < n; i += (int)blockDim.x) {
+        const float v = logits[i];
+        if (better(v, i, b.v, b.i)) {
+            b.v = v;
+            b.i = i;
+        }
+    }
+    b = wave_best(b);
+    const int wave = (int)(threadIdx.x >> 6), waves = (int)((blockDim.x + 63) >> 6);
+    if (lane_id() == 0) {
+        sv[wave] = b.v;
+        si[wave] = b.i;
+    }
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        for (int w = 1; w < waves; w++)
+            if (better(sv[w], si[w], b.v, b.i)) {
+                b.v = sv[w];
+                b.i = si[w];
+            }
+        out[0] = b.i;
+    }
+}

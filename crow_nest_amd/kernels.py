@@ -1,0 +1,139 @@
+"""Host-side mirror of the reference's kernel table and launch shim for the NVFP4 path.
+
+Reference interface (engine/src/kernels.rs:5128-5348, engine/src/cuda.rs:274-284,485-509):
+
+    let module = cuda::compile(&kgeo.source());      ->  module = compile(geo)
+    let k = Kernels::new(&module, p2);               ->  k = Kernels(module)
+    launch_v(k.f("gemv_nvfp4_w"), gx, gy, gz, bx, &[w, x, gs, y, k_p, rows_p]);
+                                                      ->  launch_v(k.f("gemv_nvfp4_w"), gx, gy, gz, bx, [w, x, gs, y, k_p, rows_p])
+
+Same names, same argument meaning (every value a device address), same failure behaviour: a missing
+name raises ``KernelMissing("kernel missing: <name>")`` where the reference panics with that text; a
+HIP error raises where the reference's ``cuda::ck`` panics.  Grid and block come from
+``launch_dims`` so that wave64 geometry stays inside the library.
+"""
+from __future__ import annotations
+
+import ctypes as C
+from dataclasses import dataclass
+
+from . import lib as _l
+
+
+class KernelMissing(KeyError):
+    pass
+
+
+@dataclass(frozen=True)
+class KernelGeo:
+    """The geometry the reference bakes into its kernel source (kernels.rs:5040-5125, CN_* defines)."""
+    experts: int = 0
+    topk: int = 0
+    hidden: int = 0
+    inter: int = 0
+
+
+class Module:
+    """``cuda::Module``: the loaded code objects (here: the ahead-of-time gfx950 objects in the library)."""
+
+    def __init__(self, handle: int):
+        self.handle = handle
+
+    def get(self, name: str) -> int:
+        out = C.c_void_p()
+        rc = _l.lib().crow_hip_module_get(self.handle, name.encode(), C.byref(out))
+        if rc == -2:
+            raise KernelMissing(f"kernel missing: {name}")
+        _l.check(rc, f"Module::get({name})")
+        return out.value
+
+    def unload(self) -> None:
+        if self.handle:
+            _l.check(_l.lib().crow_hip_module_unload(self.handle), "Module::unload")
+            self.handle = 0
+
+
+def compile(geo: KernelGeo | None = None) -> Module:  # noqa: A001 - the reference's name
+    """``cuda::compile``: nothing is compiled at run time; loads the module and writes the geometry."""
+    _l.ensure_init()
+    out = C.c_void_p()
+    _l.check(_l.lib().crow_hip_module_load(C.byref(out)), "crow_hip_module_load")
+    if geo is not None:
+        set_geo(geo)
+    return Module(out.value)
+
+
+def set_geo(geo: KernelGeo) -> None:
+    _l.ensure_init()
+    _l.check(_l.lib().crow_hip_set_geo(geo.experts, geo.topk, geo.hidden, geo.inter), "crow_hip_set_geo")
+
+
+class Kernels:
+    """``Kernels::new`` resolves every launched name once; ``f`` looks one up."""
+
+    def __init__(self, module: Module):
+        L = _l.lib()
+        self.map = {}
+        for i in range(L.crow_hip_function_count()):
+            name = L.crow_hip_function_name(i).decode()
+            self.map[name] = module.get(name)
+
+    def f(self, name: str) -> int:
+        try:
+            return self.map[name]
+        except KeyError:
+            raise KernelMissing(f"kernel missing: {name}") from None
+
+
+def launch_v(f: int, gx: int, gy: int, gz: int, bx: int, vals) -> None:
+    """``launch_v``: asynchronous launch on the current stream; every value is a device address."""
+    n = len(vals)
+    arr = (C.c_uint64 * n)(*[int(v) for v in vals])
+    _l.check(_l.lib().crow_hip_launch(f, gx, gy, gz, bx, arr, n, None), "launch_v")
+
+
+def sync() -> None:
+    _l.check(_l.lib().crow_hip_sync(), "sync")
+
+
+def launch_sync(f: int, gx: int, gy: int, gz: int, bx: int, vals) -> None:
+    launch_v(f, gx, gy, gz, bx, vals)
+    sync()
+
+
+def status() -> None:
+    """Raise if a launch since the last call refused its shape or did not fit the workspace."""
+    _l.check(_l.lib().crow_hip_status(), "kernel status")
+
+
+def launch_dims(name: str, rows: int, k_dim: int, z: int = 1) -> tuple[int, int, int, int]:
+    d = _l.Dims()
+    rc = _l.lib().crow_hip_launch_dims(name.encode(), rows, k_dim, z, C.byref(d))
+    if rc == -2:
+        raise KernelMissing(f"kernel missing: {name}")
+    _l.check(rc, f"launch_dims({name}, {rows}, {k_dim}, {z})")
+    return d.gx, d.gy, d.gz, d.bx
+
+
+class Event:
+    """A HIP event on the library's current stream (the stream every launch_v goes to)."""
+
+    def __init__(self):
+        h = C.c_void_p()
+        _l.check(_l.lib().crow_hip_event_create(C.byref(h)), "crow_hip_event_create")
+        self.h = h
+
+    def record(self) -> "Event":
+        _l.check(_l.lib().crow_hip_event_record(self.h), "crow_hip_event_record")
+        return self
+
+    def elapsed_ms(self, stop: "Event") -> float:
+        ms = C.c_float()
+        _l.check(_l.lib().crow_hip_event_elapsed_ms(self.h, stop.h, C.byref(ms)), "crow_hip_event_elapsed_ms")
+        return float(ms.value)
+
+    def __del__(self):
+        try:
+            _l.lib().crow_hip_event_destroy(self.h)
+        except Exception:
+            pass

@@ -1,0 +1,157 @@
+"""Host-side weight types and the load path: container bytes -> device -> tiled layout.
+
+Mirrors, for the NVFP4 path only:
+  * ``cpu_nvfp4::Nvfp4Matrix`` (engine/src/cpu_nvfp4.rs:107-141): borrowed container bytes +
+    rows / cols / global scale, with the same shape checks and error texts;
+  * ``weights::load_fp4 -> Fp4 {w, gs}`` and ``PW::Fp4(w, gs)`` (engine/src/weights.rs:26-33,
+    engine/src/gen.rs:234-237): device bytes + a one-float device scalar;
+  * the loader's scale rule 0x7F -> 0x7E (engine/src/gen.rs:2178-2187, residency.rs:126-137), which the
+    library's repacker applies while it re-tiles (``crow_hip_repack_nvfp4``);
+  * ``Params`` (engine/src/gen.rs:2913-2925): the 4-byte device words kernels read their scalars from.
+PyTorch tensors are used as device allocations only.
+"""
+from __future__ import annotations
+
+from dataclasses import dataclass
+
+import numpy as np
+import torch
+
+from . import lib as _l
+
+BLOCK_BYTES = 36
+BLOCK_VALUES = 64
+
+
+@dataclass(frozen=True)
+class Nvfp4Matrix:
+    """One NVFP4 matrix [rows, cols] over container bytes on the host."""
+    bytes: np.ndarray
+    rows: int
+    cols: int
+    global_scale: float
+
+    @staticmethod
+    def byte_len(rows: int, cols: int) -> int:
+        return rows * (cols // BLOCK_VALUES) * BLOCK_BYTES
+
+    @staticmethod
+    def new(data, rows: int, cols: int, global_scale: float) -> "Nvfp4Matrix":
+        b = np.ascontiguousarray(np.asarray(data, dtype=np.uint8).reshape(-1))
+        if cols == 0 or cols % BLOCK_VALUES != 0:
+            raise ValueError(f"cpu_nvfp4: {cols} columns are not whole 64-value NVFP4 blocks")
+        want = Nvfp4Matrix.byte_len(rows, cols)
+        if b.size != want:
+            raise ValueError(f"cpu_nvfp4: [{rows}, {cols}] needs {want} B, got {b.size}")
+        return Nvfp4Matrix(b, rows, cols, float(np.float32(global_scale)))
+
+
+def _device() -> torch.device:
+    if not torch.cuda.is_available():
+        raise RuntimeError("crow_nest_amd needs a gfx950 GPU: no HIP device is visible (there is no CPU path)")
+    return torch.device("cuda", 0)
+
+
+def tiled_bytes(rows: int, cols: int) -> int:
+    return int(_l.lib().crow_hip_tiled_bytes(rows, cols))
+
+
+@dataclass
+class Fp4:
+    """``PW::Fp4(w, gs)``: tiled weight bytes and the global scale, both on the device."""
+    w: torch.Tensor   # uint8 [tiled_bytes]
+    gs: torch.Tensor  # float32 [1]
+    rows: int
+    cols: int
+
+    @property
+    def w_ptr(self) -> int:
+        return self.w.data_ptr()
+
+    @property
+    def gs_ptr(self) -> int:
+        return self.gs.data_ptr()
+
+
+def repack_into(raw_dev: torch.Tensor, rows: int, cols: int, dst: torch.Tensor) -> None:
+    """Container bytes on the device -> tiled layout (applies the scale rule)."""
+    _l.ensure_init()
+    assert raw_dev.is_cuda and dst.is_cuda and raw_dev.dtype == torch.uint8 and dst.dtype == torch.uint8
+    if raw_dev.numel() != Nvfp4Matrix.byte_len(rows, cols):
+        raise ValueError(f"cpu_nvfp4: [{rows}, {cols}] needs {Nvfp4Matrix.byte_len(rows, cols)} B, got {raw_dev.numel()}")
+    if dst.numel() < tiled_bytes(rows, cols):
+        raise ValueError("tiled destination too small")
+    _l.check(_l.lib().crow_hip_repack_nvfp4(raw_dev.data_ptr(), rows, cols, dst.data_ptr()), "crow_hip_repack_nvfp4")
+
+
+def load_fp4(m: Nvfp4Matrix) -> Fp4:
+    """``load_fp4``: upload the container bytes, re-tile them on the device, keep (w, gs)."""
+    dev = _device()
+    _l.ensure_init()
+    raw = torch.from_numpy(m.bytes).to(dev)
+    w = torch.empty(tiled_bytes(m.rows, m.cols), dtype=torch.uint8, device=dev)
+    repack_into(raw, m.rows, m.cols, w)
+    gs = torch.tensor([m.global_scale], dtype=torch.float32, device=dev)
+    return Fp4(w, gs, m.rows, m.cols)
+
+
+def unpack(w: Fp4) -> np.ndarray:
+    """Tiled -> container bytes (scale bytes canonical); for round-trip checks."""
+    out = torch.empty(Nvfp4Matrix.byte_len(w.rows, w.cols), dtype=torch.uint8, device=w.w.device)
+    _l.check(_l.lib().crow_hip_unpack_nvfp4(w.w.data_ptr(), w.rows, w.cols, out.data_ptr()), "crow_hip_unpack_nvfp4")
+    return out.cpu().numpy()
+
+
+def dequant(w: Fp4) -> torch.Tensor:
+    """f32 [rows, cols] on the device, bit-exact with the reference decode after the scale rule."""
+    out = torch.empty((w.rows, w.cols), dtype=torch.float32, device=w.w.device)
+    _l.check(_l.lib().crow_hip_dequant_tiled(w.w.data_ptr(), w.gs.data_ptr(), w.rows, w.cols, out.data_ptr()),
+             "crow_hip_dequant_tiled")
+    return out
+
+
+@dataclass
+class ExpertSlabs:
+    """An expert tensor [E][rows][cols] re-tiled per expert: slab e starts at e * slab_bytes."""
+    w: torch.Tensor
+    gs: torch.Tensor
+    experts: int
+    rows: int
+    cols: int
+    slab_bytes: int
+
+    def ptr(self, e: int) -> int:
+        return self.w.data_ptr() + e * self.slab_bytes
+
+
+def load_expert_slabs(data, experts: int, rows: int, cols: int, global_scale: float) -> ExpertSlabs:
+    """Flash-Next style expert tensor (engine/src/residency.rs:108-117: one global scale, expert e's
+    container slab at e * rows * cols / 64 * 36) -> per-expert contiguous tiled slabs."""
+    dev = _device()
+    _l.ensure_init()
+    b = np.ascontiguousarray(np.asarray(data, dtype=np.uint8).reshape(-1))
+    per = Nvfp4Matrix.byte_len(rows, cols)
+    if b.size != experts * per:
+        raise ValueError(f"cpu_nvfp4: [{experts}][{rows}, {cols}] needs {experts * per} B, got {b.size}")
+    slab = tiled_bytes(rows, cols)
+    raw = torch.from_numpy(b).to(dev)
+    w = torch.empty(experts * slab, dtype=torch.uint8, device=dev)
+    for e in range(experts):
+        repack_into(raw[e * per:(e + 1) * per], rows, cols, w[e * slab:(e + 1) * slab])
+    gs = torch.tensor([float(np.float32(global_scale))], dtype=torch.float32, device=dev)
+    return ExpertSlabs(w, gs, experts, rows, cols, slab)
+
+
+class Params:
+    """Device words for kernel scalars (``Params`` of engine/src/gen.rs:2913-2925), created on demand."""
+
+    def __init__(self):
+        self._dev = _device()
+        self._cache: dict[int, torch.Tensor] = {}
+
+    def i32(self, v: int) -> int:
+        t = self._cache.get(v)
+        if t is None:
+            t = torch.tensor([v], dtype=torch.int32, device=self._dev)
+            self._cache[v] = t
+        return t.data_ptr()

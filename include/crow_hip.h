@@ -1,0 +1,110 @@
+/*
+ * libcrow_hip.so - the C ABI of the MI355X (gfx950) NVFP4 weight x activation library.
+ *
+ * It replaces, for the NVFP4 hot path only, the reference engine's NVRTC compile/launch layer:
+ *   engine/src/cuda.rs:274-284      compile(src) -> Module            -> crow_hip_module_load
+ *   engine/src/cuda.rs:485-509      Module::get(name), Module::unload -> crow_hip_module_get / _unload
+ *   engine/src/kernels.rs:5128-5240 Kernels::new / Kernels::f(name)   -> crow_hip_get_function
+ *   engine/src/kernels.rs:5284-5348 launch_v / launch_sync            -> crow_hip_launch (+ crow_hip_sync)
+ *   engine/src/kernels.rs:5040-5125 KernelGeo prelude (CN_* defines)  -> crow_hip_set_geo
+ *   engine/src/cuda.rs:398-687      alloc / free / upload / dtoh      -> crow_hip_alloc ... crow_hip_download
+ *   engine/src/cuda.rs:13-24        set_stream / cur_stream           -> crow_hip_set_stream / crow_hip_cur_stream
+ *   engine/src/weights.rs:26-33, gen.rs:2178-2198 (load_fp4 + the 0x7F rule) -> crow_hip_repack_nvfp4
+ * The code objects are built ahead of time for gfx950 and live inside the library; nothing is
+ * compiled at run time.  Plain pointers and sizes only; every call returns 0 on success or a
+ * negative crow_status / a positive hipError_t, never aborts and never throws.
+ *
+ * Kernel arguments keep the reference convention: every value handed to crow_hip_launch is a
+ * 64-bit device address; scalars live in 4-byte device words.  Weight pointers are to tensors in
+ * the library's tiled layout (crow_hip_repack_nvfp4), not to raw container bytes.
+ *
+ * Threading: like the reference engine (one engine thread, one process-global current stream)
+ * the library keeps one workspace per process; launches that use it must be ordered on one stream.
+ */
+#ifndef CROW_HIP_H
+#define CROW_HIP_H
+#include <stddef.h>
+#include <stdint.h>
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef struct crow_fn_s* crow_fn_t;     /* opaque kernel handle (CUfunction in the reference) */
+typedef struct crow_module_s* crow_module_t; /* opaque module handle (CUmodule in the reference) */
+
+enum crow_status {
+    CROW_OK = 0,
+    CROW_ERR_NOT_INITIALIZED = -1,
+    CROW_ERR_KERNEL_MISSING = -2, /* the Rust shim turns this into panic!("kernel missing: {name}") */
+    CROW_ERR_BAD_ARGUMENT = -3,
+    CROW_ERR_ARG_COUNT = -4,      /* launch with a different number of values than the kernel takes */
+    CROW_ERR_WORKSPACE = -5,      /* a launch needed more split-K workspace than the library holds */
+    CROW_ERR_SCALE_BYTE = -6,     /* repack met scale byte 0xFF (reads 480 in the reference; E4M3 cannot hold it) */
+    CROW_ERR_SHAPE = -7,
+    CROW_ERR_GEO = -8
+};
+
+/* launch geometry chosen by the library for a kernel and a problem (wave64 shapes stay out of the caller) */
+typedef struct crow_dims {
+    uint32_t gx, gy, gz, bx;
+} crow_dims;
+
+/* ---- lifetime ---- */
+int crow_hip_init(int device);            /* Ctx::init, engine/src/cuda.rs:435 */
+int crow_hip_shutdown(void);
+const char* crow_hip_error_string(int code);
+int crow_hip_device_name(char* out, size_t n);
+
+/* ---- module / kernel table ---- */
+int crow_hip_module_load(crow_module_t* out);
+int crow_hip_module_unload(crow_module_t m);
+int crow_hip_module_get(crow_module_t m, const char* name, crow_fn_t* out);
+int crow_hip_get_function(const char* name, crow_fn_t* out);
+int crow_hip_function_count(void);
+const char* crow_hip_function_name(int index);
+int crow_hip_function_arg_count(crow_fn_t f);
+
+/* ---- geometry the reference compiles into its kernel text ---- */
+int crow_hip_set_geo(int experts, int topk, int hidden, int inter);
+
+/* ---- launch ---- */
+int crow_hip_launch(crow_fn_t f, uint32_t gx, uint32_t gy, uint32_t gz, uint32_t bx, const uint64_t* vals,
+                    uint32_t n_vals, void* stream);
+/* grid/block for `name` on a [rows, k_dim] tensor with `z` token rows (batched kernels) or combos
+ * (routed kernels); 1 otherwise.  The choice depends on (rows, k_dim) only, never on z. */
+int crow_hip_launch_dims(const char* name, uint32_t rows, uint32_t k_dim, uint32_t z, crow_dims* out);
+/* reads and clears the device status word (synchronises the current stream): CROW_OK or CROW_ERR_* */
+int crow_hip_status(void);
+int crow_hip_reset_workspace(void);
+
+/* ---- streams and memory (thin shims over HIP) ---- */
+void crow_hip_set_stream(void* stream);
+void* crow_hip_cur_stream(void);
+int crow_hip_sync(void);
+int crow_hip_alloc(size_t bytes, void** out);   /* zero-filled, like alloc_named (engine/src/cuda.rs:398-427) */
+int crow_hip_free(void* p);
+int crow_hip_upload(void* dst, const void* src, size_t bytes);   /* upload_into: async on a capture stream, else + sync */
+int crow_hip_download(void* dst, const void* src, size_t bytes); /* dtoh: blocking */
+
+/* ---- timing on the current stream (HIP events; what CROW_KPROF books per launch in the reference,
+ * engine/src/kernels.rs:5245-5280, is measured by the caller with these) ---- */
+int crow_hip_event_create(void** out);
+int crow_hip_event_record(void* ev);                              /* on the current stream */
+int crow_hip_event_elapsed_ms(void* start, void* stop, float* ms); /* waits for `stop` */
+int crow_hip_event_destroy(void* ev);
+
+/* ---- load-time repack (the one call the reference does not have) ---- */
+size_t crow_hip_container_bytes(uint32_t rows, uint32_t cols);
+size_t crow_hip_tiled_bytes(uint32_t rows, uint32_t cols);
+/* src_dev: container bytes [rows][cols/64][36] already on the device; dst_dev: crow_hip_tiled_bytes.
+ * Applies the scale rule (0x7F -> 0x7E).  Expert tensors [E][rows][cols]: call once per expert
+ * slab, the tiled slabs are then contiguous per expert. */
+int crow_hip_repack_nvfp4(const void* src_dev, uint32_t rows, uint32_t cols, void* dst_dev);
+int crow_hip_unpack_nvfp4(const void* src_dev, uint32_t rows, uint32_t cols, void* dst_dev);
+/* out_dev: f32 [rows][cols], bit-exact with the reference decode after the scale rule */
+int crow_hip_dequant_tiled(const void* w_dev, const float* gs_dev, uint32_t rows, uint32_t cols, float* out_dev);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

@@ -1,0 +1,54 @@
+"""Shared helpers of the GPU parity tests: input builders, the parity metrics, env overrides."""
+from __future__ import annotations
+
+import contextlib
+import os
+
+import numpy as np
+
+from oracle import oracle as orc
+from refgen import normal_f32
+
+TOL = 1e-3  # north star: GEMV outputs within max relative error 1e-3 of the CPU path
+
+
+def rel_err(y: np.ndarray, ref: np.ndarray) -> float:
+    """max_i |y_i - ref_i| / max(|ref_i|, 1e-3 * rms(ref)) per output row, worst row."""
+    y = np.asarray(y, np.float64).reshape(ref.shape)
+    r = np.asarray(ref, np.float64)
+    if r.ndim == 1:
+        r, y = r[None], y[None]
+    rms = np.sqrt((r * r).mean(axis=1, keepdims=True))
+    den = np.maximum(np.abs(r), 1e-3 * np.maximum(rms, 1e-30))
+    return float(np.max(np.abs(y - r) / den))
+
+
+def gamma_ratio(y, w, rows, cols, gs, x) -> float:
+    """max |y - y_f64| / (gamma(K/16 + 10) * sum|w x|): <= 1 means inside the reference's own fp32 bound."""
+    yr, ab = orc.gemv_f64(w, rows, cols, gs, x)
+    y = np.asarray(y, np.float64).reshape(yr.shape)
+    return float(np.max(np.abs(y - yr) / np.maximum(orc.gamma(cols) * ab, np.finfo(np.float64).tiny)))
+
+
+def quantized_normal(seed: int, stream: int, rows: int, cols: int, sigma: float = 0.02):
+    """BASELINE's weights: N(0, sigma^2) through the ceil encoder -> (container bytes, global scale)."""
+    v = normal_f32(seed, stream, rows * cols, sigma)
+    return orc.quantize_ceil(v)
+
+
+@contextlib.contextmanager
+def env(**kv):
+    old = {k: os.environ.get(k) for k in kv}
+    try:
+        for k, v in kv.items():
+            if v is None:
+                os.environ.pop(k, None)
+            else:
+                os.environ[k] = str(v)
+        yield
+    finally:
+        for k, v in old.items():
+            if v is None:
+                os.environ.pop(k, None)
+            else:
+                os.environ[k] = v

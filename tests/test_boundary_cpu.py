@@ -1,0 +1,83 @@
+"""CPU-side checks of the drop-in boundary: the shared library loads and exports exactly what
+include/crow_hip.h declares, host-side types refuse bad shapes with the reference's messages, and
+nothing computes without a GPU (no CPU fallback)."""
+import os
+import re
+
+import numpy as np
+import pytest
+
+from conftest import ROOT
+from crow_nest_amd import lib as L
+from crow_nest_amd.weights import Nvfp4Matrix
+
+
+def _declared():
+    text = open(os.path.join(ROOT, "include", "crow_hip.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(crow_hip_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_library_exports_every_declared_symbol():
+    assert os.path.exists(L.library_path()), "libcrow_hip.so is not built: run __graft_entry__.build()"
+    lib = L.lib()
+    declared = _declared()
+    assert declared, "no declarations found"
+    for name in declared:
+        assert hasattr(lib, name), f"{name} is declared in include/crow_hip.h but not exported"
+    assert sorted(L.EXPORTS) == declared
+
+
+def test_kernel_table_names_without_a_device():
+    lib = L.lib()
+    n = lib.crow_hip_function_count()
+    names = [lib.crow_hip_function_name(i).decode() for i in range(n)]
+    for want in ["gemv_nvfp4_w", "gemv_nvfp4_gu", "gemv_nvfp4_wm", "gemv_nvfp4_gum", "gemv_fp4", "gemv_fp4_b", "gemv_fp4_bs",
+                 "gemv_fp4_b1k", "gemv_fp4_ptrb", "router_top10", "silu_mul_combo", "acc_combo", "argmax_k",
+                 "dequant_fp4_flat", "gemv_nvfp4_w_argmax", "moe_gate_up_silu", "moe_down_combine", "gemm_nvfp4_bf16"]:
+        assert want in names, want
+    import ctypes as C
+    out = C.c_void_p()
+    assert lib.crow_hip_get_function(b"no_such_kernel", C.byref(out)) == -2  # CROW_ERR_KERNEL_MISSING
+    assert b"kernel missing" in lib.crow_hip_error_string(-2)
+    assert lib.crow_hip_tiled_bytes(17408, 5120) == 17408 * 5120 // 64 * 36 == lib.crow_hip_container_bytes(17408, 5120)
+    assert lib.crow_hip_tiled_bytes(1, 64) == 9216  # one padded tile
+
+
+def test_launch_dims_depend_on_the_matrix_only():
+    import ctypes as C
+    lib = L.lib()
+    d1, d4 = L.Dims(), L.Dims()
+    assert lib.crow_hip_launch_dims(b"gemv_nvfp4_w", 17408, 5120, 1, C.byref(d1)) == 0
+    assert lib.crow_hip_launch_dims(b"gemv_nvfp4_wm", 17408, 5120, 1, C.byref(d4)) == 0
+    assert (d1.gx, d1.gy, d1.gz, d1.bx) == (d4.gx, d4.gy, d4.gz, d4.bx)  # verify rows == decode row, bit for bit
+    assert d1.gy == 272 and d1.bx % 64 == 0
+    assert lib.crow_hip_launch_dims(b"gemv_nvfp4_w", 8, 96, 1, C.byref(d1)) == -7  # 96 columns: not whole blocks
+
+
+def test_matrix_shapes_are_checked_like_the_reference():
+    b = np.zeros(Nvfp4Matrix.byte_len(3, 128), np.uint8)
+    Nvfp4Matrix.new(b, 3, 128, 1.0)
+    with pytest.raises(ValueError, match="96 columns are not whole 64-value NVFP4 blocks"):
+        Nvfp4Matrix.new(b, 3, 96, 1.0)
+    with pytest.raises(ValueError, match=r"\[3, 128\] needs 216 B, got 215"):
+        Nvfp4Matrix.new(b[1:], 3, 128, 1.0)
+
+
+def test_no_cpu_fallback():
+    import torch
+    if torch.cuda.is_available():
+        pytest.skip("a GPU is visible")
+    from crow_nest_amd.weights import load_fp4
+    m = Nvfp4Matrix.new(np.zeros(Nvfp4Matrix.byte_len(64, 256), np.uint8), 64, 256, 1.0)
+    with pytest.raises(RuntimeError, match="no HIP device"):
+        load_fp4(m)
+
+
+def test_product_does_not_import_the_oracle():
+    pkg = os.path.join(ROOT, "crow_nest_amd")
+    for dirpath, _, files in os.walk(pkg):
+        for f in files:
+            if f.endswith((".py", ".h", ".hip", ".cpp", "Makefile")):
+                text = open(os.path.join(dirpath, f)).read()
+                assert "oracle" not in text.lower(), (dirpath, f)

@@ -1,0 +1,293 @@
+"""GPU parity: the HIP path (through the C ABI, via the host mirror) against the CPU oracle.
+
+Bars: dequantised weights bit-exact; integer / index results bit-exact; GEMV outputs within
+max relative error 1e-3 of the CPU path (TOL below; the denominator floors at 1e-3 of the row's
+rms so that an output that cancels to ~0 does not divide by nothing), and additionally inside the
+reference's own fp32 bound gamma(K/16 + 10) * sum|w x| against an f64 evaluation.
+"""
+import numpy as np
+import pytest
+import torch
+
+from gpu_common import TOL, env, gamma_ratio, quantized_normal, rel_err
+from oracle import oracle as orc
+from refgen import SplitMix64, normal_f32, random_nvfp4, scale_mix, synth_nvfp4
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def eng():
+    from crow_nest_amd.engine import Engine
+    from crow_nest_amd.kernels import KernelGeo
+    return Engine(KernelGeo(experts=256, topk=8, hidden=2048, inter=512))
+
+
+def _load(w, rows, cols, gs):
+    from crow_nest_amd.weights import Nvfp4Matrix, load_fp4
+    return load_fp4(Nvfp4Matrix.new(w, rows, cols, gs))
+
+
+def _dev(a):
+    return torch.from_numpy(np.ascontiguousarray(a)).cuda()
+
+
+def _bf16_dev(a_f32):
+    """RNE to bf16 on the host (the oracle's rounding), bits shipped to the device."""
+    bits = orc.f32_to_bf16_bits(a_f32)
+    return torch.from_numpy(bits.view(np.int16)).cuda().view(torch.bfloat16), orc.bf16_bits_to_f32(bits)
+
+
+# ---------------------------------------------------------------- layout + dequant (bit-exact)
+
+@pytest.mark.parametrize("rows,cols", [(64, 256), (37, 256), (1, 64), (65, 320), (128, 64), (200, 5120), (16, 2048)])
+def test_repack_round_trip_and_dequant_bits(eng, rows, cols):
+    from crow_nest_amd.weights import dequant, unpack
+    print(f"case rows={rows} cols={cols}", flush=True)
+    w = random_nvfp4(rows * 1000 + cols, rows, cols, scale_lo=0, scale_hi=0x7F, p7f=1 / 32)
+    gs = 1.7e-3
+    f = _load(w, rows, cols, gs)
+    back = unpack(f)
+    canon = w.copy().reshape(-1, 36)
+    canon[:, :4][canon[:, :4] == 0x7F] = 0x7E
+    assert np.array_equal(back, canon.reshape(-1))  # exact inverse up to the scale rule
+    got = dequant(f).cpu().numpy().reshape(-1)
+    want = orc.dequant(w, gs)
+    assert np.array_equal(got.view(np.uint32), want.view(np.uint32))
+    eng.check()
+
+
+def test_dequant_every_scale_byte_and_the_refused_one(eng):
+    from crow_nest_amd.lib import CrowHipError
+    from crow_nest_amd.weights import dequant
+    rows, cols = 256, 64
+    blocks = np.zeros((rows, 36), np.uint8)
+    g = np.random.default_rng(1)
+    blocks[:, 4:] = g.integers(0, 256, size=(rows, 32), dtype=np.uint8)
+    for r in range(rows):
+        blocks[r, :4] = [r, (r + 64) % 256, (r + 128) % 256, (r + 192) % 256]
+    ok = blocks.copy()
+    ok[:, :4][ok[:, :4] == 0xFF] = 0x7F
+    gs = 9.3e-5
+    got = dequant(_load(ok.reshape(-1), rows, cols, gs)).cpu().numpy().reshape(-1)
+    want = orc.dequant(ok.reshape(-1), gs)  # bit 7 ignored, 0x7F -> 448
+    assert np.array_equal(got.view(np.uint32), want.view(np.uint32))
+    with pytest.raises(CrowHipError) as ei:  # 0xFF reads 480 in the reference; the tiled layout cannot hold it
+        _load(blocks.reshape(-1), rows, cols, gs)
+    assert ei.value.code == -6
+    eng.check()
+
+
+def test_dequant_fp4_flat_is_the_raw_container_decode(eng):
+    from crow_nest_amd.kernels import launch_v
+    w = random_nvfp4(5, 64, 512, scale_lo=0, scale_hi=0x100, p7f=1 / 16)
+    gs = torch.tensor([2.3e-4], dtype=torch.float32, device="cuda")
+    n = 64 * 512
+    out = torch.empty(n, dtype=torch.float32, device="cuda")
+    wd = _dev(w)
+    launch_v(eng.k.f("dequant_fp4_flat"), (n + 255) // 256, 1, 1, 256, [wd.data_ptr(), gs.data_ptr(), out.data_ptr(), eng.p.i32(n)])
+    want = orc.dequant(w, 2.3e-4, rule=False)  # 0x7F reads 480 here, as in the reference kernel
+    assert np.array_equal(out.cpu().numpy().view(np.uint32), want.view(np.uint32))
+
+
+# ---------------------------------------------------------------- dense GEMV
+
+SHAPES = [(37, 256), (16, 2048), (9, 4096), (41, 1024), (64, 64), (130, 320), (1024, 5120), (512, 17408), (2048, 512), (100, 2560)]
+
+
+@pytest.mark.parametrize("rows,cols", SHAPES)
+def test_gemv_w_against_the_cpu_path(eng, rows, cols):
+    print(f"case rows={rows} cols={cols}", flush=True)
+    rng = SplitMix64(173 + rows)
+    w = synth_nvfp4(rng, rows, cols, scale_mix) if rows * cols <= 1 << 18 else random_nvfp4(rows, rows, cols)
+    gs = 1.7e-3
+    x = rng.f(cols, 2.0)
+    ref = orc.gemv(w, rows, cols, gs, x)[0]
+    f = _load(w, rows, cols, gs)
+    y = eng.dense_proj(f, 1, _dev(x)).cpu().numpy()[0]
+    eng.check()
+    assert rel_err(y, ref) <= TOL
+    assert gamma_ratio(y, w, rows, cols, gs, x) <= 1.0
+
+
+@pytest.mark.parametrize("s,wv", [(1, 1), (1, 4), (3, 2), (5, 1), (20, 1), (2, 16)])
+def test_gemv_is_correct_for_every_split(eng, s, wv):
+    """Any (slices, waves) split gives an answer inside the bound; the same split gives the same bits."""
+    rows, cols = 300, 5120
+    w = random_nvfp4(77, rows, cols)
+    gs = 4.0e-4
+    x = normal_f32(1, 5, cols)
+    ref = orc.gemv(w, rows, cols, gs, x)[0]
+    f = _load(w, rows, cols, gs)
+    with env(CROW_GEMV_S=s, CROW_GEMV_W=wv):
+        y1 = eng.dense_proj(f, 1, _dev(x)).cpu().numpy()[0]
+        y2 = eng.dense_proj(f, 1, _dev(x)).cpu().numpy()[0]
+    eng.check()
+    assert np.array_equal(y1.view(np.uint32), y2.view(np.uint32))
+    assert rel_err(y1, ref) <= TOL and gamma_ratio(y1, w, rows, cols, gs, x) <= 1.0
+
+
+def test_verify_rows_are_bit_identical_to_one_row_decode(eng):
+    """kernels_p2.rs:391-396: row m of an M-row launch == a one-row launch on x row m."""
+    rows, cols = 700, 5120
+    w = random_nvfp4(3, rows, cols)
+    gs = 3.1e-4
+    f = _load(w, rows, cols, gs)
+    x = normal_f32(2, 9, 4 * cols).reshape(4, cols)
+    one = [eng.dense_proj(f, 1, _dev(x[m])).cpu().numpy()[0] for m in range(4)]
+    for m in (1, 2, 3, 4):
+        ym = eng.proj_m(f, m, _dev(x[:m])).cpu().numpy()
+        for j in range(m):
+            assert np.array_equal(ym[j].view(np.uint32), one[j].view(np.uint32)), (m, j)
+        assert rel_err(ym, orc.gemv(w, rows, cols, gs, x[:m])) <= TOL
+    eng.check()
+
+
+@pytest.mark.parametrize("t", [1, 2, 4])
+def test_fused_gate_up_silu_and_down(eng, t):
+    from crow_nest_amd.engine import MlpW
+    H, I = 1024, 2816
+    wg, wu, wd = random_nvfp4(11, I, H), random_nvfp4(12, I, H), random_nvfp4(13, H, I)
+    gs = (2.0e-3, 1.5e-3, 1.1e-3)
+    mlp = MlpW(_load(wg, I, H, gs[0]), _load(wu, I, H, gs[1]), _load(wd, H, I, gs[2]))
+    x = normal_f32(3, t, t * H).reshape(t, H) * np.float32(0.05)
+    # f32 activations (the reference's dtype)
+    h = eng.gate_up(mlp, t, _dev(x)).cpu().numpy()
+    g_ref, u_ref = orc.gemv(wg, I, H, gs[0], x), orc.gemv(wu, I, H, gs[1], x)
+    h_ref = orc.silu_mul(g_ref, u_ref)
+    assert rel_err(h, h_ref) <= TOL
+    y = eng.dense_ffn_w(mlp, _dev(x), t).cpu().numpy()
+    y_ref = orc.ffn(wg, gs[0], wu, gs[1], wd, gs[2], H, I, x)
+    assert rel_err(y, y_ref) <= TOL
+    # bf16 activations (BASELINE config 1): the oracle gets the exactly widened values
+    xb, xw = _bf16_dev(x)
+    hb = eng.gate_up(mlp, t, xb.reshape(t, H).contiguous()).cpu().numpy()
+    hb_ref = orc.silu_mul(orc.gemv(wg, I, H, gs[0], xw), orc.gemv(wu, I, H, gs[1], xw))
+    assert rel_err(hb, hb_ref) <= TOL
+    eng.check()
+
+
+def test_batched_token_rows(eng):
+    rows, cols, t = 192, 1024, 7
+    w = random_nvfp4(21, rows, cols)
+    gs = 8.0e-4
+    f = _load(w, rows, cols, gs)
+    x = normal_f32(4, 1, t * cols).reshape(t, cols)
+    y = eng.dense_proj(f, t, _dev(x)).cpu().numpy()
+    assert rel_err(y, orc.gemv(w, rows, cols, gs, x)) <= TOL
+    eng.check()
+
+
+# ---------------------------------------------------------------- head
+
+def test_lm_head_logits_and_greedy_token(eng):
+    rows, cols = 4096 + 64 * 3, 1024
+    w, gs = quantized_normal(0, 31, rows, cols)
+    f = _load(w, rows, cols, gs)
+    x = normal_f32(0, 32, cols)
+    ref = orc.gemv(w, rows, cols, gs, x)[0]
+    for fused in (True, False):
+        logits, idx = eng.lm_head_row(f, _dev(x), fused=fused)
+        got = logits.cpu().numpy()
+        assert rel_err(got, ref) <= TOL
+        assert int(idx.item()) == orc.argmax_ref(got)  # the index is exact on the logits the device wrote
+    assert int(idx.item()) == int(np.argmax(ref))
+    eng.check()
+
+
+def test_argmax_tie_rule(eng):
+    for n, hot in [(4096, [1030, 7, 2055]), (151936, [150000, 1023 + 1024 * 3, 1023]), (5, [4, 2]), (2048, [1, 1536, 512]),
+                   (151936, [3, 5, 6, 9, 10, 12, 100000]), (3000, [])]:
+        l = np.zeros(n, np.float32) if hot else np.full(n, -3.2e38, np.float32)
+        for i in hot:
+            l[i] = 5.0
+        got = int(eng.argmax(_dev(l)).item())
+        assert got == orc.argmax_ref(l), (n, hot)
+    g = np.random.default_rng(8)
+    l = g.standard_normal(151936).astype(np.float32)
+    assert int(eng.argmax(_dev(l)).item()) == int(np.argmax(l))
+
+
+def test_fused_head_tie_rule(eng):
+    """Equal logits in different row tiles: the fused head must pick by the reference's tree order too."""
+    rows, cols = 2048 + 128, 64
+    blocks = np.zeros((rows, 36), np.uint8)
+    blocks[:, 0] = 0x38  # scale 1.0
+    for r in (1030, 7, 2055):  # value 2 (code 4) at column 0
+        blocks[r, 4] = 0x04
+    f = _load(blocks.reshape(-1), rows, cols, 1.0)
+    x = np.ones(cols, np.float32)
+    logits, idx = eng.lm_head_row(f, _dev(x), fused=True)
+    l = logits.cpu().numpy()
+    assert l[7] == 2.0 and l[1030] == 2.0 and l[0] == 0.0
+    assert int(idx.item()) == orc.argmax_ref(l) == 1030
+    eng.check()
+
+
+# ---------------------------------------------------------------- routed experts
+
+def test_router_small_kernels(eng):
+    g = np.random.default_rng(12)
+    logits = g.standard_normal((5, 256)).astype(np.float32)
+    logits[3, [9, 200, 77]] = 4.0  # three-way tie for the top: lowest ids first
+    ids, wts, _, _ = eng.router(_dev(logits))
+    ids_ref, w_ref = orc.router_topk(logits, 8)
+    assert np.array_equal(ids.cpu().numpy(), ids_ref)
+    assert np.allclose(wts.cpu().numpy(), w_ref, rtol=2e-6, atol=0)  # device expf vs libm expf: last-ulp
+    assert ids_ref[3, :3].tolist() == [9, 77, 200]
+    # SwiGLU per combo and the weighted combine: same f32 operations as the oracle -> bit-exact
+    from crow_nest_amd.kernels import launch_v
+    h1 = g.standard_normal((40, 1024)).astype(np.float32)
+    h2 = torch.empty((40, 512), dtype=torch.float32, device="cuda")
+    h1d = _dev(h1)
+    launch_v(eng.k.f("silu_mul_combo"), (40 * 512 + 255) // 256, 1, 1, 256, [h1d.data_ptr(), h2.data_ptr(), eng.p.i32(40 * 512)])
+    assert np.allclose(h2.cpu().numpy(), orc.silu_mul_combo(h1, 512), rtol=1e-6, atol=1e-30)
+    eo = g.standard_normal((5 * 8, 2048)).astype(np.float32)
+    rw = g.random((5, 8)).astype(np.float32)
+    y0 = g.standard_normal((5, 2048)).astype(np.float32)
+    y = _dev(y0.copy())
+    eod, rwd = _dev(eo), _dev(rw)
+    launch_v(eng.k.f("acc_combo"), 2048 // 256, 5, 1, 256, [eod.data_ptr(), rwd.data_ptr(), y.data_ptr()])
+    want = orc.acc_combo(eo, rw, 5, 8, 2048, y0)
+    assert np.array_equal(y.cpu().numpy().view(np.uint32), want.view(np.uint32))
+    eng.check()
+
+
+@pytest.mark.parametrize("t", [1, 4])
+def test_moe_layer_both_launch_sequences(eng, t):
+    from crow_nest_amd.engine import MoeW, expert_table
+    from crow_nest_amd.weights import load_expert_slabs
+    E, H, I, K = 256, 2048, 512, 8
+    gu = random_nvfp4(41, E * 2 * I, H, scale_lo=0x30, scale_hi=0x48, p7f=0)
+    dn = random_nvfp4(42, E * H, I, scale_lo=0x30, scale_hi=0x48, p7f=0)
+    gs_gu, gs_dn = 2.0e-3, 3.0e-3
+    s_gu, s_dn = load_expert_slabs(gu, E, 2 * I, H, gs_gu), load_expert_slabs(dn, E, H, I, gs_dn)
+    moe = MoeW(s_gu, s_dn, expert_table(s_gu, s_dn))
+    x = (normal_f32(5, t, t * H) * np.float32(0.1)).reshape(t, H)
+    logits = normal_f32(6, t, t * E).reshape(t, E)
+    ids_ref, w_ref, y_ref = orc.moe_layer(gu, gs_gu, dn, gs_dn, E, H, I, x, logits, K, threads=8)
+    for fused in (False, True):
+        ids, wts, y = eng.moe_run(moe, _dev(x), _dev(logits), fused=fused)
+        assert np.array_equal(ids.cpu().numpy(), ids_ref)
+        assert np.allclose(wts.cpu().numpy(), w_ref, rtol=2e-6, atol=0)
+        assert rel_err(y.cpu().numpy(), y_ref) <= TOL, fused
+    eng.check()
+
+
+# ---------------------------------------------------------------- BASELINE config 0 at full size
+
+def test_config0_full_size(eng):
+    rows, cols = 17408, 5120
+    w, gs = quantized_normal(0, 0, rows, cols)
+    x = normal_f32(0, 1, cols)
+    f = _load(w, rows, cols, gs)
+    y = eng.dense_proj(f, 1, _dev(x)).cpu().numpy()[0]
+    eng.check()
+    ref = orc.gemv(w, rows, cols, gs, x, threads=8)[0]
+    assert rel_err(y, ref) <= TOL
+    sub = slice(0, 512)
+    assert gamma_ratio(y[sub], w[:512 * cols // 64 * 36], 512, cols, gs, x) <= 1.0
+    # dequantised weights bit-exact on a slab of the full tensor
+    from crow_nest_amd.weights import dequant
+    d = dequant(f)[:256].cpu().numpy().reshape(-1)
+    assert np.array_equal(d.view(np.uint32), orc.dequant(w[:256 * cols // 64 * 36], gs).view(np.uint32))

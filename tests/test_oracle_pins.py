@@ -377,10 +377,17 @@ def test_argmax_rule():
     for n in (1, 5, 1023, 1024, 1025, 151936):
         l = g.standard_normal(n).astype(np.float32)
         assert orc.argmax_ref(l) == int(np.argmax(l))
-    # ties: the reference keeps the smallest (i mod 1024), then the smallest i
+    # ties: the halving tree (strides 512 .. 1, left slot kept) prefers even slots in its last round,
+    # then slots with bit 1 clear, ...: smallest bit-reversed (i mod 1024), then smallest i.
     l = np.zeros(4096, np.float32)
-    l[[1030, 7, 2055]] = 5.0  # i mod 1024 = 6, 7, 7
+    l[[1030, 7, 2055]] = 5.0  # slots 6, 7, 7: 6 is even
     assert orc.argmax_ref(l) == 1030
+    l = np.zeros(5, np.float32)
+    l[[2, 4]] = 5.0  # by hand: stride 4 moves slot 4 into slot 0, stride 2 then keeps slot 0 -> index 4
+    assert orc.argmax_ref(l) == 4
+    l = np.zeros(2048, np.float32)
+    l[[1, 1024 + 512, 512]] = 1.0  # slots 1, 512, 512: stride 512 pairs slot 0 with 512 -> slot 0 holds 512 (smallest i of the two)
+    assert orc.argmax_ref(l) == 512
     l = np.full(3000, -3.2e38, np.float32)  # everything below the start value: index 0
     assert orc.argmax_ref(l) == 0
 
