@@ -27,7 +27,8 @@ const FnEntry g_table[] = {
     CROW_FN(gemv_fp4_ptrb, 8),     CROW_FN(moe_gate_up_silu, 8),    CROW_FN(moe_down_combine, 7),
     CROW_FN(router_top10, 10),     CROW_FN(silu_mul_combo, 3),      CROW_FN(acc_combo, 3),
     CROW_FN(argmax_k, 3),          CROW_FN(dequant_fp4_flat, 4),    CROW_FN(repack_nvfp4, 4),
-    CROW_FN(unpack_nvfp4, 4),      CROW_FN(dequant_nvfp4_tiled, 5),
+    CROW_FN(unpack_nvfp4, 4),      CROW_FN(dequant_nvfp4_tiled, 5), CROW_FN(gemm_nvfp4_bf16, 7),
+    CROW_FN(gemm_nvfp4_bf16_m64, 7), CROW_FN(gemm_nvfp4_bf16_m32, 7),
 };
 const int g_table_n = (int)(sizeof(g_table) / sizeof(g_table[0]));
 
@@ -210,23 +211,27 @@ int crow_hip_launch_dims(const char* name, uint32_t rows, uint32_t k_dim, uint32
         const bool two = strstr(name, "_gu") != nullptr || strncmp(name, "moe_gate_up", 11) == 0;
         uint32_t tiles = two && !strncmp(name, "moe_", 4) ? rt : rt;  // rows = output rows for every kernel
         const uint32_t gz = moe ? z : (tokens ? (z + 3) / 4 : 1);
-        long target = env_long("CROW_GEMV_TARGET_WAVES", 20L * g.cus);
-        long max_w = env_long("CROW_GEMV_MAX_W", 1);
-        long force_s = env_long("CROW_GEMV_S", 0), force_w = env_long("CROW_GEMV_W", 0);
-        // routed / batched launches multiply the tile count by gz, but the split must not depend on z
-        // for the dense kernels (bit-identity across M); routed kernels have their own fixed z per model.
-        long per_tile = (target + (long)tiles * (moe ? gz : 1) - 1) / ((long)tiles * (moe ? gz : 1));
-        if (per_tile < 1) per_tile = 1;
-        if (per_tile > (long)panels) per_tile = panels;
-        long w = per_tile < max_w ? per_tile : max_w;
-        long s = (per_tile + w - 1) / w;
-        if (force_w > 0) w = force_w;
+        // A tile's panels are dealt to S blocks of W waves.  Measured on MI355X (17408 x 5120,
+        // 5120 x 17408, 151936 x 5120): a wave that owns ONE panel, with every wave of the launch
+        // resident at once, streams best (all loads are in flight from the start; a second panel in
+        // the same wave pays the memory latency again); W = 4..8 waves combine in LDS, the S
+        // blocks of a tile through the workspace (each costs a round trip, so S stays small).
+        // When there are more (tile, panel) units than resident waves, waves take several panels.
+        const long resident = 32L * g.cus;  // wave slots at <= 64 VGPRs
+        const long all_tiles = (long)tiles * (moe ? gz : 1);
+        long units = all_tiles * (long)panels <= resident ? (long)panels : (2 * resident + all_tiles - 1) / all_tiles;
+        if (units < 1) units = 1;
+        if (units > (long)panels) units = panels;
+        long w = units <= 8 ? units : (panels > 32 ? 8 : 4);
+        long s = (units + w - 1) / w;
+        const long force_s = env_long("CROW_GEMV_S", 0), force_w = env_long("CROW_GEMV_W", 0);
         if (force_s > 0) s = force_s;
+        if (force_w > 0) w = force_w;
         if (w > 16) w = 16;
-        const int nrm = (two ? 2 : 1) * 4;
-        while (w > 1 && (w - 1) * nrm * 64 > CROW_RED_FLOATS) w--;
-        if (s * w > (long)panels) s = (panels + w - 1) / w;
+        if (w < 1) w = 1;
         if (s < 1) s = 1;
+        if (s * w > (long)panels) s = (panels + w - 1) / w;
+        const int nrm = (two ? 2 : 1) * 4;
         out->gx = (uint32_t)s;
         out->gy = tiles;
         out->gz = gz;
@@ -234,6 +239,12 @@ int crow_hip_launch_dims(const char* name, uint32_t rows, uint32_t k_dim, uint32
         const unsigned long long need = (unsigned long long)tiles * gz * s * nrm * 64;
         if (s > 1 && (need > PARTIAL_FLOATS || (unsigned long long)tiles * gz > COUNTER_SLOTS)) return CROW_ERR_WORKSPACE;
         if (strcmp(name, "gemv_nvfp4_w_argmax") == 0 && tiles > AM_SLOTS) return CROW_ERR_WORKSPACE;
+        return CROW_OK;
+    }
+    if (strncmp(name, "gemm_nvfp4_bf16", 15) == 0) {  // z = M token rows
+        if (k_dim == 0 || k_dim % CROW_BLOCK_VALUES != 0) return CROW_ERR_SHAPE;
+        const uint32_t mt = strcmp(name, "gemm_nvfp4_bf16_m32") == 0 ? 32 : (strcmp(name, "gemm_nvfp4_bf16_m64") == 0 ? 64 : 128);
+        *out = crow_dims{(rt + 3) / 4, (z + mt - 1) / mt, 1, 256};
         return CROW_OK;
     }
     if (strcmp(name, "moe_down_combine") == 0) {
@@ -322,6 +333,29 @@ int crow_hip_event_elapsed_ms(void* start, void* stop, float* ms) {
     return hip_rc(hipEventElapsedTime(ms, (hipEvent_t)start, (hipEvent_t)stop));
 }
 int crow_hip_event_destroy(void* ev) { return ev ? hip_rc(hipEventDestroy((hipEvent_t)ev)) : CROW_OK; }
+
+int crow_hip_time_launches(crow_fn_t f, uint32_t gx, uint32_t gy, uint32_t gz, uint32_t bx, const uint64_t* vals, uint32_t n_vals,
+                           uint32_t n_sets, uint32_t iters, float* us_per_launch) {
+    if (!g.ready) return CROW_ERR_NOT_INITIALIZED;
+    const FnEntry* e = (const FnEntry*)(void*)f;
+    if (e < g_table || e >= g_table + g_table_n) return CROW_ERR_KERNEL_MISSING;
+    if (!vals || !us_per_launch || n_sets == 0 || iters == 0) return CROW_ERR_BAD_ARGUMENT;
+    hipEvent_t a, b;
+    hipError_t rc;
+    if ((rc = hipEventCreate(&a)) != hipSuccess) return (int)rc;
+    if ((rc = hipEventCreate(&b)) != hipSuccess) return (int)rc;
+    int out = hip_rc(hipEventRecord(a, g.stream));
+    for (uint32_t i = 0; i < iters && out == CROW_OK; i++)
+        out = launch_entry(e, dim3(gx, gy, gz), dim3(bx), vals + (size_t)(i % n_sets) * n_vals, n_vals, g.stream);
+    if (out == CROW_OK) out = hip_rc(hipEventRecord(b, g.stream));
+    if (out == CROW_OK) out = hip_rc(hipEventSynchronize(b));
+    float ms = 0.0f;
+    if (out == CROW_OK) out = hip_rc(hipEventElapsedTime(&ms, a, b));
+    (void)hipEventDestroy(a);
+    (void)hipEventDestroy(b);
+    *us_per_launch = ms * 1000.0f / (float)iters;
+    return out;
+}
 
 size_t crow_hip_container_bytes(uint32_t rows, uint32_t cols) { return crow_container_bytes(rows, cols); }
 size_t crow_hip_tiled_bytes(uint32_t rows, uint32_t cols) { return crow_tiled_bytes(rows, cols); }

@@ -13,18 +13,22 @@
 //   for each 16-value sub-block, in column order:
 //       part = fma(w15, x15, ... fma(w1, x1, w0 * x0))        (w exact, 16 fused steps)
 //       acc  = fma(part, ue4m3(scale), acc)
-//   a row split over several waves / workgroups: the per-slice `acc` values are added in slice
-//   order (slice 0 first), each slice covering whole 256-column panels p = slice, slice + S, ...
+//   a row split over S blocks of W waves: unit u = slice * W + wave owns panels u, u + S W, ...;
+//   a block adds its waves' `acc` values in wave order, then the blocks' sums are added in
+//   slice order (slice 0 first)
 //   y = acc * gs                                               (gs last, as kernels_p2.rs:367)
 // The order depends only on (K, slices), never on M: row m of an M-row launch is bit-identical to
 // a one-row launch with the same slicing (the verify contract of kernels_p2.rs:391-396).
 //
-// Launch geometry: grid (S, row_tiles, Z), block 64 * W.  blockIdx.x = column slice, blockIdx.y =
-// row tile, blockIdx.z = token group / expert combo.  The W waves of a block and the S blocks of
-// a row tile split the panels round-robin: unit u = slice * W + wave takes panels u, u + S W, ...
-// Waves combine through LDS, blocks through the library workspace: every block stores its
-// partial sums, bumps the tile's arrival counter, and the block that arrives last adds all
-// partials in slice order and writes y (deterministic whatever the arrival order).
+// Launch geometry: grid (S, row_tiles, Z), block 64 * W.  blockIdx.y = row tile, blockIdx.x = column
+// slice, blockIdx.z = token group / expert combo.  The W waves of a block and the S blocks of a row
+// tile deal the tile's 256-column panels round-robin: unit u = slice * W + wave takes panels u,
+// u + S W, ...  (the split is chosen so that a wave usually owns one or two panels and all of the
+// launch's waves are resident at once: every load of the launch is then in flight from the start).
+// Waves combine through LDS in wave order; blocks combine through the library workspace: every
+// block stores its partial sums, bumps the tile's arrival counter, and the block that arrives
+// last adds all partials in slice order and writes y - deterministic whatever the arrival order.
+// With S = 1 the workspace is not touched.
 #pragma once
 #include "device_common.h"
 
@@ -42,9 +46,6 @@ struct GemvArgs {
     int k_dim, rows, m;  // m <= MMAX of the instantiation
     int* argmax_out;     // not null: also write the greedy argmax of y row 0 (fused lm_head head)
 };
-
-// LDS floats for the wave -> wave 0 hand-over: (waves - 1) * NR * M * 64 must fit
-#define CROW_RED_FLOATS 4096
 
 // 16 consecutive activation values of row m, wave-uniform (scalar loads)
 template <bool XBF16>
@@ -214,8 +215,52 @@ struct PanelFull<NR, M, XBF16, 2 * CROW_STEPS> {
                                                XChunk<XBF16> (&)[M], float (&)[NR][M]) {}
 };
 
+template <int NR>
+__device__ __forceinline__ void load_tile(const unsigned char* const (&w)[2], int rt, int panels, int p, int lane,
+                                          uint4 (&sc)[NR], uint4 (&cd)[NR][CROW_STEPS]) {
+#pragma unroll
+    for (int r = 0; r < NR; r++) {
+        const uint4* t = (const uint4*)(w[r] + ((size_t)rt * panels + p) * CROW_TILE_BYTES) + lane;
+        sc[r] = t[0];
+#pragma unroll
+        for (int s = 0; s < CROW_STEPS; s++) cd[r][s] = t[64 * (s + 1)];
+    }
+}
+
+template <int NR, int M, bool XBF16>
+__device__ __forceinline__ void panel_compute(const uint4 (&sc)[NR], const uint4 (&cd)[NR][CROW_STEPS], int p, int k_dim,
+                                              const void* x, size_t x_stride, int m_rows, float (&acc)[NR][M]) {
+    const int left = (k_dim - p * CROW_PANEL_COLS) / CROW_STEP_COLS;
+#ifdef CROW_DEBUG_X0
+    p = 0;  // experiment only: every panel reads the same 1 KB of x
+#endif
+    if (left >= CROW_STEPS) {
+        XChunk<XBF16> first[M];
+#pragma unroll
+        for (int m = 0; m < M; m++)
+            if (m < m_rows) first[m].load(x, (size_t)m * x_stride + (size_t)p * CROW_PANEL_COLS);
+        PanelFull<NR, M, XBF16, 0>::run(sc, cd, x, (size_t)p * CROW_PANEL_COLS, x_stride, m_rows, first, acc);
+    } else {
+        Steps<NR, M, XBF16, 0>::run(sc, cd, x, (size_t)p * CROW_PANEL_COLS, x_stride, m_rows, left, acc);
+    }
+}
+
+// Ordering point of the cross-block hand-over.  Every access to the shared partials and counters
+// is a device-scope atomic (store / load / add carry the device-coherence bits, so each one is
+// performed at the level all compute dies share); what is left to guarantee is program order
+// between them, which a wait for this wave's outstanding memory operations gives: the partial
+// stores are acknowledged before the arrival counter is bumped, and the counter's value is back
+// before any partial is read.  No cache-wide write-back or invalidate is issued: device-scope
+// fences were measured at tens of microseconds per launch here because every block pays one.
+__device__ __forceinline__ void device_order() {
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+    __builtin_amdgcn_s_waitcnt(0);
+    asm volatile("" ::: "memory");
+}
+
 // acc[r][m] = sum over panels p = p0, p0 + stride, ... of the 64-row tile `rt` of tensor r against
-// activation row m: the per-lane (= per-row) partial dot product of one wave.
+// activation row m: the per-lane (= per-row) partial dot product of one wave.  One register buffer
+// per wave; loads and arithmetic of different waves overlap through occupancy (about 52 VGPRs).
 template <int NR, int M, bool XBF16>
 __device__ __forceinline__ void tile_accumulate(const unsigned char* const (&w)[2], int rt, int panels, int p0, int stride,
                                                 int k_dim, const void* x, size_t x_stride, int m_rows, float (&acc)[NR][M]) {
@@ -226,49 +271,53 @@ __device__ __forceinline__ void tile_accumulate(const unsigned char* const (&w)[
         for (int m = 0; m < M; m++) acc[r][m] = 0.0f;
     for (int p = p0; p < panels; p += stride) {
         uint4 sc[NR], cd[NR][CROW_STEPS];
-#pragma unroll
+        load_tile<NR>(w, rt, panels, p, lane, sc, cd);
+#ifdef CROW_EXP_NOCOMPUTE
         for (int r = 0; r < NR; r++) {
-            const uint4* t = (const uint4*)(w[r] + ((size_t)rt * panels + p) * CROW_TILE_BYTES) + lane;
-            sc[r] = t[0];
-#pragma unroll
-            for (int s = 0; s < CROW_STEPS; s++) cd[r][s] = t[64 * (s + 1)];
+            unsigned q = sc[r].x ^ sc[r].y ^ sc[r].z ^ sc[r].w;
+            for (int s = 0; s < CROW_STEPS; s++) q ^= cd[r][s].x ^ cd[r][s].y ^ cd[r][s].z ^ cd[r][s].w;
+            acc[r][0] += __uint_as_float(q & 0x3fffffffu);
         }
-        const int left = (k_dim - p * CROW_PANEL_COLS) / CROW_STEP_COLS;
-        if (left >= CROW_STEPS) {
-            XChunk<XBF16> first[M];
-#pragma unroll
-            for (int m = 0; m < M; m++)
-                if (m < m_rows) first[m].load(x, (size_t)m * x_stride + (size_t)p * CROW_PANEL_COLS);
-            PanelFull<NR, M, XBF16, 0>::run(sc, cd, x, (size_t)p * CROW_PANEL_COLS, x_stride, m_rows, first, acc);
-        } else Steps<NR, M, XBF16, 0>::run(sc, cd, x, (size_t)p * CROW_PANEL_COLS, x_stride, m_rows, left, acc);
+#else
+        panel_compute<NR, M, XBF16>(sc, cd, p, k_dim, x, x_stride, m_rows, acc);
+#endif
     }
 }
 
-// The body every GEMV entry point runs.  `z` selects nothing here: the caller has already
-// offset the pointers in `a` for its token group / combo; `tile_id` indexes the workspace.
-template <int NR, int M, bool XBF16, int EPI>
-__device__ __forceinline__ void gemv_body(const GemvArgs& a, unsigned tile_id, float* red) {
+typedef __attribute__((address_space(1))) float* gfloat_p;
+typedef __attribute__((address_space(1))) unsigned* guint_p;
+typedef __attribute__((address_space(1))) int* gint_p;
+
+// The body every GEMV entry point runs.  The caller has already offset the pointers in `a` for
+// its token group / combo `z`, which only indexes the workspace here.  `red` is the block's LDS
+// hand-over buffer of (W - 1) * NR * M * 64 floats (RED_FLOATS of them are there).
+template <int NR, int M, bool XBF16, int EPI, int RED_FLOATS>
+__device__ __forceinline__ void gemv_body(const GemvArgs& a, unsigned z, float* red) {
     const int lane = lane_id();
     const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6)), waves = (int)(blockDim.x >> 6);  // wave-uniform on purpose
     const int slice = (int)blockIdx.x, slices = (int)gridDim.x;
     const int rt = (int)blockIdx.y;
+    const int row_tiles = (int)gridDim.y;
     const int panels = (a.k_dim + CROW_PANEL_COLS - 1) / CROW_PANEL_COLS;
     const int m_rows = a.m < M ? a.m : M;
+    const unsigned tile_id = z * (unsigned)row_tiles + (unsigned)rt;
+    const Workspace ws = g_ws;  // read early: its latency hides behind the weight loads
 
     float acc[NR][M];
     tile_accumulate<NR, M, XBF16>(a.w, rt, panels, slice * waves + wave, slices * waves, a.k_dim, a.x, a.x_stride, m_rows, acc);
 
     // waves of the block -> wave 0, in wave order
     if (waves > 1) {
-        if ((waves - 1) * NR * M * 64 > CROW_RED_FLOATS) {  // uniform: the launch does not fit this kernel
-            if (threadIdx.x == 0) atomicOr(g_ws.status, STATUS_BAD_SHAPE);
+        if ((waves - 1) * NR * M * 64 > RED_FLOATS) {  // uniform: the launch does not fit this kernel
+            if (threadIdx.x == 0) atomicOr(ws.status, STATUS_BAD_SHAPE);
             return;
         }
         if (wave > 0) {
 #pragma unroll
             for (int r = 0; r < NR; r++)
 #pragma unroll
-                for (int m = 0; m < M; m++) red[((wave - 1) * NR * M + r * M + m) * 64 + lane] = acc[r][m];
+                for (int m = 0; m < M; m++)
+                    if (m < m_rows) red[((wave - 1) * NR * M + r * M + m) * 64 + lane] = acc[r][m];
         }
         __syncthreads();
         if (wave > 0) return;
@@ -276,44 +325,62 @@ __device__ __forceinline__ void gemv_body(const GemvArgs& a, unsigned tile_id, f
 #pragma unroll
             for (int r = 0; r < NR; r++)
 #pragma unroll
-                for (int m = 0; m < M; m++) acc[r][m] += red[((w - 1) * NR * M + r * M + m) * 64 + lane];
+                for (int m = 0; m < M; m++)
+                    if (m < m_rows) acc[r][m] += red[((w - 1) * NR * M + r * M + m) * 64 + lane];
         }
     }
 
-    // blocks of the row tile -> the last one to arrive, in slice order
+    // slices of the row tile -> the last one to arrive, in slice order
+#ifdef CROW_EXP_NOREDUCE
+    if (false) {
+#else
     if (slices > 1) {
-        const Workspace ws = g_ws;
+#endif
         const size_t need = ((size_t)tile_id + 1) * slices * (NR * M) * 64;
         if (need > ws.partial_floats || tile_id >= ws.counter_slots) {
             if (lane == 0) atomicOr(ws.status, STATUS_WORKSPACE_TOO_SMALL);
             return;
         }
-        float* base = ws.partials + (size_t)tile_id * slices * (NR * M) * 64;
-        float* mine = base + (size_t)slice * (NR * M) * 64;
+        gfloat_p base = (gfloat_p)ws.partials + (size_t)tile_id * slices * (NR * M) * 64;
+        gfloat_p mine = base + (size_t)slice * (NR * M) * 64;
+        guint_p counter = (guint_p)ws.counters + tile_id;
 #pragma unroll
         for (int r = 0; r < NR; r++)
 #pragma unroll
             for (int m = 0; m < M; m++)
                 if (m < m_rows) __hip_atomic_store(mine + (r * M + m) * 64 + lane, acc[r][m], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "agent");
+        device_order();
         unsigned arrived = 0;
-        if (lane == 0) arrived = __hip_atomic_fetch_add(ws.counters + tile_id, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        if (lane == 0) arrived = __hip_atomic_fetch_add(counter, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         arrived = __builtin_amdgcn_readfirstlane(arrived);
         if (arrived != (unsigned)slices - 1) return;
-        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
+        device_order();
 #pragma unroll
         for (int r = 0; r < NR; r++)
 #pragma unroll
             for (int m = 0; m < M; m++) acc[r][m] = 0.0f;
-        for (int s = 0; s < slices; s++) {
-            const float* q = base + (size_t)s * (NR * M) * 64;
+        // up to PB slices' loads in flight at a time, added in slice order
+        constexpr int PB = (NR * M <= 2) ? 16 : 8;
+        for (int s0 = 0; s0 < slices; s0 += PB) {
+            float t[PB][NR * M];
 #pragma unroll
-            for (int r = 0; r < NR; r++)
+            for (int j = 0; j < PB; j++) {
+                gfloat_p q = base + (size_t)(s0 + j) * (NR * M) * 64 + lane;
 #pragma unroll
-                for (int m = 0; m < M; m++)
-                    if (m < m_rows) acc[r][m] += __hip_atomic_load(q + (r * M + m) * 64 + lane, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                for (int i = 0; i < NR * M; i++)
+                    t[j][i] = (s0 + j < slices && (i % M) < m_rows) ? __hip_atomic_load(q + i * 64, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) : 0.0f;
+            }
+#pragma unroll
+            for (int j = 0; j < PB; j++) {
+                if (s0 + j < slices) {
+#pragma unroll
+                    for (int r = 0; r < NR; r++)
+#pragma unroll
+                        for (int m = 0; m < M; m++) acc[r][m] += t[j][r * M + m];
+                }
+            }
         }
-        if (lane == 0) __hip_atomic_store(ws.counters + tile_id, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        if (lane == 0) __hip_atomic_store(counter, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     }
 
     const int row = rt * CROW_TILE_ROWS + lane;
@@ -323,26 +390,28 @@ __device__ __forceinline__ void gemv_body(const GemvArgs& a, unsigned tile_id, f
         const float v = acc[0][0] * a.gs[0][0];
         if (row < a.rows) a.y[row] = v;
         Best b = wave_best(Best{row < a.rows ? v : -3.0e38f, row < a.rows ? row : 0});
-        const Workspace ws = g_ws;
-        const unsigned tiles = gridDim.y;
+        const unsigned tiles = (unsigned)row_tiles;
         if (tiles > ws.am_slots) {
             if (lane == 0) atomicOr(ws.status, STATUS_WORKSPACE_TOO_SMALL);
             return;
         }
+        gfloat_p am_val = (gfloat_p)ws.am_val;
+        gint_p am_idx = (gint_p)ws.am_idx;
+        guint_p am_counter = (guint_p)ws.am_counter;
         unsigned arrived = 0;
         if (lane == 0) {
-            __hip_atomic_store(ws.am_val + rt, b.v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-            __hip_atomic_store(ws.am_idx + rt, b.i, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "agent");
-            arrived = __hip_atomic_fetch_add(ws.am_counter, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            __hip_atomic_store(am_val + rt, b.v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            __hip_atomic_store(am_idx + rt, b.i, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            device_order();
+            arrived = __hip_atomic_fetch_add(am_counter, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         }
         arrived = __builtin_amdgcn_readfirstlane(arrived);
         if (arrived != tiles - 1) return;
-        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
+        device_order();
         Best g{-3.0e38f, 0};
         for (unsigned t = lane; t < tiles; t += 64) {
-            const float tv = __hip_atomic_load(ws.am_val + t, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-            const int ti = __hip_atomic_load(ws.am_idx + t, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            const float tv = __hip_atomic_load(am_val + t, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            const int ti = __hip_atomic_load(am_idx + t, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
             if (better(tv, ti, g.v, g.i)) {
                 g.v = tv;
                 g.i = ti;
@@ -351,7 +420,7 @@ __device__ __forceinline__ void gemv_body(const GemvArgs& a, unsigned tile_id, f
         g = wave_best(g);
         if (lane == 0) {
             a.argmax_out[0] = g.i;
-            __hip_atomic_store(ws.am_counter, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            __hip_atomic_store(am_counter, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         }
         return;
     }

@@ -188,4 +188,13 @@ class Engine:
 
     # ------------------------------------------------------------------ prefill GEMM (M >= 16)
     def gemm(self, w: Fp4, m: int, x: torch.Tensor, y: torch.Tensor | None = None) -> torch.Tensor:
-        raise NotImplementedError("the MFMA GEMM entry is not built yet")
+        """Y[m][rows] = X[m][cols] W^T on the matrix cores (bf16 X, exact bf16 weight tiles, f32 accumulate)."""
+        rows, k = w.rows, w.cols
+        assert x.is_cuda and x.is_contiguous() and x.dtype == torch.bfloat16 and x.numel() == m * k
+        if y is None:
+            y = torch.empty((m, rows), dtype=torch.float32, device=self.dev)
+        name = "gemm_nvfp4_bf16_m32" if m <= 32 else ("gemm_nvfp4_bf16_m64" if m <= 64 else "gemm_nvfp4_bf16")
+        gx, gy, gz, bx = launch_dims(name, rows, k, m)
+        p = self.p
+        launch_v(self.k.f(name), gx, gy, gz, bx, [w.w_ptr, x.data_ptr(), w.gs_ptr, y.data_ptr(), p.i32(k), p.i32(rows), p.i32(m)])
+        return y

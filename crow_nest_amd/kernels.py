@@ -115,6 +115,17 @@ def launch_dims(name: str, rows: int, k_dim: int, z: int = 1) -> tuple[int, int,
     return d.gx, d.gy, d.gz, d.bx
 
 
+def time_launches(f: int, gx: int, gy: int, gz: int, bx: int, arg_sets, iters: int) -> float:
+    """Mean microseconds per launch over `iters` back-to-back launches that rotate over `arg_sets`
+    (the loop runs inside the library, between two HIP events on the launch stream)."""
+    n = len(arg_sets[0])
+    flat = [int(v) for s in arg_sets for v in s]
+    arr = (C.c_uint64 * len(flat))(*flat)
+    us = C.c_float()
+    _l.check(_l.lib().crow_hip_time_launches(f, gx, gy, gz, bx, arr, n, len(arg_sets), iters, C.byref(us)), "crow_hip_time_launches")
+    return float(us.value)
+
+
 class Event:
     """A HIP event on the library's current stream (the stream every launch_v goes to)."""
 

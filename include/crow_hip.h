@@ -92,6 +92,11 @@ int crow_hip_event_create(void** out);
 int crow_hip_event_record(void* ev);                              /* on the current stream */
 int crow_hip_event_elapsed_ms(void* start, void* stop, float* ms); /* waits for `stop` */
 int crow_hip_event_destroy(void* ev);
+/* `iters` back-to-back launches of `f` on the current stream between two events, launch i taking
+ * the argument set vals[(i % n_sets) * n_vals ...] (rotating weight copies keep the working set
+ * larger than the 256 MB memory-side cache).  Returns the mean microseconds per launch. */
+int crow_hip_time_launches(crow_fn_t f, uint32_t gx, uint32_t gy, uint32_t gz, uint32_t bx, const uint64_t* vals,
+                           uint32_t n_vals, uint32_t n_sets, uint32_t iters, float* us_per_launch);
 
 /* ---- load-time repack (the one call the reference does not have) ---- */
 size_t crow_hip_container_bytes(uint32_t rows, uint32_t cols);

@@ -12,14 +12,23 @@ from refgen import normal_f32
 TOL = 1e-3  # north star: GEMV outputs within max relative error 1e-3 of the CPU path
 
 
+FLOOR = 1e-2  # outputs below 1 % of their row's rms are compared absolutely (1e-5 rms), see rel_err
+
+
 def rel_err(y: np.ndarray, ref: np.ndarray) -> float:
-    """max_i |y_i - ref_i| / max(|ref_i|, 1e-3 * rms(ref)) per output row, worst row."""
+    """max_i |y_i - ref_i| / max(|ref_i|, FLOOR * rms(ref)) per output row, worst row.
+
+    A dot product of K ~ 5000 terms summed in f32 carries an absolute error of about 1e-6 of the
+    row's rms whatever the order (the CPU path against f64 shows the same); an output that happens
+    to cancel to almost nothing therefore has no meaningful RELATIVE error, and is held to
+    TOL * FLOOR * rms instead.  Every GEMV test additionally holds the reference's own acceptance
+    bound gamma(K/16 + 10) * sum|w x| against an f64 evaluation (gamma_ratio), which has no floor."""
     y = np.asarray(y, np.float64).reshape(ref.shape)
     r = np.asarray(ref, np.float64)
     if r.ndim == 1:
         r, y = r[None], y[None]
     rms = np.sqrt((r * r).mean(axis=1, keepdims=True))
-    den = np.maximum(np.abs(r), 1e-3 * np.maximum(rms, 1e-30))
+    den = np.maximum(np.abs(r), FLOOR * np.maximum(rms, 1e-30))
     return float(np.max(np.abs(y - r) / den))
 
 

@@ -1,9 +1,9 @@
 """GPU parity: the HIP path (through the C ABI, via the host mirror) against the CPU oracle.
 
 Bars: dequantised weights bit-exact; integer / index results bit-exact; GEMV outputs within
-max relative error 1e-3 of the CPU path (TOL below; the denominator floors at 1e-3 of the row's
-rms so that an output that cancels to ~0 does not divide by nothing), and additionally inside the
-reference's own fp32 bound gamma(K/16 + 10) * sum|w x| against an f64 evaluation.
+max relative error 1e-3 of the CPU path (TOL; the denominator floors at 1 % of the row's rms so that
+an output that cancels to ~0 does not divide by nothing - see gpu_common.rel_err), and additionally
+inside the reference's own fp32 bound gamma(K/16 + 10) * sum|w x| against an f64 evaluation.
 """
 import numpy as np
 import pytest
@@ -291,3 +291,39 @@ def test_config0_full_size(eng):
     from crow_nest_amd.weights import dequant
     d = dequant(f)[:256].cpu().numpy().reshape(-1)
     assert np.array_equal(d.view(np.uint32), orc.dequant(w[:256 * cols // 64 * 36], gs).view(np.uint32))
+
+
+# ---------------------------------------------------------------- batched GEMM on the matrix cores (config 4)
+
+@pytest.mark.parametrize("m,rows,cols", [(16, 320, 1024), (17, 100, 320), (33, 256, 512), (128, 512, 2048), (200, 192, 5120)])
+def test_gemm_bf16_against_the_cpu_path(eng, m, rows, cols):
+    """Weights decode to exact bf16, X is bf16, products are exact in f32: only the summation order
+    differs from the CPU path (which gets the exactly widened X)."""
+    print(f"case m={m} rows={rows} cols={cols}", flush=True)
+    w = random_nvfp4(m * 7 + rows, rows, cols)
+    gs = 6.0e-4
+    f = _load(w, rows, cols, gs)
+    xb, xw = _bf16_dev(normal_f32(7, m, m * cols))
+    y = eng.gemm(f, m, xb.reshape(m, cols).contiguous()).cpu().numpy()
+    eng.check()
+    ref = orc.gemv(w, rows, cols, gs, xw.reshape(m, cols), threads=8)
+    assert rel_err(y, ref) <= TOL
+    assert gamma_ratio(y[:4], w, rows, cols, gs, xw.reshape(m, cols)[:4]) <= 1.0
+
+
+def test_gemm_full_size_sampled_rows(eng):
+    """BASELINE config 4 at M = 512 on the full [17408, 5120] tensor; the CPU path checks 768 sampled rows."""
+    rows, cols, m = 17408, 5120, 512
+    w, gs = quantized_normal(0, 0, rows, cols)
+    f = _load(w, rows, cols, gs)
+    xb, xw = _bf16_dev(normal_f32(0, 40, m * cols))
+    y = eng.gemm(f, m, xb.reshape(m, cols).contiguous()).cpu().numpy()
+    eng.check()
+    rb = cols // 64 * 36
+    for r0 in (0, 8704 - 128, 17408 - 256):
+        ref = orc.gemv(w[r0 * rb:(r0 + 256) * rb], 256, cols, gs, xw.reshape(m, cols), threads=8)
+        assert rel_err(y[:, r0:r0 + 256], ref) <= TOL, r0
+    # linearity, a size-independent property: rows of X scaled by powers of two scale Y exactly
+    x2 = (xb.reshape(m, cols).float() * 4.0).to(torch.bfloat16).contiguous()
+    y2 = eng.gemm(f, m, x2).cpu().numpy()
+    assert np.array_equal(y2.view(np.uint32), (y * np.float32(4.0)).view(np.uint32))
