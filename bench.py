@@ -1,0 +1,302 @@
+#!/usr/bin/env python3
+"""Benchmark of the NVFP4 weight x activation hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-others] [--no-cpu]
+
+One "step" is one pass of BASELINE config 1 at batch 1 (M = 1): the fused gate/up + SiLU GEMV
+(W_gate, W_up [17408, 5120] NVFP4, X bf16) followed by the down projection (W_down [5120, 17408]
+on the f32 H) - the dense FFN of one decode token at the 27B shape.  Weights are N(0, 0.02^2),
+seed 0, through the ceil encoder; they are resident in HBM before the timed region and every step
+reads a different copy (10 copies, 1.5 GB) so that the 256 MB memory-side cache cannot serve them.
+`value` = algorithmic bytes of the step / wall time per step.  The JSON line also carries the
+roofline of the dominant kernel (HIP events around back-to-back launches of that kernel alone on
+the launch stream), the CPU baseline (the C restatement of the reference's CPU NVFP4 path on this
+host's cores: a port, not the Rust binary), and microseconds per call for the other BASELINE shapes.
+"""
+from __future__ import annotations
+
+import argparse
+import ctypes as C
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+for p in (ROOT, os.path.join(ROOT, "tests")):
+    if p not in sys.path:
+        sys.path.insert(0, p)
+
+PEAK_HBM_GBS = 8000.0
+# HBM bytes per launch of the dominant kernel, measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE and scaled by
+# a 256 MiB copy kernel in the same run (profiles/gemv_nvfp4_gum_bf16__config1_m1.md): 101,337,112 read + 818,176 written
+TRAFFIC_GATE_UP_M1 = 102155288
+N, K = 17408, 5120
+W_BYTES = N * K // 64 * 36  # 50,135,040: container encoding, 4.5 bits per weight
+
+
+def alg_bytes_gate_up(m: int, x_bytes: int = 2) -> int:
+    return 2 * W_BYTES + m * K * x_bytes + m * N * 4 + 8
+
+
+def alg_bytes_down(m: int) -> int:
+    return W_BYTES + m * N * 4 + m * K * 4 + 4
+
+
+class Launch:
+    """A prepared launch: handle, dims and one ctypes argument array per rotating weight copy."""
+
+    def __init__(self, eng, name, rows, k, z, arg_sets):
+        from crow_nest_amd.kernels import launch_dims
+        self.f = eng.k.f(name)
+        self.dims = launch_dims(name, rows, k, z)
+        self.sets = [(C.c_uint64 * len(a))(*[int(v) for v in a]) for a in arg_sets]
+        self.raw = arg_sets
+        self.n = len(arg_sets[0])
+
+    def go(self, lib, i):
+        rc = lib.crow_hip_launch(self.f, *self.dims, self.sets[i % len(self.sets)], self.n, None)
+        if rc != 0:
+            raise RuntimeError(f"crow_hip_launch failed: {rc}")
+
+    def us(self, iters=200, reps=3):
+        from crow_nest_amd.kernels import time_launches
+        time_launches(self.f, *self.dims, self.raw, 20)
+        return min(time_launches(self.f, *self.dims, self.raw, iters) for _ in range(reps))
+
+
+def main() -> int:
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=400)
+    ap.add_argument("--warmup", type=int, default=40)
+    ap.add_argument("--no-others", action="store_true")
+    ap.add_argument("--no-cpu", action="store_true")
+    ap.add_argument("--copy-calibration", action="store_true",
+                    help="also run three device copies of 256 MiB (a plain copy kernel of known size) so that a rocprofv3 --pmc "
+                         "FETCH_SIZE / WRITE_SIZE run of this command holds its own scale")
+    a = ap.parse_args()
+    if a.gpus != 1:
+        print(f"bench.py: this build runs on ONE GPU (every box here has one); --gpus {a.gpus} is not supported. "
+              "DESIGN.md says how the path would shard.", file=sys.stderr)
+        return 2
+
+    import numpy as np
+    import torch
+
+    from crow_nest_amd import lib as L
+    from crow_nest_amd.engine import Engine
+    from crow_nest_amd.kernels import KernelGeo, status
+    from crow_nest_amd.weights import Nvfp4Matrix, load_fp4, tiled_bytes
+    from oracle import oracle as orc  # only for the synthetic inputs' encoder and the cpu_baseline leg
+    from refgen import normal_f32
+
+    eng = Engine(KernelGeo(experts=256, topk=8, hidden=2048, inter=512))
+    lib = L.lib()
+    dev = torch.device("cuda", 0)
+    name_buf = C.create_string_buffer(256)
+    lib.crow_hip_device_name(name_buf, 256)
+    p = eng.p
+
+    # ---------------- synthetic inputs of config 1 (seed 0)
+    t0 = time.time()
+    host = {}
+    for i, (nm, rows, cols) in enumerate([("gate", N, K), ("up", N, K), ("down", K, N)]):
+        wb, gs = orc.quantize_ceil(normal_f32(0, i, rows * cols, 0.02))
+        host[nm] = (wb, gs, rows, cols)
+    x32 = normal_f32(0, 10, K)
+    xb_bits = orc.f32_to_bf16_bits(x32)
+    xb = torch.from_numpy(xb_bits.view(np.int16)).to(dev).view(torch.bfloat16)
+    base = {nm: load_fp4(Nvfp4Matrix.new(host[nm][0], host[nm][2], host[nm][3], host[nm][1])) for nm in host}
+    copies = 10
+    sets = []
+    for c in range(copies):
+        sets.append({nm: (base[nm].w.clone() if c else base[nm].w) for nm in base})
+    h = torch.empty(N, dtype=torch.float32, device=dev)
+    y = torch.empty(K, dtype=torch.float32, device=dev)
+    gen_s = time.time() - t0
+
+    gu = Launch(eng, "gemv_nvfp4_gum_bf16", N, K, 1,
+                [[s["gate"].data_ptr(), s["up"].data_ptr(), xb.data_ptr(), base["gate"].gs_ptr, base["up"].gs_ptr, h.data_ptr(),
+                  p.i32(K), p.i32(N), p.i32(1)] for s in sets])
+    dn = Launch(eng, "gemv_nvfp4_w", K, N, 1,
+                [[s["down"].data_ptr(), h.data_ptr(), base["down"].gs_ptr, y.data_ptr(), p.i32(N), p.i32(K)] for s in sets])
+
+    def step(i):
+        gu.go(lib, i)
+        dn.go(lib, i)
+
+    if a.copy_calibration:
+        src = torch.ones(256 << 20, dtype=torch.uint8, device=dev)
+        dst = torch.empty_like(src)
+        for _ in range(3):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        del src, dst
+    for i in range(a.warmup):
+        step(i)
+    torch.cuda.synchronize()
+    t1 = time.perf_counter()
+    for i in range(a.steps):
+        step(i)
+    torch.cuda.synchronize()
+    dt = time.perf_counter() - t1
+    status()
+    ms_per_step = dt * 1e3 / a.steps
+    step_bytes = alg_bytes_gate_up(1) + alg_bytes_down(1)
+    value = step_bytes / (ms_per_step * 1e-3) / 1e9
+
+    # parity of what was just timed, against the CPU path (the checker, outside the timed region)
+    ref_h = orc.silu_mul(orc.gemv(host["gate"][0], N, K, host["gate"][1], orc.bf16_bits_to_f32(xb_bits), threads=8),
+                         orc.gemv(host["up"][0], N, K, host["up"][1], orc.bf16_bits_to_f32(xb_bits), threads=8))[0]
+    from gpu_common import rel_err
+    gu.go(lib, 0)
+    dn.go(lib, 0)
+    torch.cuda.synchronize()
+    parity_h = rel_err(h.cpu().numpy(), ref_h)
+    parity_y = rel_err(y.cpu().numpy(), orc.gemv(host["down"][0], K, N, host["down"][1], ref_h, threads=8)[0])
+
+    # ---------------- roofline of the dominant kernel (gate/up + SiLU), HIP events on the launch stream
+    gu_us = gu.us()
+    dn_us = dn.us()
+    gu_bytes = alg_bytes_gate_up(1)
+    roof = {"bound": "hbm", "kernel": "gemv_nvfp4_gum_bf16", "achieved": round(gu_bytes / gu_us / 1e3, 1), "peak": PEAK_HBM_GBS,
+            "unit": "GB/s", "frac": round(gu_bytes / gu_us / 1e3 / PEAK_HBM_GBS, 4), "traffic": TRAFFIC_GATE_UP_M1,
+            "us_per_launch": round(gu_us, 2), "algorithmic_bytes": gu_bytes, "grid": list(gu.dims)}
+
+    out = {
+        "metric": "NVFP4 GEMV achieved HBM GB/s (% of peak) and us/call at batch 1, 1 MI355X",
+        "value": round(value, 1), "unit": "GB/s", "n_gpus": 1, "steps": a.steps, "warmup": a.warmup,
+        "ms_per_step": round(ms_per_step, 5), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "f32", "data": "synthetic",
+        "config": {"workload": "BASELINE config 1 at M=1: fused gate/up+SiLU GEMV (W_gate,W_up [17408,5120] NVFP4, X bf16) + down "
+                               "projection (W_down [5120,17408] on f32 H), batch 1; 10 rotating weight copies (1.5 GB)",
+                   "algorithmic_bytes_per_step": step_bytes, "pct_of_peak": round(100 * value / PEAK_HBM_GBS, 1),
+                   "us_per_call": {"gate_up_silu": round(gu_us, 2), "down": round(dn_us, 2)},
+                   "parity_max_rel_err": {"h": float(f"{parity_h:.3g}"), "y": float(f"{parity_y:.3g}")},
+                   "device": name_buf.value.decode(), "input_generation_s": round(gen_s, 1)},
+        "roofline": roof,
+    }
+
+    # ---------------- the other BASELINE shapes: us per call (timing only: random codes, valid scale bytes)
+    if not a.no_others:
+        others = {}
+
+        def rnd(nbytes):
+            return torch.randint(0, 64, (nbytes,), dtype=torch.uint8, device=dev)
+
+        gs1 = torch.tensor([1e-3], dtype=torch.float32, device=dev)
+        xf = torch.randn(4, N, device=dev)
+        xk = torch.randn(4, K, device=dev)
+        xkb = xk.to(torch.bfloat16)
+        ybuf = torch.empty(4 * 151936, dtype=torch.float32, device=dev)
+
+        def entry(us, nbytes):
+            return {"us": round(us, 2), "GB/s": round(nbytes / us / 1e3, 1), "pct_peak": round(nbytes / us / 1e3 / 80, 1)}
+
+        # config 0: dense GEMV, f32 x
+        l0 = Launch(eng, "gemv_nvfp4_w", N, K, 1, [[s["gate"].data_ptr(), xk.data_ptr(), gs1.data_ptr(), ybuf.data_ptr(), p.i32(K), p.i32(N)] for s in sets])
+        others["config0_gemv_17408x5120_f32x"] = entry(l0.us(), W_BYTES + K * 4 + N * 4 + 4)
+        # config 1 at verify widths
+        for m in (2, 4):
+            lg = Launch(eng, "gemv_nvfp4_gum_bf16", N, K, 1,
+                        [[s["gate"].data_ptr(), s["up"].data_ptr(), xkb.data_ptr(), gs1.data_ptr(), gs1.data_ptr(), ybuf.data_ptr(), p.i32(K), p.i32(N), p.i32(m)] for s in sets])
+            ld = Launch(eng, "gemv_nvfp4_wm", K, N, 1,
+                        [[s["down"].data_ptr(), xf.data_ptr(), gs1.data_ptr(), ybuf.data_ptr(), p.i32(N), p.i32(K), p.i32(m)] for s in sets])
+            others[f"config1_gate_up_silu_M{m}"] = entry(lg.us(), alg_bytes_gate_up(m))
+            others[f"config1_down_M{m}"] = entry(ld.us(), alg_bytes_down(m))
+        # config 3: lm_head + fused argmax
+        V = 151936
+        vb = tiled_bytes(V, K)
+        heads = [rnd(vb) for _ in range(4)]
+        idx = torch.zeros(1, dtype=torch.int32, device=dev)
+        l3 = Launch(eng, "gemv_nvfp4_w_argmax", V, K, 1, [[hd.data_ptr(), xk.data_ptr(), gs1.data_ptr(), ybuf.data_ptr(), p.i32(K), p.i32(V), idx.data_ptr()] for hd in heads])
+        others["config3_lm_head_151936x5120_argmax"] = entry(l3.us(iters=100), V * K // 64 * 36 + K * 4 + V * 4 + 4)
+        del heads
+        # config 4: batched GEMM on the matrix cores
+        for m in (16, 128, 512):
+            xm = torch.randn(m, K, device=dev).to(torch.bfloat16)
+            ym = torch.empty(m, N, dtype=torch.float32, device=dev)
+            nm = "gemm_nvfp4_bf16_m32" if m <= 32 else ("gemm_nvfp4_bf16_m64" if m <= 64 else "gemm_nvfp4_bf16")
+            l4 = Launch(eng, nm, N, K, m, [[s["gate"].data_ptr(), xm.data_ptr(), gs1.data_ptr(), ym.data_ptr(), p.i32(K), p.i32(N), p.i32(m)] for s in sets])
+            us = l4.us(iters=50)
+            e = entry(us, W_BYTES + m * K * 2 + m * N * 4)
+            e["TFLOP/s"] = round(2.0 * m * N * K / us / 1e6, 1)
+            e["pct_mfma_peak_bf16"] = round(2.0 * m * N * K / us / 1e6 / 2500 * 100, 1)
+            others[f"config4_gemm_M{m}"] = e
+        # config 2: one MoE layer, 256 experts top-8, H 2048, I 512 (router + fused gate|up+SiLU + fused down+combine)
+        from crow_nest_amd.engine import MoeW, expert_table
+        from crow_nest_amd.weights import ExpertSlabs
+        E, H, I = 256, 2048, 512
+        sg, sd = tiled_bytes(2 * I, H), tiled_bytes(H, I)
+        moes = []
+        for _ in range(3):  # 3 x 453 MB of expert slabs
+            g_ = ExpertSlabs(rnd(E * sg), gs1, E, 2 * I, H, sg)
+            d_ = ExpertSlabs(rnd(E * sd), gs1, E, H, I, sd)
+            moes.append(MoeW(g_, d_, expert_table(g_, d_)))
+        from crow_nest_amd.kernels import Event
+        K8 = 8
+        for t in (1, 4):
+            xt = torch.randn(t, H, device=dev) * 0.1
+            lg_ = torch.randn(t, E, device=dev)
+            yt = torch.zeros(t, H, device=dev)
+            ids = torch.empty((t, K8), dtype=torch.int32, device=dev)
+            wts = torch.empty((t, K8), dtype=torch.float32, device=dev)
+            gup = torch.zeros((t, K8), dtype=torch.int64, device=dev)
+            dnp = torch.zeros((t, K8), dtype=torch.int64, device=dev)
+            h2 = torch.empty((t * K8, I), dtype=torch.float32, device=dev)
+            lr = Launch(eng, "router_top10", 1, 64, t, [[lg_.data_ptr(), 0, ids.data_ptr(), wts.data_ptr(), gup.data_ptr(), dnp.data_ptr(),
+                                                          m_.table.data_ptr(), 0, 0, 0] for m_ in moes])
+            lgu = Launch(eng, "moe_gate_up_silu", I, H, t * K8, [[gup.data_ptr(), xt.data_ptr(), gs1.data_ptr(), h2.data_ptr(), p.i32(H), p.i32(K8),
+                                                                  p.i32(H), p.i32(I)]])
+            ldn = Launch(eng, "moe_down_combine", H, I, t, [[dnp.data_ptr(), h2.data_ptr(), gs1.data_ptr(), wts.data_ptr(), yt.data_ptr(), p.i32(I), p.i32(H)]])
+            ldn.dims = (1, (H + 63) // 64, t, 64 * K8)
+
+            def layer(i):
+                lr.go(lib, i)
+                lgu.go(lib, 0)
+                ldn.go(lib, 0)
+            for i in range(10):
+                layer(i)
+            e0, e1 = Event(), Event()
+            e0.record()
+            reps = 200
+            for i in range(reps):
+                layer(i)
+            e1.record()
+            us = e0.elapsed_ms(e1) * 1e3 / reps
+            nbytes = min(t * 8, E) * (E and (2 * I * H // 64 * 36 + H * I // 64 * 36)) + t * H * 8 + t * E * 4  # t*8 distinct experts at most
+            others[f"config2_moe_layer_T{t}"] = entry(us, nbytes)
+            others[f"config2_moe_layer_T{t}"]["launches"] = 3
+        status()
+        out["others"] = others
+
+    # ---------------- CPU baseline: the C port of the reference's CPU path on this host (rank 0, N = 1 only)
+    if not a.no_cpu:
+        threads = max(1, min(os.cpu_count() or 1, 64))
+        units = []
+        g = np.random.default_rng(0)
+        for u in range(8):  # 8 distinct units of 150 MB: larger than any L3 (the reference's method, cpu_nvfp4.rs:729-777)
+            units.append([np.roll(host[nm][0].reshape(-1, 36), 1 + u, axis=0).reshape(-1) if u else host[nm][0] for nm in ("gate", "up", "down")])
+        xs = x32.reshape(1, K)
+        gsv = [host[nm][1] for nm in ("gate", "up", "down")]
+        for u in units:  # warm-up pass
+            orc.ffn(u[0], gsv[0], u[1], gsv[1], u[2], gsv[2], K, N, xs, threads=threads, path=1)
+        ts = []
+        for rep in range(24):
+            u = units[rep % 8]
+            c0 = time.perf_counter()
+            orc.ffn(u[0], gsv[0], u[1], gsv[1], u[2], gsv[2], K, N, xs, threads=threads, path=1)
+            ts.append(time.perf_counter() - c0)
+        ts.sort()
+        med = ts[len(ts) // 2]
+        out["cpu_baseline"] = {"value": round(3 * W_BYTES / med / 1e9, 2), "unit": "GB/s", "cores": threads, "kind": "port",
+                               "ms_per_step": round(med * 1e3, 3),
+                               "sample": "same step (gate/up + SiLU + down, one token, f32 x) on 8 rotating 150 MB weight units, median of 24 calls "
+                                         "after a warm-up pass; AVX2 path of the C restatement of engine/src/cpu_nvfp4.rs (OpenMP row split)"}
+    print(json.dumps(out))
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())
