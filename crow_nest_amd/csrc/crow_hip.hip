@@ -26,7 +26,7 @@ const FnEntry g_table[] = {
     CROW_FN(gemv_fp4_b, 7),        CROW_FN(gemv_fp4_b1k, 7),        CROW_FN(gemv_fp4_bs, 8),
     CROW_FN(gemv_fp4_ptrb, 8),     CROW_FN(moe_gate_up_silu, 8),    CROW_FN(moe_down_combine, 7),
     CROW_FN(router_top10, 10),     CROW_FN(silu_mul_combo, 3),      CROW_FN(acc_combo, 3),
-    CROW_FN(argmax_k, 3),          CROW_FN(dequant_fp4_flat, 4),    CROW_FN(repack_nvfp4, 4),
+    CROW_FN(argmax_k, 3),          CROW_FN(argmax_tiles, 2),          CROW_FN(dequant_fp4_flat, 4),    CROW_FN(repack_nvfp4, 4),
     CROW_FN(unpack_nvfp4, 4),      CROW_FN(dequant_nvfp4_tiled, 5), CROW_FN(gemm_nvfp4_bf16, 7),
     CROW_FN(gemm_nvfp4_bf16_m64, 7), CROW_FN(gemm_nvfp4_bf16_m32, 7),
 };
@@ -45,6 +45,8 @@ struct State {
 const unsigned long long PARTIAL_FLOATS = 16ull << 20;  // 64 MiB of split-K partial sums
 const unsigned COUNTER_SLOTS = 1u << 16;
 const unsigned AM_SLOTS = 1u << 16;
+// tile counters, then the status word, then 1 + AM_SLOTS / 64 argmax counters (top, groups)
+const unsigned COUNTER_WORDS = COUNTER_SLOTS + 1 + 1 + AM_SLOTS / 64;
 
 int hip_rc(hipError_t e) { return e == hipSuccess ? CROW_OK : (int)e; }
 
@@ -94,11 +96,11 @@ int crow_hip_init(int device) {
     ws.counter_slots = COUNTER_SLOTS;
     ws.am_slots = AM_SLOTS;
     if ((e = hipMalloc((void**)&ws.partials, PARTIAL_FLOATS * sizeof(float))) != hipSuccess) return (int)e;
-    if ((e = hipMalloc((void**)&ws.counters, (COUNTER_SLOTS + 2) * sizeof(unsigned))) != hipSuccess) return (int)e;
+    if ((e = hipMalloc((void**)&ws.counters, COUNTER_WORDS * sizeof(unsigned))) != hipSuccess) return (int)e;
     if ((e = hipMalloc((void**)&ws.am_val, AM_SLOTS * sizeof(float))) != hipSuccess) return (int)e;
     if ((e = hipMalloc((void**)&ws.am_idx, AM_SLOTS * sizeof(int))) != hipSuccess) return (int)e;
     if ((e = hipMalloc((void**)&g.scalars, 16 * sizeof(int))) != hipSuccess) return (int)e;
-    if ((e = hipMemset(ws.counters, 0, (COUNTER_SLOTS + 2) * sizeof(unsigned))) != hipSuccess) return (int)e;
+    if ((e = hipMemset(ws.counters, 0, COUNTER_WORDS * sizeof(unsigned))) != hipSuccess) return (int)e;
     ws.status = ws.counters + COUNTER_SLOTS;
     ws.am_counter = ws.counters + COUNTER_SLOTS + 1;
     if ((e = hipMemcpyToSymbol(HIP_SYMBOL(crow::g_ws), &ws, sizeof ws)) != hipSuccess) return (int)e;
@@ -244,7 +246,12 @@ int crow_hip_launch_dims(const char* name, uint32_t rows, uint32_t k_dim, uint32
     if (strncmp(name, "gemm_nvfp4_bf16", 15) == 0) {  // z = M token rows
         if (k_dim == 0 || k_dim % CROW_BLOCK_VALUES != 0) return CROW_ERR_SHAPE;
         const uint32_t mt = strcmp(name, "gemm_nvfp4_bf16_m32") == 0 ? 32 : (strcmp(name, "gemm_nvfp4_bf16_m64") == 0 ? 64 : 128);
-        *out = crow_dims{(rt + 3) / 4, (z + mt - 1) / mt, 1, 256};
+        if (mt == 32) {
+            if (z > 32) return CROW_ERR_SHAPE;
+            *out = crow_dims{rt, 1, 1, 256};
+        } else {
+            *out = crow_dims{(rt + 3) / 4, (z + mt - 1) / mt, 1, 256};
+        }
         return CROW_OK;
     }
     if (strcmp(name, "moe_down_combine") == 0) {
@@ -257,6 +264,7 @@ int crow_hip_launch_dims(const char* name, uint32_t rows, uint32_t k_dim, uint32
     }
     if (strcmp(name, "router_top10") == 0) { *out = crow_dims{z, 1, 1, 64}; return CROW_OK; }
     if (strcmp(name, "argmax_k") == 0) { *out = crow_dims{1, 1, 1, 1024}; return CROW_OK; }
+    if (strcmp(name, "argmax_tiles") == 0) { *out = crow_dims{1, 1, 1, 256}; return CROW_OK; }
     if (strcmp(name, "acc_combo") == 0) { *out = crow_dims{(rows + 255) / 256, z, 1, 256}; return CROW_OK; }  // rows = hidden
     if (strcmp(name, "silu_mul_combo") == 0 || strcmp(name, "dequant_fp4_flat") == 0) {  // rows = element count
         *out = crow_dims{(rows + 255) / 256, 1, 1, 256};
@@ -274,7 +282,7 @@ int crow_hip_status(void) {
     if (st == 0) return CROW_OK;
     (void)hipMemset(g.ws.status, 0, sizeof st);
     // a launch that bailed out may have left arrival counters behind
-    (void)hipMemset(g.ws.counters, 0, (COUNTER_SLOTS + 2) * sizeof(unsigned));
+    (void)hipMemset(g.ws.counters, 0, COUNTER_WORDS * sizeof(unsigned));
     if (st & CROW_STATUS_BAD_SCALE_BYTE) return CROW_ERR_SCALE_BYTE;
     if (st & crow::STATUS_WORKSPACE_TOO_SMALL) return CROW_ERR_WORKSPACE;
     if (st & crow::STATUS_BAD_GEO) return CROW_ERR_GEO;
@@ -285,7 +293,7 @@ int crow_hip_reset_workspace(void) {
     if (!g.ready) return CROW_ERR_NOT_INITIALIZED;
     hipError_t e = hipDeviceSynchronize();
     if (e != hipSuccess) return (int)e;
-    return hip_rc(hipMemset(g.ws.counters, 0, (COUNTER_SLOTS + 2) * sizeof(unsigned)));
+    return hip_rc(hipMemset(g.ws.counters, 0, COUNTER_WORDS * sizeof(unsigned)));
 }
 
 void crow_hip_set_stream(void* stream) { g.stream = (hipStream_t)stream; }

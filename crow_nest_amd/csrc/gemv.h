@@ -215,6 +215,60 @@ struct PanelFull<NR, M, XBF16, 2 * CROW_STEPS> {
                                                XChunk<XBF16> (&)[M], float (&)[NR][M]) {}
 };
 
+// f32 activations with M >= 3 rows: two 16-value chunks per row (current + prefetched) would need 128
+// SGPRs, more than a wave has, and the compiler then parks them in VGPR lanes.  The same chains
+// are therefore fed in 8-value chunks (one code word): chunk C is word C & 3 of step C >> 2, i.e.
+// half C & 1 of sub-block C >> 1.  Operation order per row is unchanged (one 16-long chain per
+// sub-block), so the results are bit-identical to the 16-value form.
+struct XHalf {
+    float v[8];
+    __device__ __forceinline__ void load(const void* x, size_t off) {
+        const float* p = (const float*)x + off;
+#pragma unroll
+        for (int j = 0; j < 8; j++) v[j] = p[j];
+    }
+};
+template <int NR, int M, int C>
+struct PanelFullHalf {
+    __device__ __forceinline__ static void run(const uint4 (&sc)[NR], const uint4 (&cd)[NR][CROW_STEPS], const void* x, size_t x_off,
+                                               size_t x_stride, int m_rows, float (&part)[NR][M], float (&acc)[NR][M]) {
+        // no software prefetch here: M * 8 SGPRs per chunk is all the scalar file affords next to the
+        // addressing; 4 + 8 M instructions per chunk and several waves per SIMD cover the scalar-cache latency
+        XHalf cur[M];
+#pragma unroll
+        for (int m = 0; m < M; m++)
+            if (m < m_rows) cur[m].load(x, (size_t)m * x_stride + x_off + C * 8);
+#pragma unroll
+        for (int r = 0; r < NR; r++) {
+            const unsigned word = u4_get(cd[r][C >> 2], C & 3);
+            const f32x2 a = fp4x2_to_f32<0>(word), b = fp4x2_to_f32<1>(word), c = fp4x2_to_f32<2>(word), d = fp4x2_to_f32<3>(word);
+            const float sf = scale_of<(C >> 1)>(sc[r]);
+#pragma unroll
+            for (int m = 0; m < M; m++) {
+                if (m < m_rows) {
+                    float p = (C & 1) ? __builtin_fmaf(a.x, cur[m].v[0], part[r][m]) : a.x * cur[m].v[0];
+                    p = __builtin_fmaf(a.y, cur[m].v[1], p);
+                    p = __builtin_fmaf(b.x, cur[m].v[2], p);
+                    p = __builtin_fmaf(b.y, cur[m].v[3], p);
+                    p = __builtin_fmaf(c.x, cur[m].v[4], p);
+                    p = __builtin_fmaf(c.y, cur[m].v[5], p);
+                    p = __builtin_fmaf(d.x, cur[m].v[6], p);
+                    p = __builtin_fmaf(d.y, cur[m].v[7], p);
+                    part[r][m] = p;
+                    if (C & 1) acc[r][m] = __builtin_fmaf(p, sf, acc[r][m]);
+                }
+            }
+        }
+        __builtin_amdgcn_sched_barrier(0);
+        PanelFullHalf<NR, M, C + 1>::run(sc, cd, x, x_off, x_stride, m_rows, part, acc);
+    }
+};
+template <int NR, int M>
+struct PanelFullHalf<NR, M, 32> {
+    __device__ __forceinline__ static void run(const uint4 (&)[NR], const uint4 (&)[NR][CROW_STEPS], const void*, size_t, size_t, int,
+                                               float (&)[NR][M], float (&)[NR][M]) {}
+};
+
 template <int NR>
 __device__ __forceinline__ void load_tile(const unsigned char* const (&w)[2], int rt, int panels, int p, int lane,
                                           uint4 (&sc)[NR], uint4 (&cd)[NR][CROW_STEPS]) {
@@ -234,7 +288,10 @@ __device__ __forceinline__ void panel_compute(const uint4 (&sc)[NR], const uint4
 #ifdef CROW_DEBUG_X0
     p = 0;  // experiment only: every panel reads the same 1 KB of x
 #endif
-    if (left >= CROW_STEPS) {
+    if (left >= CROW_STEPS && !XBF16 && M >= 3) {
+        float part[NR][M];
+        PanelFullHalf<NR, M, 0>::run(sc, cd, x, (size_t)p * CROW_PANEL_COLS, x_stride, m_rows, part, acc);
+    } else if (left >= CROW_STEPS) {
         XChunk<XBF16> first[M];
 #pragma unroll
         for (int m = 0; m < M; m++)
@@ -385,42 +442,19 @@ __device__ __forceinline__ void gemv_body(const GemvArgs& a, unsigned z, float* 
 
     const int row = rt * CROW_TILE_ROWS + lane;
     if (EPI == EPI_SCALE && a.argmax_out != nullptr) {
-        // fused head: logits out, then one (value, index) candidate per row tile; the tile that
-        // arrives last scans all candidates.  The order is total, so arrival order cannot matter.
+        // fused head, stage 1: logits out and one (value, index) candidate per row tile into the
+        // workspace, plain stores, no waiting (a wave that lingers for an arrival protocol keeps
+        // its block's slots busy: measured +15 % on the whole launch).  Stage 2 is argmax_tiles.
         const float v = acc[0][0] * a.gs[0][0];
         if (row < a.rows) a.y[row] = v;
-        Best b = wave_best(Best{row < a.rows ? v : -3.0e38f, row < a.rows ? row : 0});
-        const unsigned tiles = (unsigned)row_tiles;
-        if (tiles > ws.am_slots) {
+        const Best b = wave_best(Best{row < a.rows ? v : -3.0e38f, row < a.rows ? row : 0});
+        if ((unsigned)row_tiles > ws.am_slots) {
             if (lane == 0) atomicOr(ws.status, STATUS_WORKSPACE_TOO_SMALL);
             return;
         }
-        gfloat_p am_val = (gfloat_p)ws.am_val;
-        gint_p am_idx = (gint_p)ws.am_idx;
-        guint_p am_counter = (guint_p)ws.am_counter;
-        unsigned arrived = 0;
         if (lane == 0) {
-            __hip_atomic_store(am_val + rt, b.v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-            __hip_atomic_store(am_idx + rt, b.i, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-            device_order();
-            arrived = __hip_atomic_fetch_add(am_counter, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        }
-        arrived = __builtin_amdgcn_readfirstlane(arrived);
-        if (arrived != tiles - 1) return;
-        device_order();
-        Best g{-3.0e38f, 0};
-        for (unsigned t = lane; t < tiles; t += 64) {
-            const float tv = __hip_atomic_load(am_val + t, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-            const int ti = __hip_atomic_load(am_idx + t, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-            if (better(tv, ti, g.v, g.i)) {
-                g.v = tv;
-                g.i = ti;
-            }
-        }
-        g = wave_best(g);
-        if (lane == 0) {
-            a.argmax_out[0] = g.i;
-            __hip_atomic_store(am_counter, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            ws.am_val[rt] = b.v;
+            ws.am_idx[rt] = b.i;
         }
         return;
     }

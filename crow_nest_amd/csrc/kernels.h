@@ -37,8 +37,11 @@ extern "C" __global__ void __launch_bounds__(1024) gemv_fp4(const unsigned char*
     RED(1, 1); gemv_body<1, 1, false, EPI_SCALE, RED_N(1, 1)>(a, 0, red);
 }
 
-// lm_head with the greedy argmax fused in: logits[rows] and out_idx[0] from one launch.  Replaces
-// lm_head_row + argmax_k (engine/src/gen.rs:4766-4784, engine/src/kernels.rs:4238-4260), same tie rule.
+// lm_head with the first stage of the greedy argmax fused in: logits[rows], and one candidate per 64-row
+// tile kept in the library workspace; argmax_tiles(out_idx, rows_p) then picks the token from those
+// ceil(rows / 64) candidates instead of re-reading all logits.  Together they replace lm_head_row +
+// argmax_k (engine/src/gen.rs:4766-4784, engine/src/kernels.rs:4238-4260), same tie rule.
+// out_idx is only a flag here (non-null selects the fused epilogue); argmax_tiles writes it.
 extern "C" __global__ void __launch_bounds__(1024) gemv_nvfp4_w_argmax(const unsigned char* __restrict__ w, const float* __restrict__ x,
                                                                        const float* __restrict__ gs_ptr, float* __restrict__ y,
                                                                        const int* __restrict__ k_dim_p, const int* __restrict__ rows_p,

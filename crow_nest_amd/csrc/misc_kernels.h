@@ -267,3 +267,36 @@ extern "C" __global__ void __launch_bounds__(1024) argmax_k(const float* __restr
         out[0] = b.i;
     }
 }
+
+// Stage 2 of the fused head: the greedy token from the per-row-tile candidates gemv_nvfp4_w_argmax left in
+// the workspace (ceil(rows / 64) of them).  grid (1), block 256.  Same total order as argmax_k.
+extern "C" __global__ void __launch_bounds__(256) argmax_tiles(int* __restrict__ out, const int* __restrict__ rows_p) {
+    __shared__ float sv[4];
+    __shared__ int si[4];
+    const Workspace ws = g_ws;
+    const int tiles = (*rows_p + CROW_TILE_ROWS - 1) / CROW_TILE_ROWS;
+    Best b{-3.0e38f, 0};
+    for (int t = (int)threadIdx.x; t < tiles && t < (int)ws.am_slots; t += 256) {
+        const float v = ws.am_val[t];
+        const int i = ws.am_idx[t];
+        if (better(v, i, b.v, b.i)) {
+            b.v = v;
+            b.i = i;
+        }
+    }
+    b = wave_best(b);
+    const int wave = (int)(threadIdx.x >> 6);
+    if (lane_id() == 0) {
+        sv[wave] = b.v;
+        si[wave] = b.i;
+    }
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        for (int w = 1; w < 4; w++)
+            if (better(sv[w], si[w], b.v, b.i)) {
+                b.v = sv[w];
+                b.i = si[w];
+            }
+        out[0] = b.i;
+    }
+}
