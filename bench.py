@@ -211,7 +211,11 @@ def main() -> int:
         heads = [rnd(vb) for _ in range(4)]
         idx = torch.zeros(1, dtype=torch.int32, device=dev)
         l3 = Launch(eng, "gemv_nvfp4_w_argmax", V, K, 1, [[hd.data_ptr(), xk.data_ptr(), gs1.data_ptr(), ybuf.data_ptr(), p.i32(K), p.i32(V), idx.data_ptr()] for hd in heads])
-        others["config3_lm_head_151936x5120_argmax"] = entry(l3.us(iters=100), V * K // 64 * 36 + K * 4 + V * 4 + 4)
+        from crow_nest_amd.kernels import time_sequence
+        seq3 = [(l3.f, l3.dims, l3.raw), (eng.k.f("argmax_tiles"), (1, 1, 1, 256), [[idx.data_ptr(), p.i32(V)]])]
+        time_sequence(seq3, 4, 10)
+        others["config3_lm_head_151936x5120_argmax"] = entry(min(time_sequence(seq3, 4, 100) for _ in range(3)), V * K // 64 * 36 + K * 4 + V * 4 + 4)
+        others["config3_lm_head_151936x5120_argmax"]["launches"] = 2
         del heads
         # config 4: batched GEMM on the matrix cores
         for m in (16, 128, 512):
@@ -252,19 +256,9 @@ def main() -> int:
             ldn = Launch(eng, "moe_down_combine", H, I, t, [[dnp.data_ptr(), h2.data_ptr(), gs1.data_ptr(), wts.data_ptr(), yt.data_ptr(), p.i32(I), p.i32(H)]])
             ldn.dims = (1, (H + 63) // 64, t, 64 * K8)
 
-            def layer(i):
-                lr.go(lib, i)
-                lgu.go(lib, 0)
-                ldn.go(lib, 0)
-            for i in range(10):
-                layer(i)
-            e0, e1 = Event(), Event()
-            e0.record()
-            reps = 200
-            for i in range(reps):
-                layer(i)
-            e1.record()
-            us = e0.elapsed_ms(e1) * 1e3 / reps
+            seq2 = [(lr.f, lr.dims, lr.raw), (lgu.f, lgu.dims, lgu.raw), (ldn.f, ldn.dims, ldn.raw)]
+            time_sequence(seq2, 3, 10)
+            us = min(time_sequence(seq2, 3, 200) for _ in range(3))
             nbytes = min(t * 8, E) * (E and (2 * I * H // 64 * 36 + H * I // 64 * 36)) + t * H * 8 + t * E * 4  # t*8 distinct experts at most
             others[f"config2_moe_layer_T{t}"] = entry(us, nbytes)
             others[f"config2_moe_layer_T{t}"]["launches"] = 3

@@ -365,6 +365,39 @@ int crow_hip_time_launches(crow_fn_t f, uint32_t gx, uint32_t gy, uint32_t gz, u
     return out;
 }
 
+int crow_hip_time_sequence(uint32_t n_kernels, const crow_fn_t* fns, const crow_dims* dims, const uint32_t* n_vals,
+                           const uint64_t* vals, uint32_t n_sets, uint32_t iters, float* us_per_iteration) {
+    if (!g.ready) return CROW_ERR_NOT_INITIALIZED;
+    if (!fns || !dims || !n_vals || !vals || !us_per_iteration || n_kernels == 0 || n_kernels > 16 || n_sets == 0 || iters == 0)
+        return CROW_ERR_BAD_ARGUMENT;
+    size_t per_set = 0;
+    for (uint32_t k = 0; k < n_kernels; k++) {
+        const FnEntry* e = (const FnEntry*)(void*)fns[k];
+        if (e < g_table || e >= g_table + g_table_n) return CROW_ERR_KERNEL_MISSING;
+        per_set += n_vals[k];
+    }
+    hipEvent_t a, b;
+    hipError_t rc;
+    if ((rc = hipEventCreate(&a)) != hipSuccess) return (int)rc;
+    if ((rc = hipEventCreate(&b)) != hipSuccess) return (int)rc;
+    int out = hip_rc(hipEventRecord(a, g.stream));
+    for (uint32_t i = 0; i < iters && out == CROW_OK; i++) {
+        const uint64_t* v = vals + (size_t)(i % n_sets) * per_set;
+        for (uint32_t k = 0; k < n_kernels && out == CROW_OK; k++) {
+            out = launch_entry((const FnEntry*)(void*)fns[k], dim3(dims[k].gx, dims[k].gy, dims[k].gz), dim3(dims[k].bx), v, n_vals[k], g.stream);
+            v += n_vals[k];
+        }
+    }
+    if (out == CROW_OK) out = hip_rc(hipEventRecord(b, g.stream));
+    if (out == CROW_OK) out = hip_rc(hipEventSynchronize(b));
+    float ms = 0.0f;
+    if (out == CROW_OK) out = hip_rc(hipEventElapsedTime(&ms, a, b));
+    (void)hipEventDestroy(a);
+    (void)hipEventDestroy(b);
+    *us_per_iteration = ms * 1000.0f / (float)iters;
+    return out;
+}
+
 size_t crow_hip_container_bytes(uint32_t rows, uint32_t cols) { return crow_container_bytes(rows, cols); }
 size_t crow_hip_tiled_bytes(uint32_t rows, uint32_t cols) { return crow_tiled_bytes(rows, cols); }
 

@@ -7,6 +7,15 @@ namespace crow {
 
 typedef float f32x2 __attribute__((ext_vector_type(2)));
 typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+typedef unsigned stream_u32x4 __attribute__((ext_vector_type(4)));
+
+// 16-byte load of weight bytes that are read exactly once per launch: the non-temporal hint keeps them from
+// displacing reusable lines in L2 and the memory-side cache (measured on a pure read of the tile pattern:
+// 6.8-6.9 TB/s against 6.1-6.3 TB/s without the hint at 437 MB, 5.8 against 5.5 at 50 MB)
+__device__ __forceinline__ uint4 stream_load(const uint4* p) {
+    const stream_u32x4 v = __builtin_nontemporal_load((const stream_u32x4*)p);
+    return make_uint4(v.x, v.y, v.z, v.w);
+}
 
 // Library-owned scratch for kernels that split one output tile over several workgroups:
 // per-slice partial sums and one arrival counter per output tile.  Set once by crow_hip_init.

@@ -114,9 +114,9 @@ __device__ __forceinline__ void gemm_body(const unsigned char* __restrict__ w, c
     auto load_w = [&](int p, uint4& sc, uint4 (&cd)[CROW_STEPS]) {
         if (has_rows && p < panels) {
             const uint4* t = wt + (size_t)p * (CROW_TILE_BYTES / 16);
-            sc = t[0];
+            sc = stream_load(t);
 #pragma unroll
-            for (int s = 0; s < CROW_STEPS; s++) cd[s] = t[64 * (s + 1)];
+            for (int s = 0; s < CROW_STEPS; s++) cd[s] = stream_load(t + 64 * (s + 1));
         }
     };
     auto stage_x = [&](int p) {
@@ -205,9 +205,9 @@ __device__ __forceinline__ void gemm_small_body(const unsigned char* __restrict_
     auto load_w = [&](int p, uint4& sc, uint4 (&cd)[CROW_STEPS]) {
         if (p < panels) {
             const uint4* t = wt + (size_t)p * (CROW_TILE_BYTES / 16);
-            sc = t[0];
+            sc = stream_load(t);
 #pragma unroll
-            for (int s = 0; s < CROW_STEPS; s++) cd[s] = t[64 * (s + 1)];
+            for (int s = 0; s < CROW_STEPS; s++) cd[s] = stream_load(t + 64 * (s + 1));
         }
     };
     auto stage_x = [&](int p) {  // 32 tokens x 256 columns = 1024 chunks of 16 bytes, 16 per lane; wave-private

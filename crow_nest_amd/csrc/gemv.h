@@ -275,9 +275,9 @@ __device__ __forceinline__ void load_tile(const unsigned char* const (&w)[2], in
 #pragma unroll
     for (int r = 0; r < NR; r++) {
         const uint4* t = (const uint4*)(w[r] + ((size_t)rt * panels + p) * CROW_TILE_BYTES) + lane;
-        sc[r] = t[0];
+        sc[r] = stream_load(t);
 #pragma unroll
-        for (int s = 0; s < CROW_STEPS; s++) cd[r][s] = t[64 * (s + 1)];
+        for (int s = 0; s < CROW_STEPS; s++) cd[r][s] = stream_load(t + 64 * (s + 1));
     }
 }
 
@@ -285,9 +285,6 @@ template <int NR, int M, bool XBF16>
 __device__ __forceinline__ void panel_compute(const uint4 (&sc)[NR], const uint4 (&cd)[NR][CROW_STEPS], int p, int k_dim,
                                               const void* x, size_t x_stride, int m_rows, float (&acc)[NR][M]) {
     const int left = (k_dim - p * CROW_PANEL_COLS) / CROW_STEP_COLS;
-#ifdef CROW_DEBUG_X0
-    p = 0;  // experiment only: every panel reads the same 1 KB of x
-#endif
     if (left >= CROW_STEPS && !XBF16 && M >= 3) {
         float part[NR][M];
         PanelFullHalf<NR, M, 0>::run(sc, cd, x, (size_t)p * CROW_PANEL_COLS, x_stride, m_rows, part, acc);
@@ -329,15 +326,7 @@ __device__ __forceinline__ void tile_accumulate(const unsigned char* const (&w)[
     for (int p = p0; p < panels; p += stride) {
         uint4 sc[NR], cd[NR][CROW_STEPS];
         load_tile<NR>(w, rt, panels, p, lane, sc, cd);
-#ifdef CROW_EXP_NOCOMPUTE
-        for (int r = 0; r < NR; r++) {
-            unsigned q = sc[r].x ^ sc[r].y ^ sc[r].z ^ sc[r].w;
-            for (int s = 0; s < CROW_STEPS; s++) q ^= cd[r][s].x ^ cd[r][s].y ^ cd[r][s].z ^ cd[r][s].w;
-            acc[r][0] += __uint_as_float(q & 0x3fffffffu);
-        }
-#else
         panel_compute<NR, M, XBF16>(sc, cd, p, k_dim, x, x_stride, m_rows, acc);
-#endif
     }
 }
 
@@ -388,11 +377,7 @@ __device__ __forceinline__ void gemv_body(const GemvArgs& a, unsigned z, float* 
     }
 
     // slices of the row tile -> the last one to arrive, in slice order
-#ifdef CROW_EXP_NOREDUCE
-    if (false) {
-#else
     if (slices > 1) {
-#endif
         const size_t need = ((size_t)tile_id + 1) * slices * (NR * M) * 64;
         if (need > ws.partial_floats || tile_id >= ws.counter_slots) {
             if (lane == 0) atomicOr(ws.status, STATUS_WORKSPACE_TOO_SMALL);

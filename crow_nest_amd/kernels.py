@@ -126,6 +126,23 @@ def time_launches(f: int, gx: int, gy: int, gz: int, bx: int, arg_sets, iters: i
     return float(us.value)
 
 
+def time_sequence(kernels, n_sets: int, iters: int) -> float:
+    """Mean microseconds per iteration of a launch SEQUENCE.  `kernels` = [(f, (gx, gy, gz, bx), arg_sets), ...];
+    every kernel has `n_sets` argument sets (a kernel with one set repeats it); iteration i uses set i % n_sets."""
+    nk = len(kernels)
+    fns = (C.c_void_p * nk)(*[k[0] for k in kernels])
+    dims = (_l.Dims * nk)(*[_l.Dims(*k[1]) for k in kernels])
+    nv = (C.c_uint32 * nk)(*[len(k[2][0]) for k in kernels])
+    flat = []
+    for s in range(n_sets):
+        for _, _, sets in kernels:
+            flat.extend(int(v) for v in sets[s % len(sets)])
+    arr = (C.c_uint64 * len(flat))(*flat)
+    us = C.c_float()
+    _l.check(_l.lib().crow_hip_time_sequence(nk, fns, dims, nv, arr, n_sets, iters, C.byref(us)), "crow_hip_time_sequence")
+    return float(us.value)
+
+
 class Event:
     """A HIP event on the library's current stream (the stream every launch_v goes to)."""
 

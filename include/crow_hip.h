@@ -97,6 +97,11 @@ int crow_hip_event_destroy(void* ev);
  * larger than the 256 MB memory-side cache).  Returns the mean microseconds per launch. */
 int crow_hip_time_launches(crow_fn_t f, uint32_t gx, uint32_t gy, uint32_t gz, uint32_t bx, const uint64_t* vals,
                            uint32_t n_vals, uint32_t n_sets, uint32_t iters, float* us_per_launch);
+/* the same for a SEQUENCE of n_kernels launches per iteration (e.g. router -> gate|up -> down): dims[k] and
+ * n_vals[k] per kernel; argument set s of iteration i = vals + (i % n_sets) * sum(n_vals), kernels back to back
+ * inside it.  Returns the mean microseconds per iteration (per sequence). */
+int crow_hip_time_sequence(uint32_t n_kernels, const crow_fn_t* fns, const crow_dims* dims, const uint32_t* n_vals,
+                           const uint64_t* vals, uint32_t n_sets, uint32_t iters, float* us_per_iteration);
 
 /* ---- load-time repack (the one call the reference does not have) ---- */
 size_t crow_hip_container_bytes(uint32_t rows, uint32_t cols);
