@@ -9,6 +9,14 @@ typedef float f32x2 __attribute__((ext_vector_type(2)));
 typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
 typedef unsigned stream_u32x4 __attribute__((ext_vector_type(4)));
 
+// blockDim.x read as a scalar from the kernel's implicit arguments (u16 group_size_x at byte 12 of the hidden block:
+// the compiler's own blockDim.x is a 16-bit VECTOR load followed by a wait, which sits in front of the first weight
+// load of every wave).  Launches here never have a partial last block, so the remainder field is not consulted.
+__device__ __forceinline__ int block_threads() {
+    const unsigned* ia = (const unsigned*)__builtin_amdgcn_implicitarg_ptr();
+    return (int)(ia[3] & 0xffffu);
+}
+
 // 16-byte load of weight bytes that are read exactly once per launch: the non-temporal hint keeps them from
 // displacing reusable lines in L2 and the memory-side cache (measured on a pure read of the tile pattern:
 // 6.8-6.9 TB/s against 6.1-6.3 TB/s without the hint at 437 MB, 5.8 against 5.5 at 50 MB)

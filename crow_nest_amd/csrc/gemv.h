@@ -338,16 +338,15 @@ typedef __attribute__((address_space(1))) int* gint_p;
 // its token group / combo `z`, which only indexes the workspace here.  `red` is the block's LDS
 // hand-over buffer of (W - 1) * NR * M * 64 floats (RED_FLOATS of them are there).
 template <int NR, int M, bool XBF16, int EPI, int RED_FLOATS>
-__device__ __forceinline__ void gemv_body(const GemvArgs& a, unsigned z, float* red) {
+__device__ __forceinline__ void gemv_body(const GemvArgs& a, unsigned z, float* red, const Workspace& ws) {
     const int lane = lane_id();
-    const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6)), waves = (int)(blockDim.x >> 6);  // wave-uniform on purpose
+    const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6)), waves = block_threads() >> 6;  // wave-uniform on purpose
     const int slice = (int)blockIdx.x, slices = (int)gridDim.x;
     const int rt = (int)blockIdx.y;
     const int row_tiles = (int)gridDim.y;
     const int panels = (a.k_dim + CROW_PANEL_COLS - 1) / CROW_PANEL_COLS;
     const int m_rows = a.m < M ? a.m : M;
     const unsigned tile_id = z * (unsigned)row_tiles + (unsigned)rt;
-    const Workspace ws = g_ws;  // read early: its latency hides behind the weight loads
 
     float acc[NR][M];
     tile_accumulate<NR, M, XBF16>(a.w, rt, panels, slice * waves + wave, slices * waves, a.k_dim, a.x, a.x_stride, m_rows, acc);

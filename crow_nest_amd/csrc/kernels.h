@@ -13,28 +13,37 @@ using namespace crow;
 // LDS hand-over buffer of a GEMV block: up to 16 waves, NR tensors, M activation rows
 #define RED_N(NR, M) (15 * (NR) * (M) * 64)
 #define RED(NR, M) __shared__ float red[RED_N(NR, M)]
+// First statement of every GEMV entry point: the workspace descriptor is fetched with the kernel arguments, in the
+// first scalar round trip.  Left alone the compiler issues it after the shape words behind k_dim_p / rows_p have
+// arrived, as a third dependent round trip in front of every wave's first weight load.
+#define ENTER(...)                \
+    const Workspace ws = g_ws;    \
+    __builtin_amdgcn_sched_barrier(0)
 
 // ------------------------------------------------------------------ dense GEMV (decode, one row)
 // reference: gemv_nvfp4_w, engine/src/kernels_p2.rs:355-368
 extern "C" __global__ void __launch_bounds__(1024) gemv_nvfp4_w(const unsigned char* __restrict__ w, const float* __restrict__ x,
                                                                 const float* __restrict__ gs_ptr, float* __restrict__ y,
                                                                 const int* __restrict__ k_dim_p, const int* __restrict__ rows_p) {
+    ENTER(w, x, gs_ptr, y, k_dim_p, rows_p);
     GemvArgs a{{w, nullptr}, {gs_ptr, nullptr}, x, 0, y, 0, *k_dim_p, *rows_p, 1, nullptr};
-    RED(1, 1); gemv_body<1, 1, false, EPI_SCALE, RED_N(1, 1)>(a, 0, red);
+    RED(1, 1); gemv_body<1, 1, false, EPI_SCALE, RED_N(1, 1)>(a, 0, red, ws);
 }
 // the same product on bf16 activations (exact widening; BASELINE configs quote X in bf16)
 extern "C" __global__ void __launch_bounds__(1024) gemv_nvfp4_w_bf16(const unsigned char* __restrict__ w, const unsigned short* __restrict__ x,
                                                                      const float* __restrict__ gs_ptr, float* __restrict__ y,
                                                                      const int* __restrict__ k_dim_p, const int* __restrict__ rows_p) {
+    ENTER(w, x, gs_ptr, y, k_dim_p, rows_p);
     GemvArgs a{{w, nullptr}, {gs_ptr, nullptr}, x, 0, y, 0, *k_dim_p, *rows_p, 1, nullptr};
-    RED(1, 1); gemv_body<1, 1, true, EPI_SCALE, RED_N(1, 1)>(a, 0, red);
+    RED(1, 1); gemv_body<1, 1, true, EPI_SCALE, RED_N(1, 1)>(a, 0, red, ws);
 }
 // reference: gemv_fp4, engine/src/kernels.rs:118-151 (+ rows_p: the reference's grid.x is the row count)
 extern "C" __global__ void __launch_bounds__(1024) gemv_fp4(const unsigned char* __restrict__ w, const float* __restrict__ x,
                                                             const float* __restrict__ gs_ptr, float* __restrict__ y,
                                                             const int* __restrict__ k_dim_p, const int* __restrict__ rows_p) {
+    ENTER(w, x, gs_ptr, y, k_dim_p, rows_p);
     GemvArgs a{{w, nullptr}, {gs_ptr, nullptr}, x, 0, y, 0, *k_dim_p, *rows_p, 1, nullptr};
-    RED(1, 1); gemv_body<1, 1, false, EPI_SCALE, RED_N(1, 1)>(a, 0, red);
+    RED(1, 1); gemv_body<1, 1, false, EPI_SCALE, RED_N(1, 1)>(a, 0, red, ws);
 }
 
 // lm_head with the first stage of the greedy argmax fused in: logits[rows], and one candidate per 64-row
@@ -46,8 +55,9 @@ extern "C" __global__ void __launch_bounds__(1024) gemv_nvfp4_w_argmax(const uns
                                                                        const float* __restrict__ gs_ptr, float* __restrict__ y,
                                                                        const int* __restrict__ k_dim_p, const int* __restrict__ rows_p,
                                                                        int* __restrict__ out_idx) {
+    ENTER(w, x, gs_ptr, y, k_dim_p, rows_p, out_idx);
     GemvArgs a{{w, nullptr}, {gs_ptr, nullptr}, x, 0, y, 0, *k_dim_p, *rows_p, 1, out_idx};
-    RED(1, 1); gemv_body<1, 1, false, EPI_SCALE, RED_N(1, 1)>(a, 0, red);
+    RED(1, 1); gemv_body<1, 1, false, EPI_SCALE, RED_N(1, 1)>(a, 0, red, ws);
 }
 
 // ------------------------------------------------------------------ fused gate/up + SiLU (decode)
@@ -56,19 +66,20 @@ extern "C" __global__ void __launch_bounds__(1024) gemv_nvfp4_gu(const unsigned 
                                                                  const float* __restrict__ x, const float* __restrict__ gs_g,
                                                                  const float* __restrict__ gs_u, float* __restrict__ y,
                                                                  const int* __restrict__ k_dim_p, const int* __restrict__ rows_p) {
+    ENTER(wg, wu, x, gs_g, gs_u, y, k_dim_p, rows_p);
     GemvArgs a{{wg, wu}, {gs_g, gs_u}, x, 0, y, 0, *k_dim_p, *rows_p, 1, nullptr};
-    RED(2, 1); gemv_body<2, 1, false, EPI_SILU_GU, RED_N(2, 1)>(a, 0, red);
+    RED(2, 1); gemv_body<2, 1, false, EPI_SILU_GU, RED_N(2, 1)>(a, 0, red, ws);
 }
 
 // ------------------------------------------------------------------ M <= 4 rows (MTP verify)
 template <int NR, bool XBF16, int EPI>
-__device__ __forceinline__ void gemv_m_dispatch(GemvArgs& a, unsigned z, float* red) {
+__device__ __forceinline__ void gemv_m_dispatch(GemvArgs& a, unsigned z, float* red, const Workspace& ws) {
     // one body per M keeps each row's operation sequence identical to the one-row kernel
     switch (a.m) {
-        case 1: gemv_body<NR, 1, XBF16, EPI, RED_N(NR, 4)>(a, z, red); break;
-        case 2: gemv_body<NR, 2, XBF16, EPI, RED_N(NR, 4)>(a, z, red); break;
-        case 3: gemv_body<NR, 3, XBF16, EPI, RED_N(NR, 4)>(a, z, red); break;
-        default: gemv_body<NR, 4, XBF16, EPI, RED_N(NR, 4)>(a, z, red); break;
+        case 1: gemv_body<NR, 1, XBF16, EPI, RED_N(NR, 4)>(a, z, red, ws); break;
+        case 2: gemv_body<NR, 2, XBF16, EPI, RED_N(NR, 4)>(a, z, red, ws); break;
+        case 3: gemv_body<NR, 3, XBF16, EPI, RED_N(NR, 4)>(a, z, red, ws); break;
+        default: gemv_body<NR, 4, XBF16, EPI, RED_N(NR, 4)>(a, z, red, ws); break;
     }
 }
 // reference: gemv_nvfp4_wm, engine/src/kernels_p2.rs:472-497
@@ -76,9 +87,10 @@ extern "C" __global__ void __launch_bounds__(1024) gemv_nvfp4_wm(const unsigned 
                                                                  const float* __restrict__ gs_ptr, float* __restrict__ y,
                                                                  const int* __restrict__ k_dim_p, const int* __restrict__ rows_p,
                                                                  const int* __restrict__ m_p) {
+    ENTER(w, x, gs_ptr, y, k_dim_p, rows_p, m_p);
     const int k = *k_dim_p, rows = *rows_p;
     GemvArgs a{{w, nullptr}, {gs_ptr, nullptr}, x, (size_t)k, y, (size_t)rows, k, rows, *m_p, nullptr};
-    RED(1, 4); gemv_m_dispatch<1, false, EPI_SCALE>(a, 0, red);
+    RED(1, 4); gemv_m_dispatch<1, false, EPI_SCALE>(a, 0, red, ws);
 }
 // reference: gemv_nvfp4_gum, engine/src/kernels_p2.rs:499-530
 extern "C" __global__ void __launch_bounds__(1024) gemv_nvfp4_gum(const unsigned char* __restrict__ wg, const unsigned char* __restrict__ wu,
@@ -86,57 +98,63 @@ extern "C" __global__ void __launch_bounds__(1024) gemv_nvfp4_gum(const unsigned
                                                                   const float* __restrict__ gs_u, float* __restrict__ y,
                                                                   const int* __restrict__ k_dim_p, const int* __restrict__ rows_p,
                                                                   const int* __restrict__ m_p) {
+    ENTER(wg, wu, x, gs_g, gs_u, y, k_dim_p, rows_p, m_p);
     const int k = *k_dim_p, rows = *rows_p;
     GemvArgs a{{wg, wu}, {gs_g, gs_u}, x, (size_t)k, y, (size_t)rows, k, rows, *m_p, nullptr};
-    RED(2, 4); gemv_m_dispatch<2, false, EPI_SILU_GU>(a, 0, red);
+    RED(2, 4); gemv_m_dispatch<2, false, EPI_SILU_GU>(a, 0, red, ws);
 }
 // bf16-activation twins of the two verify kernels (X [M][k_dim] bf16, outputs f32)
 extern "C" __global__ void __launch_bounds__(1024) gemv_nvfp4_wm_bf16(const unsigned char* __restrict__ w, const unsigned short* __restrict__ x,
                                                                       const float* __restrict__ gs_ptr, float* __restrict__ y,
                                                                       const int* __restrict__ k_dim_p, const int* __restrict__ rows_p,
                                                                       const int* __restrict__ m_p) {
+    ENTER(w, x, gs_ptr, y, k_dim_p, rows_p, m_p);
     const int k = *k_dim_p, rows = *rows_p;
     GemvArgs a{{w, nullptr}, {gs_ptr, nullptr}, x, (size_t)k, y, (size_t)rows, k, rows, *m_p, nullptr};
-    RED(1, 4); gemv_m_dispatch<1, true, EPI_SCALE>(a, 0, red);
+    RED(1, 4); gemv_m_dispatch<1, true, EPI_SCALE>(a, 0, red, ws);
 }
 extern "C" __global__ void __launch_bounds__(1024) gemv_nvfp4_gum_bf16(const unsigned char* __restrict__ wg, const unsigned char* __restrict__ wu,
                                                                        const unsigned short* __restrict__ x, const float* __restrict__ gs_g,
                                                                        const float* __restrict__ gs_u, float* __restrict__ y,
                                                                        const int* __restrict__ k_dim_p, const int* __restrict__ rows_p,
                                                                        const int* __restrict__ m_p) {
+    ENTER(wg, wu, x, gs_g, gs_u, y, k_dim_p, rows_p, m_p);
     const int k = *k_dim_p, rows = *rows_p;
     GemvArgs a{{wg, wu}, {gs_g, gs_u}, x, (size_t)k, y, (size_t)rows, k, rows, *m_p, nullptr};
-    RED(2, 4); gemv_m_dispatch<2, true, EPI_SILU_GU>(a, 0, red);
+    RED(2, 4); gemv_m_dispatch<2, true, EPI_SILU_GU>(a, 0, red, ws);
 }
 
 // ------------------------------------------------------------------ batched over token rows
 // reference: gemv_fp4_b / gemv_fp4_b1k, engine/src/kernels.rs:154-189,1302-1337 and gemv_fp4_bs,
 // :1022-1058.  grid.z = ceil(T / 4): each block decodes its weights once for up to 4 token rows.
 __device__ __forceinline__ void gemv_tokens(const unsigned char* w, const float* x, const float* gs, float* y, int k, int rows,
-                                            int t_total, size_t y_stride) {
+                                            int t_total, size_t y_stride, const Workspace& ws) {
     const int t0 = (int)blockIdx.z * 4;
     if (t0 >= t_total) return;
     GemvArgs a{{w, nullptr}, {gs, nullptr}, x + (size_t)t0 * k, (size_t)k, y + (size_t)t0 * y_stride, y_stride, k, rows,
                t_total - t0 < 4 ? t_total - t0 : 4, nullptr};
-    RED(1, 4); gemv_m_dispatch<1, false, EPI_SCALE>(a, blockIdx.z, red);
+    RED(1, 4); gemv_m_dispatch<1, false, EPI_SCALE>(a, blockIdx.z, red, ws);
 }
 extern "C" __global__ void __launch_bounds__(1024) gemv_fp4_b(const unsigned char* __restrict__ w, const float* __restrict__ x,
                                                               const float* __restrict__ gs_ptr, float* __restrict__ y,
                                                               const int* __restrict__ k_dim_p, const int* __restrict__ rows_p,
                                                               const int* __restrict__ t_p) {
-    gemv_tokens(w, x, gs_ptr, y, *k_dim_p, *rows_p, *t_p, (size_t)*rows_p);
+    ENTER(w, x, gs_ptr, y, k_dim_p, rows_p, t_p);
+    gemv_tokens(w, x, gs_ptr, y, *k_dim_p, *rows_p, *t_p, (size_t)*rows_p, ws);
 }
 extern "C" __global__ void __launch_bounds__(1024) gemv_fp4_b1k(const unsigned char* __restrict__ w, const float* __restrict__ x,
                                                                 const float* __restrict__ gs_ptr, float* __restrict__ y,
                                                                 const int* __restrict__ k_dim_p, const int* __restrict__ rows_p,
                                                                 const int* __restrict__ t_p) {
-    gemv_tokens(w, x, gs_ptr, y, *k_dim_p, *rows_p, *t_p, (size_t)*rows_p);
+    ENTER(w, x, gs_ptr, y, k_dim_p, rows_p, t_p);
+    gemv_tokens(w, x, gs_ptr, y, *k_dim_p, *rows_p, *t_p, (size_t)*rows_p, ws);
 }
 extern "C" __global__ void __launch_bounds__(1024) gemv_fp4_bs(const unsigned char* __restrict__ w, const float* __restrict__ x,
                                                                const float* __restrict__ gs_ptr, float* __restrict__ y,
                                                                const int* __restrict__ k_dim_p, const int* __restrict__ y_stride_p,
                                                                const int* __restrict__ rows_p, const int* __restrict__ t_p) {
-    gemv_tokens(w, x, gs_ptr, y, *k_dim_p, *rows_p, *t_p, (size_t)*y_stride_p);
+    ENTER(w, x, gs_ptr, y, k_dim_p, y_stride_p, rows_p, t_p);
+    gemv_tokens(w, x, gs_ptr, y, *k_dim_p, *rows_p, *t_p, (size_t)*y_stride_p, ws);
 }
 
 // ------------------------------------------------------------------ routed experts
@@ -146,10 +164,11 @@ extern "C" __global__ void __launch_bounds__(1024) gemv_fp4_ptrb(const unsigned 
                                                                  const float* __restrict__ gs_ptr, float* __restrict__ y,
                                                                  const int* __restrict__ k_dim_p, const int* __restrict__ x_div_p,
                                                                  const int* __restrict__ x_stride_p, const int* __restrict__ rows_p) {
+    ENTER(ptrs, x, gs_ptr, y, k_dim_p, x_div_p, x_stride_p, rows_p);
     const int combo = (int)blockIdx.z, rows = *rows_p;
     const unsigned char* w = (const unsigned char*)ptrs[combo];
     GemvArgs a{{w, nullptr}, {gs_ptr, nullptr}, x + (size_t)(combo / *x_div_p) * *x_stride_p, 0, y + (size_t)combo * rows, 0, *k_dim_p, rows, 1, nullptr};
-    RED(1, 1); gemv_body<1, 1, false, EPI_SCALE, RED_N(1, 1)>(a, blockIdx.z, red);
+    RED(1, 1); gemv_body<1, 1, false, EPI_SCALE, RED_N(1, 1)>(a, blockIdx.z, red, ws);
 }
 // Fused routed gate|up + SwiGLU: the expert's fused tensor [2 I][H] holds gate in rows 0..I and up
 // in rows I..2I (converter/tests/fixtures/cnq45m-index.tsv:351); h[combo][I] = silu(gate x) * up x.
@@ -158,11 +177,12 @@ extern "C" __global__ void __launch_bounds__(1024) moe_gate_up_silu(const unsign
                                                                     const float* __restrict__ gs_ptr, float* __restrict__ h,
                                                                     const int* __restrict__ k_dim_p, const int* __restrict__ x_div_p,
                                                                     const int* __restrict__ x_stride_p, const int* __restrict__ inter_p) {
+    ENTER(ptrs, x, gs_ptr, h, k_dim_p, x_div_p, x_stride_p, inter_p);
     const int combo = (int)blockIdx.z, inter = *inter_p, k = *k_dim_p;
     const unsigned char* w = (const unsigned char*)ptrs[combo];
     const size_t up_off = (size_t)(inter / CROW_TILE_ROWS) * ((k + CROW_PANEL_COLS - 1) / CROW_PANEL_COLS) * CROW_TILE_BYTES;
     GemvArgs a{{w, w + up_off}, {gs_ptr, gs_ptr}, x + (size_t)(combo / *x_div_p) * *x_stride_p, 0, h + (size_t)combo * inter, 0, k, inter, 1, nullptr};
-    RED(2, 1); gemv_body<2, 1, false, EPI_SILU_GU, RED_N(2, 1)>(a, blockIdx.z, red);
+    RED(2, 1); gemv_body<2, 1, false, EPI_SILU_GU, RED_N(2, 1)>(a, blockIdx.z, red, ws);
 }
 
 // Fused routed down projection + weighted combine: y[t][row] += sum_j rw[t][j] * (gs * <down_{e(t,j)} row, h[t K + j]>),
@@ -174,7 +194,7 @@ extern "C" __global__ void __launch_bounds__(1024) moe_down_combine(const unsign
                                                                     float* __restrict__ y, const int* __restrict__ k_dim_p,
                                                                     const int* __restrict__ rows_p) {
     __shared__ float red[16 * 64];
-    const int k = *k_dim_p, rows = *rows_p, topk = (int)(blockDim.x >> 6);
+    const int k = *k_dim_p, rows = *rows_p, topk = block_threads() >> 6;
     if (topk != g_geo.topk || topk > 16) {
         if (threadIdx.x == 0) atomicOr(g_ws.status, STATUS_BAD_GEO);
         return;
