@@ -16,17 +16,20 @@ struct FnEntry {
     const char* name;
     const void* stub;
     int nargs;
+    unsigned lds_fixed, lds_per_wave;  // dynamic LDS of a launch = lds_fixed + lds_per_wave * (block size / 64)
 };
 
-#define CROW_FN(name, nargs) {#name, (const void*)&name, nargs}
+// GEMV blocks (gemv.h): 512 zero bytes, then per wave XR staging rows of 512 bytes and NR * M hand-over rows of 256
+#define CROW_FN(name, nargs) {#name, (const void*)&name, nargs, 0u, 0u}
+#define CROW_GEMV(name, nargs, NR, M, XR) {#name, (const void*)&name, nargs, 512u, (XR) * 512u + (NR) * (M) * 256u}
 const FnEntry g_table[] = {
-    CROW_FN(gemv_nvfp4_w, 6),      CROW_FN(gemv_nvfp4_w_bf16, 6),   CROW_FN(gemv_nvfp4_w_argmax, 7),
-    CROW_FN(gemv_nvfp4_gu, 8),     CROW_FN(gemv_nvfp4_wm, 7),       CROW_FN(gemv_nvfp4_gum, 9),
-    CROW_FN(gemv_nvfp4_wm_bf16, 7), CROW_FN(gemv_nvfp4_gum_bf16, 9), CROW_FN(gemv_fp4, 6),
-    CROW_FN(gemv_fp4_b, 7),        CROW_FN(gemv_fp4_b1k, 7),        CROW_FN(gemv_fp4_bs, 8),
-    CROW_FN(gemv_fp4_ptrb, 8),     CROW_FN(moe_gate_up_silu, 8),    CROW_FN(moe_down_combine, 7),
+    CROW_GEMV(gemv_nvfp4_w, 6, 1, 1, 3),       CROW_GEMV(gemv_nvfp4_w_bf16, 6, 1, 1, 1),  CROW_GEMV(gemv_nvfp4_w_argmax, 7, 1, 1, 3),
+    CROW_GEMV(gemv_nvfp4_gu, 8, 2, 1, 3),      CROW_GEMV(gemv_nvfp4_wm, 7, 1, 4, 12),     CROW_GEMV(gemv_nvfp4_gum, 9, 2, 4, 12),
+    CROW_GEMV(gemv_nvfp4_wm_bf16, 7, 1, 4, 4), CROW_GEMV(gemv_nvfp4_gum_bf16, 9, 2, 4, 4), CROW_GEMV(gemv_fp4, 6, 1, 1, 3),
+    CROW_GEMV(gemv_fp4_b, 7, 1, 4, 12),        CROW_GEMV(gemv_fp4_b1k, 7, 1, 4, 12),      CROW_GEMV(gemv_fp4_bs, 8, 1, 4, 12),
+    CROW_GEMV(gemv_fp4_ptrb, 8, 1, 1, 3),      CROW_GEMV(moe_gate_up_silu, 8, 2, 1, 3),   CROW_GEMV(moe_down_combine, 7, 1, 1, 3),
     CROW_FN(router_top10, 10),     CROW_FN(silu_mul_combo, 3),      CROW_FN(acc_combo, 3),
-    CROW_FN(argmax_k, 3),          CROW_FN(argmax_tiles, 2),          CROW_FN(dequant_fp4_flat, 4),    CROW_FN(repack_nvfp4, 4),
+    CROW_FN(argmax_k, 3),          CROW_FN(argmax_tiles, 2),        CROW_FN(dequant_fp4_flat, 4),    CROW_FN(repack_nvfp4, 4),
     CROW_FN(unpack_nvfp4, 4),      CROW_FN(dequant_nvfp4_tiled, 5), CROW_FN(gemm_nvfp4_bf16, 7),
     CROW_FN(gemm_nvfp4_bf16_m64, 7), CROW_FN(gemm_nvfp4_bf16_m32, 7),
 };
@@ -72,7 +75,8 @@ int launch_entry(const FnEntry* e, dim3 grid, dim3 block, const uint64_t* vals, 
     if (grid.x == 0 || grid.y == 0 || grid.z == 0 || block.x == 0 || block.x > 1024) return CROW_ERR_BAD_ARGUMENT;
     void* args[16];
     for (uint32_t i = 0; i < n; i++) args[i] = (void*)&vals[i];
-    return hip_rc(hipLaunchKernel(e->stub, grid, block, args, 0, s));
+    const size_t lds = e->lds_fixed + (size_t)e->lds_per_wave * (block.x / 64);
+    return hip_rc(hipLaunchKernel(e->stub, grid, block, args, lds, s));
 }
 
 }  // namespace
@@ -106,6 +110,13 @@ int crow_hip_init(int device) {
     if ((e = hipMemcpyToSymbol(HIP_SYMBOL(crow::g_ws), &ws, sizeof ws)) != hipSuccess) return (int)e;
     crow::Geo geo{0, 0, 0, 0};
     if ((e = hipMemcpyToSymbol(HIP_SYMBOL(crow::g_geo), &geo, sizeof geo)) != hipSuccess) return (int)e;
+    // a GEMV block of 16 waves may need more dynamic LDS than the default per-block limit
+    for (int i = 0; i < g_table_n; i++) {
+        const size_t most = g_table[i].lds_fixed + 16 * (size_t)g_table[i].lds_per_wave;
+        if (most > 48 * 1024 &&
+            (e = hipFuncSetAttribute(g_table[i].stub, hipFuncAttributeMaxDynamicSharedMemorySize, (int)most)) != hipSuccess)
+            return (int)e;
+    }
     if ((e = hipDeviceSynchronize()) != hipSuccess) return (int)e;
     g.ws = ws;
     g.device = device;

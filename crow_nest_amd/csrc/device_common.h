@@ -8,6 +8,10 @@ namespace crow {
 typedef float f32x2 __attribute__((ext_vector_type(2)));
 typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
 typedef unsigned stream_u32x4 __attribute__((ext_vector_type(4)));
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef unsigned u32x2 __attribute__((ext_vector_type(2)));
+typedef unsigned u32x4 __attribute__((ext_vector_type(4)));
 
 // blockDim.x read as a scalar from the kernel's implicit arguments (u16 group_size_x at byte 12 of the hidden block:
 // the compiler's own blockDim.x is a 16-bit VECTOR load followed by a wait, which sits in front of the first weight

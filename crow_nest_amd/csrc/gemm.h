@@ -1,37 +1,30 @@
-// NVFP4 x bf16 batched GEMM on the gfx950 matrix cores: Y[M][N] = X[M][K] W[N][K]^T, M >= 16 token rows.
+// NVFP4 x bf16 batched GEMM on the gfx950 matrix cores: Y[M][N] = X[M][K] W[N][K]^T, M > 4 token rows.
 //
 // The reference's prefill projection (engine/src/gen.rs:3922-3924 -> gemm_fp4_dense, engine/src/kernels.rs:
 // 533-751) quantises the activations to FP4 and runs Blackwell block-scaled MMA; its structural twin
 // glm5_gemm_fp4_tc (engine/src/kernels_glm5_moe.cu:349-449) decodes the weights losslessly to 16-bit
 // tiles and runs a plain tensor-core MMA with f32 accumulation and gs in the epilogue.  This kernel
 // is the CDNA4 form of the latter: weights decode to EXACT bf16 (e2m1 * ue4m3 has at most 6
-// significant bits), X is bf16, products are exact in f32, v_mfma_f32_32x32x16_bf16 accumulates.
+// significant bits), X is bf16, products are exact in f32, v_mfma_f32_16x16x32_bf16 accumulates.
 //
-// Data flow.  A block is 4 waves; wave w owns row tile 4 * blockIdx.x + w (64 weight rows) and all
-// of the block's MT = 32 * TB token rows.  Per 256-column panel:
-//   * every wave loads its own 9216-byte weight tile straight into registers (the GEMV's loads);
-//   * the block stages X[m0 .. m0 + MT][panel] into LDS (row stride 528 B: conflict-free b128 reads);
-//   * per 16-column sub-block the two code words a lane holds for ITS row are exchanged between the
-//     wave halves with v_permlane32_swap, which turns "lane = row, 16 columns" into the MFMA operand
-//     shape "lane % 32 = row, lane / 32 = which 8 columns" for rows 0..31 and rows 32..63 at once -
-//     on the 4-bit codes, before any decode; each half then decodes 8 values (cvt to f32, times the
-//     sub-block scale, keep the high 16 bits: exact) and feeds TB MFMAs per row half.
-// The weight rows ride on the MFMA's N side and the tokens on its M side, so a lane's 16 results
-// are 16 tokens of one weight row and every store instruction writes 128 contiguous bytes of Y.
+// Data flow.  A wave owns one 64-row weight tile per panel and MT = 16 * TBK token rows.  Per 256-column panel:
+//   * the wave loads its 9216-byte weight tile straight into registers (the GEMV's loads); every code dword
+//     is the B operand of one "unit" (16 weight rows x 32 columns, layout.h) as it stands;
+//   * X[m0 .. m0 + MT][panel] is staged in LDS (row stride 528 B) and read back as A operands, 16 token rows x
+//     32 columns per 16-byte-per-lane read, each used for the four row groups of the tile;
+//   * per unit a lane turns its 8 codes into 8 bf16 values times the sub-block scale (cvt to f32, multiply,
+//     keep the high 16 bits: exact) and feeds TBK matrix instructions.
+// The weight rows ride on the N side and the tokens on the M side, so a lane's 4 results of an instruction are
+// 4 tokens of one weight row and a store instruction writes four 64-byte runs of Y.
 #pragma once
 #include "device_common.h"
 
 namespace crow {
 
-typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
-typedef float f32x16 __attribute__((ext_vector_type(16)));
-typedef unsigned u32x2 __attribute__((ext_vector_type(2)));
-typedef unsigned u32x4 __attribute__((ext_vector_type(4)));
-
 #define CROW_GEMM_XS_STRIDE 264  // bf16 elements per staged X row (256 + 8 of padding)
 
 // 8 codes (one word) times a sub-block scale -> 8 exact bf16 values, as an MFMA operand
-__device__ __forceinline__ bf16x8 decode8_bf16(unsigned codes, float scale) {
+__device__ __forceinline__ bf16x8 decode8_scaled(unsigned codes, float scale) {
     const f32x2 a = fp4x2_to_f32<0>(codes), b = fp4x2_to_f32<1>(codes), c = fp4x2_to_f32<2>(codes), d = fp4x2_to_f32<3>(codes);
     u32x4 r;
     // byte selector 0x07060302: high halves of (hi, lo) -> {lo[31:16], hi[31:16]}
@@ -42,51 +35,82 @@ __device__ __forceinline__ bf16x8 decode8_bf16(unsigned codes, float scale) {
     return __builtin_bit_cast(bf16x8, r);
 }
 
-template <int SB>
-__device__ __forceinline__ float scale_byte(unsigned word) {
-    return e4m3_to_f32<SB & 3>(word);
-}
-
-// one 16-column sub-block SB (0..15) of the panel
-template <int TB, int SB>
-__device__ __forceinline__ void gemm_subblock(const uint4& cd, unsigned sc_lo, unsigned sc_hi, const __bf16* xs_lane,
-                                              f32x16 (&acc)[2][TB]) {
-    const unsigned d0 = (SB & 1) ? cd.z : cd.x, d1 = (SB & 1) ? cd.w : cd.y;
-    // after the swap: .x = codes of rows 0..31 (lanes 0..31: columns 0..7, lanes 32..63: columns 8..15),
-    //                 .y = the same for rows 32..63
-    const u32x2 sw = __builtin_amdgcn_permlane32_swap(d0, d1, false, false);
-    const bf16x8 w_lo = decode8_bf16(sw.x, scale_byte<SB>(sc_lo));
-    const bf16x8 w_hi = decode8_bf16(sw.y, scale_byte<SB>(sc_hi));
+// The tile's scale bytes as the GEMM needs them.  A lane (g, n) holds, for row groups j = 2 jp + (g & 1) only, the
+// scales of the sub-block half g >> 1 (layout.h); the other two row groups are in the neighbouring 16-lane group.
+// After the exchange `even` holds the words of the even group of each pair in both groups, `odd` those of the odd one.
+struct TileScales {
+    unsigned even[4], odd[4];
+    __device__ __forceinline__ void set(const uint4& sc) {
 #pragma unroll
-    for (int tb = 0; tb < TB; tb++) {
-        const bf16x8 xv = *(const bf16x8*)(xs_lane + tb * 32 * CROW_GEMM_XS_STRIDE + SB * 16);
-        acc[0][tb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(xv, w_lo, acc[0][tb], 0, 0, 0);
-        acc[1][tb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(xv, w_hi, acc[1][tb], 0, 0, 0);
+        for (int q = 0; q < 4; q++) {
+            const unsigned own = u4_get(sc, q);
+            const u32x2 sw = __builtin_amdgcn_permlane16_swap(own, own, false, false);
+            even[q] = sw.x;
+            odd[q] = sw.y;
+        }
+    }
+    // scale of this lane's operand of unit (row group J, segment S)
+    template <int S, int J>
+    __device__ __forceinline__ float get() const {
+        return e4m3_to_f32<S & 3>((J & 1) ? odd[2 * (J >> 1) + (S >> 2)] : even[2 * (J >> 1) + (S >> 2)]);
+    }
+};
+
+// one 32-column segment S of the panel: four units, TBK token blocks each
+template <int TBK, int S>
+__device__ __forceinline__ void gemm_segment(const uint4 (&cd)[CROW_STEPS], const TileScales& ts, const __bf16* xs_lane, f32x4 (&acc)[TBK][4]) {
+    bf16x8 A[TBK];
+#pragma unroll
+    for (int tb = 0; tb < TBK; tb++) A[tb] = *(const bf16x8*)(xs_lane + tb * 16 * CROW_GEMM_XS_STRIDE + S * 32);
+#define CROW_GEMM_UNIT(J)                                                                                      \
+    {                                                                                                          \
+        const bf16x8 B = decode8_scaled(u4_get(cd[S], J), ts.get<S, J>());                                     \
+        _Pragma("unroll") for (int tb = 0; tb < TBK; tb++)                                                     \
+            acc[tb][J] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(A[tb], B, acc[tb][J], 0, 0, 0);               \
+    }
+    CROW_GEMM_UNIT(0) CROW_GEMM_UNIT(1) CROW_GEMM_UNIT(2) CROW_GEMM_UNIT(3)
+#undef CROW_GEMM_UNIT
+}
+
+template <int TBK>
+__device__ __forceinline__ void gemm_panel(const uint4& sc, const uint4 (&cd)[CROW_STEPS], const __bf16* xs_lane, f32x4 (&acc)[TBK][4]) {
+    TileScales ts;
+    ts.set(sc);
+    gemm_segment<TBK, 0>(cd, ts, xs_lane, acc);
+    gemm_segment<TBK, 1>(cd, ts, xs_lane, acc);
+    gemm_segment<TBK, 2>(cd, ts, xs_lane, acc);
+    gemm_segment<TBK, 3>(cd, ts, xs_lane, acc);
+    gemm_segment<TBK, 4>(cd, ts, xs_lane, acc);
+    gemm_segment<TBK, 5>(cd, ts, xs_lane, acc);
+    gemm_segment<TBK, 6>(cd, ts, xs_lane, acc);
+    gemm_segment<TBK, 7>(cd, ts, xs_lane, acc);
+}
+
+// acc[tb][j][r] of lane (g, n): token m0 + 16 tb + 4 g + r, weight row 64 rt + 16 j + n
+template <int TBK>
+__device__ __forceinline__ void gemm_store(const f32x4 (&acc)[TBK][4], float gs, float* __restrict__ y, int rt, int m0, int rows, int m_total,
+                                           int lane) {
+    const int g = lane >> 4, n = lane & 15;
+#pragma unroll
+    for (int j = 0; j < 4; j++) {
+        const int col = rt * CROW_TILE_ROWS + 16 * j + n;
+        if (col >= rows) continue;
+#pragma unroll
+        for (int tb = 0; tb < TBK; tb++)
+#pragma unroll
+            for (int r = 0; r < 4; r++) {
+                const int m = m0 + 16 * tb + 4 * g + r;
+                if (m < m_total) y[(size_t)m * rows + col] = acc[tb][j][r] * gs;
+            }
     }
 }
 
-template <int TB, int SB>
-struct GemmPanel {
-    __device__ __forceinline__ static void run(const uint4 (&cd)[CROW_STEPS], const unsigned (&lo)[4], const unsigned (&hi)[4],
-                                               const __bf16* xs_lane, f32x16 (&acc)[2][TB]) {
-        gemm_subblock<TB, SB>(cd[SB >> 1], lo[SB >> 2], hi[SB >> 2], xs_lane, acc);
-        // keep sub-blocks in program order: a wave's decode then overlaps the OTHER resident waves' MFMAs,
-        // and the register count stays low enough for several waves per SIMD
-        __builtin_amdgcn_sched_barrier(0);
-        GemmPanel<TB, SB + 1>::run(cd, lo, hi, xs_lane, acc);
-    }
-};
-template <int TB>
-struct GemmPanel<TB, 16> {
-    __device__ __forceinline__ static void run(const uint4 (&)[CROW_STEPS], const unsigned (&)[4], const unsigned (&)[4], const __bf16*,
-                                               f32x16 (&)[2][TB]) {}
-};
-
-template <int TB>
+// Block = 4 waves; wave w owns row tile 4 * blockIdx.x + w and all of the block's MT = 16 * TBK token rows.
+template <int TBK>
 __device__ __forceinline__ void gemm_body(const unsigned char* __restrict__ w, const unsigned short* __restrict__ x,
                                           const float* __restrict__ gs_ptr, float* __restrict__ y, int k_dim, int rows, int m_total,
                                           __bf16* xs) {
-    constexpr int MT = 32 * TB;
+    constexpr int MT = 16 * TBK;
     const int lane = lane_id();
     const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
     const int row_tiles = (rows + CROW_TILE_ROWS - 1) / CROW_TILE_ROWS;
@@ -95,31 +119,25 @@ __device__ __forceinline__ void gemm_body(const unsigned char* __restrict__ w, c
     const int m0 = (int)blockIdx.y * MT;
     const int panels = (k_dim + CROW_PANEL_COLS - 1) / CROW_PANEL_COLS;
 
-    f32x16 acc[2][TB];
+    f32x4 acc[TBK][4];
 #pragma unroll
-    for (int h = 0; h < 2; h++)
+    for (int tb = 0; tb < TBK; tb++)
 #pragma unroll
-        for (int tb = 0; tb < TB; tb++)
-#pragma unroll
-            for (int i = 0; i < 16; i++) acc[h][tb][i] = 0.0f;
+        for (int j = 0; j < 4; j++) acc[tb][j] = f32x4{0.f, 0.f, 0.f, 0.f};
 
-    // this lane's fixed read position in the staged X tile: token lane % 32, columns 8 * (lane / 32) ..
-    const __bf16* xs_lane = xs + (lane & 31) * CROW_GEMM_XS_STRIDE + (lane >> 5) * 8;
-
-    // two register buffers for the weight tile: panel p + 1 is in flight while panel p is multiplied
-    uint4 scA = make_uint4(0, 0, 0, 0), cdA[CROW_STEPS], scB = make_uint4(0, 0, 0, 0), cdB[CROW_STEPS];
-#pragma unroll
-    for (int s = 0; s < CROW_STEPS; s++) cdA[s] = cdB[s] = make_uint4(0, 0, 0, 0);
+    // this lane's fixed read position in the staged X tile: token lane % 16, columns 8 * (lane / 16) .. of a segment
+    const __bf16* xs_lane = xs + (lane & 15) * CROW_GEMM_XS_STRIDE + (lane >> 4) * 8;
     const uint4* wt = (const uint4*)(w + (size_t)rt * panels * CROW_TILE_BYTES) + lane;
-    auto load_w = [&](int p, uint4& sc, uint4 (&cd)[CROW_STEPS]) {
-        if (has_rows && p < panels) {
+    for (int p = 0; p < panels; p++) {
+        uint4 sc = make_uint4(0, 0, 0, 0), cd[CROW_STEPS];
+#pragma unroll
+        for (int s = 0; s < CROW_STEPS; s++) cd[s] = make_uint4(0, 0, 0, 0);
+        if (has_rows) {
             const uint4* t = wt + (size_t)p * (CROW_TILE_BYTES / 16);
             sc = stream_load(t);
 #pragma unroll
             for (int s = 0; s < CROW_STEPS; s++) cd[s] = stream_load(t + 64 * (s + 1));
         }
-    };
-    auto stage_x = [&](int p) {
         // X[m0 .. m0 + MT][256 p .. 256 p + 255] (zero beyond M and K): MT * 32 chunks of 16 bytes
         __syncthreads();  // the previous panel's reads are done
         for (int c = (int)threadIdx.x; c < MT * 32; c += 256) {
@@ -130,52 +148,10 @@ __device__ __forceinline__ void gemm_body(const unsigned char* __restrict__ w, c
             *(uint4*)(xs + r * CROW_GEMM_XS_STRIDE + q * 8) = v;
         }
         __syncthreads();
-    };
-    auto multiply = [&](const uint4& sc, const uint4 (&cd)[CROW_STEPS]) {
-        // scale words of rows 0..31 / 32..63 in both wave halves
-        unsigned lo[4], hi[4];
-        const u32x2 a = __builtin_amdgcn_permlane32_swap(sc.x, sc.x, false, false);
-        const u32x2 b = __builtin_amdgcn_permlane32_swap(sc.y, sc.y, false, false);
-        const u32x2 c = __builtin_amdgcn_permlane32_swap(sc.z, sc.z, false, false);
-        const u32x2 d = __builtin_amdgcn_permlane32_swap(sc.w, sc.w, false, false);
-        lo[0] = a.x; lo[1] = b.x; lo[2] = c.x; lo[3] = d.x;
-        hi[0] = a.y; hi[1] = b.y; hi[2] = c.y; hi[3] = d.y;
-        GemmPanel<TB, 0>::run(cd, lo, hi, xs_lane, acc);
-    };
-    if (TB <= 2) {
-        load_w(0, scA, cdA);
-        for (int p = 0; p < panels; p += 2) {
-            stage_x(p);
-            load_w(p + 1, scB, cdB);
-            multiply(scA, cdA);
-            if (p + 1 >= panels) break;
-            stage_x(p + 1);
-            load_w(p + 2, scA, cdA);
-            multiply(scB, cdB);
-        }
-    } else {  // 128 tokens: the accumulators leave no room for a second weight buffer; two blocks per CU overlap instead
-        for (int p = 0; p < panels; p++) {
-            load_w(p, scA, cdA);
-            stage_x(p);
-            multiply(scA, cdA);
-        }
+        gemm_panel<TBK>(sc, cd, xs_lane, acc);
     }
     if (!has_rows) return;
-
-    // acc[h][tb][v]: token 32 tb + 8 (v / 4) + 4 (lane / 32) + v % 4, weight row 64 rt + 32 h + lane % 32
-    const float gs = gs_ptr[0];
-#pragma unroll
-    for (int h = 0; h < 2; h++) {
-        const int n = rt * CROW_TILE_ROWS + h * 32 + (lane & 31);
-        if (n >= rows) continue;
-#pragma unroll
-        for (int tb = 0; tb < TB; tb++)
-#pragma unroll
-            for (int v = 0; v < 16; v++) {
-                const int m = m0 + tb * 32 + 8 * (v >> 2) + 4 * (lane >> 5) + (v & 3);
-                if (m < m_total) y[(size_t)m * rows + n] = acc[h][tb][v] * gs;
-            }
-    }
+    gemm_store<TBK>(acc, gs_ptr[0], y, rt, m0, rows, m_total, lane);
 }
 
 // M <= 32 token rows: the product is bandwidth-bound and needs every CU streaming, so a block is ONE row
@@ -185,108 +161,82 @@ __device__ __forceinline__ void gemm_body(const unsigned char* __restrict__ w, c
 __device__ __forceinline__ void gemm_small_body(const unsigned char* __restrict__ w, const unsigned short* __restrict__ x,
                                                 const float* __restrict__ gs_ptr, float* __restrict__ y, int k_dim, int rows,
                                                 int m_total, __bf16* xs_all) {
+    constexpr int TBK = 2;
     const int lane = lane_id();
     const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
     const int rt = (int)blockIdx.x;
     const int panels = (k_dim + CROW_PANEL_COLS - 1) / CROW_PANEL_COLS;
     __bf16* xs = xs_all + wave * (32 * CROW_GEMM_XS_STRIDE);
-    const __bf16* xs_lane = xs + (lane & 31) * CROW_GEMM_XS_STRIDE + (lane >> 5) * 8;
+    const __bf16* xs_lane = xs + (lane & 15) * CROW_GEMM_XS_STRIDE + (lane >> 4) * 8;
 
-    f32x16 acc[2][1];
+    f32x4 acc[TBK][4];
 #pragma unroll
-    for (int h = 0; h < 2; h++)
+    for (int tb = 0; tb < TBK; tb++)
 #pragma unroll
-        for (int i = 0; i < 16; i++) acc[h][0][i] = 0.0f;
+        for (int j = 0; j < 4; j++) acc[tb][j] = f32x4{0.f, 0.f, 0.f, 0.f};
 
-    uint4 scA = make_uint4(0, 0, 0, 0), cdA[CROW_STEPS], scB = make_uint4(0, 0, 0, 0), cdB[CROW_STEPS];
-#pragma unroll
-    for (int s = 0; s < CROW_STEPS; s++) cdA[s] = cdB[s] = make_uint4(0, 0, 0, 0);
     const uint4* wt = (const uint4*)(w + (size_t)rt * panels * CROW_TILE_BYTES) + lane;
-    auto load_w = [&](int p, uint4& sc, uint4 (&cd)[CROW_STEPS]) {
-        if (p < panels) {
-            const uint4* t = wt + (size_t)p * (CROW_TILE_BYTES / 16);
-            sc = stream_load(t);
-#pragma unroll
-            for (int s = 0; s < CROW_STEPS; s++) cd[s] = stream_load(t + 64 * (s + 1));
-        }
-    };
-    auto stage_x = [&](int p) {  // 32 tokens x 256 columns = 1024 chunks of 16 bytes, 16 per lane; wave-private
+    for (int p = wave; p < panels; p += 4) {
+        // 32 tokens x 256 columns = 1024 chunks of 16 bytes, 16 per lane; wave-private.  Fetched before the weight
+        // loads are issued so that they do not queue behind them.
+        uint4 xv[16];
 #pragma unroll
         for (int i = 0; i < 16; i++) {
             const int c = i * 64 + lane, r = c >> 5, q = c & 31;
             const int k = p * CROW_PANEL_COLS + q * 8;
-            uint4 v = make_uint4(0, 0, 0, 0);
-            if (r < m_total && k < k_dim) v = *(const uint4*)(x + (size_t)r * k_dim + k);
-            *(uint4*)(xs + r * CROW_GEMM_XS_STRIDE + q * 8) = v;
+            xv[i] = make_uint4(0, 0, 0, 0);
+            if (r < m_total && k < k_dim) xv[i] = *(const uint4*)(x + (size_t)r * k_dim + k);
         }
-        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        uint4 sc, cd[CROW_STEPS];
+        const uint4* t = wt + (size_t)p * (CROW_TILE_BYTES / 16);
+        sc = stream_load(t);
+#pragma unroll
+        for (int s = 0; s < CROW_STEPS; s++) cd[s] = stream_load(t + 64 * (s + 1));
+#pragma unroll
+        for (int i = 0; i < 16; i++) {
+            const int c = i * 64 + lane, r = c >> 5, q = c & 31;
+            *(uint4*)(xs + r * CROW_GEMM_XS_STRIDE + q * 8) = xv[i];
+        }
         __builtin_amdgcn_wave_barrier();
-        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-    };
-    auto multiply = [&](const uint4& sc, const uint4 (&cd)[CROW_STEPS]) {
-        unsigned lo[4], hi[4];
-        const u32x2 a = __builtin_amdgcn_permlane32_swap(sc.x, sc.x, false, false);
-        const u32x2 b = __builtin_amdgcn_permlane32_swap(sc.y, sc.y, false, false);
-        const u32x2 c = __builtin_amdgcn_permlane32_swap(sc.z, sc.z, false, false);
-        const u32x2 d = __builtin_amdgcn_permlane32_swap(sc.w, sc.w, false, false);
-        lo[0] = a.x; lo[1] = b.x; lo[2] = c.x; lo[3] = d.x;
-        hi[0] = a.y; hi[1] = b.y; hi[2] = c.y; hi[3] = d.y;
-        GemmPanel<1, 0>::run(cd, lo, hi, xs_lane, acc);
-        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");  // the tile is read before the next stage overwrites it
-        __builtin_amdgcn_wave_barrier();
-    };
-    load_w(wave, scA, cdA);
-    for (int p = wave; p < panels; p += 8) {
-        stage_x(p);
-        load_w(p + 4, scB, cdB);
-        multiply(scA, cdA);
-        if (p + 4 >= panels) break;
-        stage_x(p + 4);
-        load_w(p + 8, scA, cdA);
-        multiply(scB, cdB);
+        gemm_panel<TBK>(sc, cd, xs_lane, acc);
+        __builtin_amdgcn_wave_barrier();  // the tile is read before the next stage overwrites it
     }
     // waves 1..3 -> wave 0 through LDS (each wave's own region is free now), added in wave order
     float* red = (float*)xs;
     if (wave > 0) {
 #pragma unroll
-        for (int h = 0; h < 2; h++)
+        for (int tb = 0; tb < TBK; tb++)
 #pragma unroll
-            for (int v = 0; v < 16; v++) red[(h * 16 + v) * 64 + lane] = acc[h][0][v];
+            for (int j = 0; j < 4; j++)
+#pragma unroll
+                for (int r = 0; r < 4; r++) red[((tb * 4 + j) * 4 + r) * 64 + lane] = acc[tb][j][r];
     }
     __syncthreads();
     if (wave > 0) return;
     for (int ww = 1; ww < 4; ww++) {
         const float* q = (const float*)(xs_all + ww * (32 * CROW_GEMM_XS_STRIDE));
 #pragma unroll
-        for (int h = 0; h < 2; h++)
+        for (int tb = 0; tb < TBK; tb++)
 #pragma unroll
-            for (int v = 0; v < 16; v++) acc[h][0][v] += q[(h * 16 + v) * 64 + lane];
+            for (int j = 0; j < 4; j++)
+#pragma unroll
+                for (int r = 0; r < 4; r++) acc[tb][j][r] += q[((tb * 4 + j) * 4 + r) * 64 + lane];
     }
-    const float gs = gs_ptr[0];
-#pragma unroll
-    for (int h = 0; h < 2; h++) {
-        const int n = rt * CROW_TILE_ROWS + h * 32 + (lane & 31);
-        if (n >= rows) continue;
-#pragma unroll
-        for (int v = 0; v < 16; v++) {
-            const int m = 8 * (v >> 2) + 4 * (lane >> 5) + (v & 3);
-            if (m < m_total) y[(size_t)m * rows + n] = acc[h][0][v] * gs;
-        }
-    }
+    gemm_store<TBK>(acc, gs_ptr[0], y, rt, 0, rows, m_total, lane);
 }
 
 }  // namespace crow
 
 // Y[M][rows] f32 = X[M][k_dim] bf16 times the tiled NVFP4 tensor, times gs.  The argument list is
 // gemm_fp4_dense's (engine/src/kernels.rs:533-541) without the quantised-activation buffer: x is bf16.
-// grid (ceil(row_tiles / 4), ceil(M / MT)), block 256, MT = 32 / 64 / 128 for the three entry points.
-#define CROW_GEMM_ENTRY(NAME, TB)                                                                                             \
-    extern "C" __global__ void __launch_bounds__(256, 2) NAME(const unsigned char* __restrict__ w, const unsigned short* __restrict__ x, \
+// grid (ceil(row_tiles / 4), ceil(M / MT)), block 256, MT = 64 / 128 for the two general entry points.
+#define CROW_GEMM_ENTRY(NAME, TBK, OCC)                                                                                       \
+    extern "C" __global__ void __launch_bounds__(256, OCC) NAME(const unsigned char* __restrict__ w, const unsigned short* __restrict__ x, \
                                                            const float* __restrict__ gs_ptr, float* __restrict__ y,            \
                                                            const int* __restrict__ k_dim_p, const int* __restrict__ rows_p,    \
                                                            const int* __restrict__ m_p) {                                      \
-        __shared__ __attribute__((aligned(16))) __bf16 xs[32 * TB * CROW_GEMM_XS_STRIDE];                                      \
-        crow::gemm_body<TB>(w, x, gs_ptr, y, *k_dim_p, *rows_p, *m_p, xs);                                                     \
+        __shared__ __attribute__((aligned(16))) __bf16 xs[16 * TBK * CROW_GEMM_XS_STRIDE];                                     \
+        crow::gemm_body<TBK>(w, x, gs_ptr, y, *k_dim_p, *rows_p, *m_p, xs);                                                    \
     }
 // M <= 32: grid (row_tiles), block 256
 extern "C" __global__ void __launch_bounds__(256, 2) gemm_nvfp4_bf16_m32(const unsigned char* __restrict__ w, const unsigned short* __restrict__ x,
@@ -296,5 +246,5 @@ extern "C" __global__ void __launch_bounds__(256, 2) gemm_nvfp4_bf16_m32(const u
     __shared__ __attribute__((aligned(16))) __bf16 xs[4 * 32 * CROW_GEMM_XS_STRIDE];
     crow::gemm_small_body(w, x, gs_ptr, y, *k_dim_p, *rows_p, *m_p, xs);
 }
-CROW_GEMM_ENTRY(gemm_nvfp4_bf16_m64, 2)
-CROW_GEMM_ENTRY(gemm_nvfp4_bf16, 4)
+CROW_GEMM_ENTRY(gemm_nvfp4_bf16_m64, 4, 3)
+CROW_GEMM_ENTRY(gemm_nvfp4_bf16, 8, 2)

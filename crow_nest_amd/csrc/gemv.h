@@ -1,24 +1,46 @@
 // NVFP4 GEMV family for gfx950: y[m][row] = gs * sum_k W[row][k] * x[m][k], M <= 4 activation rows.
 //
-// Mapping.  One wavefront owns one 64-row tile: lane l computes row l.  All lanes of a wave walk
-// the same columns, so the activation is wave-uniform and is read through scalar loads into
-// SGPRs; the FMA takes it as its scalar operand and nothing is ever shuffled between lanes.
-// Weights are read exactly once, as 16-byte-per-lane loads that cover 1024 contiguous bytes per
-// instruction (layout.h).  E2M1 pairs decode with v_cvt_scalef32_pk_f32_fp4 (exact), UE4M3 scales
-// with v_cvt_f32_fp8 (exact on canonical bytes).
+// Mapping.  One wavefront owns one 64-row x 256-column tile at a time and multiplies it on the matrix
+// cores: v_mfma_f32_16x16x32_bf16 with the WEIGHT rows on the N side (16 rows per instruction), 32
+// columns on the K side and the activation rows on the M side.  The weights are read exactly once,
+// as 16-byte-per-lane non-temporal loads that cover 1024 contiguous bytes per instruction, and every
+// dword a lane loads is its B operand as it stands (layout.h): eight E2M1 codes become eight exact
+// bf16 values with four v_cvt_scalef32_pk_bf16_fp4.  The per-16-column UE4M3 scale is NOT multiplied
+// into the weights.  Instead the two 16-column halves of a 32-column segment are kept apart on the M
+// side - an activation row occupies one operand row that is zero for K >= 16 and another that is zero
+// for K < 16 - so that every lane receives, per matrix instruction pair, the unscaled dot product of
+// ITS weight row with ONE 16-column sub-block, and applies that sub-block's scale with a single FMA:
+//
+//   A1 operand rows 0..3 : r-th activation row, columns  0..15 of the segment   (lane group g = 0 of D)
+//   A2 operand rows 4..7 : r-th activation row, columns  0..15                  (g = 1)
+//   A1 operand rows 8..11: r-th activation row, columns 16..31                  (g = 2)
+//   A2 operand rows 12..15: r-th activation row, columns 16..31                 (g = 3)
+//   D = A1 * B(row group 2 jp) ; D = A2 * B(row group 2 jp + 1) + D
+//   acc[jp][r] = fma(D[r], ue4m3(scale of this lane's row and sub-block), acc[jp][r])
+//
+// so one FMA per activation row serves two matrix instructions (1024 weights), and the decode costs
+// half an instruction per weight.  bf16 activations ride as they are (r = token).  f32 activations are
+// split exactly into three bf16 terms (x = hi + mid + lo, 8 + 8 + 8 significant bits by truncation);
+// the three terms of ONE token are the rows r = 0..2 of a matrix instruction pair and their results are
+// added as (hi + mid) + lo before the scale FMA: every product w * term is exact in f32, so the only
+// roundings are the f32 additions, as in any f32 dot product.
+//
+// Each wave stages its own activation slice (M rows x 256 columns, 512 bytes per bf16 row) in LDS and
+// reads its A operands from there with one 16-byte read per lane; lanes whose operand row is zero read
+// a zeroed 512-byte area instead.
 //
 // FP32 accumulation order (per output row and activation row), documented because it differs
 // from the reference CPU path's 8-lane order (cpu_nvfp4.rs:22-31) and from its GPU kernel of
 // record (kernels_p2.rs:304-347); all three are within the same gamma bound of the exact sum:
-//   for each 16-value sub-block, in column order:
-//       part = fma(w15, x15, ... fma(w1, x1, w0 * x0))        (w exact, 16 fused steps)
-//       acc  = fma(part, ue4m3(scale), acc)
+//   for each 16-value sub-block: part = the matrix core's f32 sum of the 16 exact products
+//       (f32 activations: ((part_hi + part_mid) + part_lo))
+//   even and odd sub-blocks of the wave's panels accumulate separately, in column order:
+//       acc = fma(part, ue4m3(scale), acc);   then acc_even + acc_odd
 //   a row split over S blocks of W waves: unit u = slice * W + wave owns panels u, u + S W, ...;
-//   a block adds its waves' `acc` values in wave order, then the blocks' sums are added in
-//   slice order (slice 0 first)
+//   a block adds its waves' sums in wave order, then the blocks' sums are added in slice order
 //   y = acc * gs                                               (gs last, as kernels_p2.rs:367)
-// The order depends only on (K, slices), never on M: row m of an M-row launch is bit-identical to
-// a one-row launch with the same slicing (the verify contract of kernels_p2.rs:391-396).
+// The order depends only on (K, slices), never on M or on the row's position: row m of an M-row launch
+// is bit-identical to a one-row launch with the same slicing (the verify contract of kernels_p2.rs:391-396).
 //
 // Launch geometry: grid (S, row_tiles, Z), block 64 * W.  blockIdx.y = row tile, blockIdx.x = column
 // slice, blockIdx.z = token group / expert combo.  The W waves of a block and the S blocks of a row
@@ -29,6 +51,11 @@
 // block stores its partial sums, bumps the tile's arrival counter, and the block that arrives
 // last adds all partials in slice order and writes y - deterministic whatever the arrival order.
 // With S = 1 the workspace is not touched.
+//
+// Dynamic LDS of a block (bytes; the launcher sizes it from the block size):
+//   [0, 512)                                   zeros
+//   [512 + (wave * XR + r) * 512, + 512)       activation staging, XR rows per wave
+//   then (W - 1) * NR * M * 64 floats          wave hand-over
 #pragma once
 #include "device_common.h"
 
@@ -47,227 +74,29 @@ struct GemvArgs {
     int* argmax_out;     // not null: also write the greedy argmax of y row 0 (fused lm_head head)
 };
 
-// 16 consecutive activation values of row m, wave-uniform (scalar loads)
-template <bool XBF16>
-struct XChunk;
-template <>
-struct XChunk<false> {
-    float v[16];
-    __device__ __forceinline__ void load(const void* x, size_t off) {
-        const float* p = (const float*)x + off;
-#pragma unroll
-        for (int j = 0; j < 16; j++) v[j] = p[j];
-    }
+// staging rows per wave: one bf16 row per token, or three (hi, mid, lo) per f32 token
+template <int M, bool XBF16>
+struct XRows {
+    static constexpr int value = XBF16 ? M : 3 * M;
 };
-template <>
-struct XChunk<true> {
-    unsigned v[8];  // bf16 pairs
-    __device__ __forceinline__ void load(const void* x, size_t off) {
-        const unsigned* p = (const unsigned*)((const unsigned short*)x + off);
-#pragma unroll
-        for (int j = 0; j < 8; j++) v[j] = p[j];
-    }
-};
+#define CROW_GEMV_ZERO_BYTES 512
+#define CROW_GEMV_XROW_BYTES 512
 
-// one 16-value sub-block: two code words (w0: values 0..7, w1: values 8..15).  The chain is split
-// into its first link and the rest so that a caller can place other work between them.
-template <bool XBF16>
-__device__ __forceinline__ float dot_head(unsigned w0, const XChunk<XBF16>& x);
-template <bool XBF16>
-__device__ __forceinline__ float dot_tail(float part, unsigned w0, unsigned w1, const XChunk<XBF16>& x);
-
-template <>
-__device__ __forceinline__ float dot_head<false>(unsigned w0, const XChunk<false>& x) {
-    return fp4x2_to_f32<0>(w0).x * x.v[0];
+typedef __attribute__((address_space(3))) unsigned char* lds_p;
+__device__ __forceinline__ void lds_store16(lds_p p, unsigned a, unsigned b, unsigned c, unsigned d) {
+    *(__attribute__((address_space(3))) u32x4*)p = u32x4{a, b, c, d};
 }
-template <>
-__device__ __forceinline__ float dot_tail<false>(float part, unsigned w0, unsigned w1, const XChunk<false>& x) {
-    f32x2 a = fp4x2_to_f32<0>(w0), b = fp4x2_to_f32<1>(w0), c = fp4x2_to_f32<2>(w0), d = fp4x2_to_f32<3>(w0);
-    part = __builtin_fmaf(a.y, x.v[1], part);
-    part = __builtin_fmaf(b.x, x.v[2], part);
-    part = __builtin_fmaf(b.y, x.v[3], part);
-    part = __builtin_fmaf(c.x, x.v[4], part);
-    part = __builtin_fmaf(c.y, x.v[5], part);
-    part = __builtin_fmaf(d.x, x.v[6], part);
-    part = __builtin_fmaf(d.y, x.v[7], part);
-    a = fp4x2_to_f32<0>(w1), b = fp4x2_to_f32<1>(w1), c = fp4x2_to_f32<2>(w1), d = fp4x2_to_f32<3>(w1);
-    part = __builtin_fmaf(a.x, x.v[8], part);
-    part = __builtin_fmaf(a.y, x.v[9], part);
-    part = __builtin_fmaf(b.x, x.v[10], part);
-    part = __builtin_fmaf(b.y, x.v[11], part);
-    part = __builtin_fmaf(c.x, x.v[12], part);
-    part = __builtin_fmaf(c.y, x.v[13], part);
-    part = __builtin_fmaf(d.x, x.v[14], part);
-    part = __builtin_fmaf(d.y, x.v[15], part);
-    return part;
-}
+__device__ __forceinline__ void lds_store8(lds_p p, unsigned a, unsigned b) { *(__attribute__((address_space(3))) u32x2*)p = u32x2{a, b}; }
 
-// bf16 activations: both factors are bf16, every product is exact in f32 and the dot
-// instruction adds two of them per step (v_dot2c_f32_bf16)
-template <>
-__device__ __forceinline__ float dot_head<true>(unsigned w0, const XChunk<true>& x) {
-    return __builtin_amdgcn_fdot2_f32_bf16(fp4x2_to_bf16<0>(w0), __builtin_bit_cast(bf16x2, x.v[0]), 0.0f, false);
+// 8 codes (one dword) -> 8 exact bf16 values: a matrix-instruction operand
+__device__ __forceinline__ bf16x8 decode8(unsigned codes) {
+    u32x4 r;
+    r.x = __builtin_bit_cast(unsigned, fp4x2_to_bf16<0>(codes));
+    r.y = __builtin_bit_cast(unsigned, fp4x2_to_bf16<1>(codes));
+    r.z = __builtin_bit_cast(unsigned, fp4x2_to_bf16<2>(codes));
+    r.w = __builtin_bit_cast(unsigned, fp4x2_to_bf16<3>(codes));
+    return __builtin_bit_cast(bf16x8, r);
 }
-template <>
-__device__ __forceinline__ float dot_tail<true>(float part, unsigned w0, unsigned w1, const XChunk<true>& x) {
-    part = __builtin_amdgcn_fdot2_f32_bf16(fp4x2_to_bf16<1>(w0), __builtin_bit_cast(bf16x2, x.v[1]), part, false);
-    part = __builtin_amdgcn_fdot2_f32_bf16(fp4x2_to_bf16<2>(w0), __builtin_bit_cast(bf16x2, x.v[2]), part, false);
-    part = __builtin_amdgcn_fdot2_f32_bf16(fp4x2_to_bf16<3>(w0), __builtin_bit_cast(bf16x2, x.v[3]), part, false);
-    part = __builtin_amdgcn_fdot2_f32_bf16(fp4x2_to_bf16<0>(w1), __builtin_bit_cast(bf16x2, x.v[4]), part, false);
-    part = __builtin_amdgcn_fdot2_f32_bf16(fp4x2_to_bf16<1>(w1), __builtin_bit_cast(bf16x2, x.v[5]), part, false);
-    part = __builtin_amdgcn_fdot2_f32_bf16(fp4x2_to_bf16<2>(w1), __builtin_bit_cast(bf16x2, x.v[6]), part, false);
-    part = __builtin_amdgcn_fdot2_f32_bf16(fp4x2_to_bf16<3>(w1), __builtin_bit_cast(bf16x2, x.v[7]), part, false);
-    return part;
-}
-template <bool XBF16>
-__device__ __forceinline__ float subblock_dot(unsigned w0, unsigned w1, const XChunk<XBF16>& x) {
-    return dot_tail<XBF16>(dot_head<XBF16>(w0, x), w0, w1, x);
-}
-
-template <int I>
-__device__ __forceinline__ float scale_of(const uint4& sc) {  // sub-block I (0..15) of the panel
-    return e4m3_to_f32<I & 3>(u4_get(sc, I >> 2));
-}
-
-// One 32-column step S of a panel for NR tensors and M activation rows.
-template <int NR, int M, bool XBF16, int S>
-__device__ __forceinline__ void step(const uint4 (&sc)[NR], const uint4 (&cd)[NR], const void* x, size_t x_off,
-                                     size_t x_stride, int m_rows, float (&acc)[NR][M]) {
-#pragma unroll
-    for (int half = 0; half < 2; half++) {
-        XChunk<XBF16> xc[M];
-#pragma unroll
-        for (int m = 0; m < M; m++)
-            if (m < m_rows) xc[m].load(x, (size_t)m * x_stride + x_off + half * 16);
-#pragma unroll
-        for (int r = 0; r < NR; r++) {
-            const unsigned w0 = half ? cd[r].z : cd[r].x, w1 = half ? cd[r].w : cd[r].y;
-            const float sf = half ? scale_of<2 * S + 1>(sc[r]) : scale_of<2 * S>(sc[r]);
-#pragma unroll
-            for (int m = 0; m < M; m++)
-                if (m < m_rows) acc[r][m] = __builtin_fmaf(subblock_dot<XBF16>(w0, w1, xc[m]), sf, acc[r][m]);
-        }
-    }
-}
-
-template <int NR, int M, bool XBF16, int S>
-struct Steps {
-    __device__ __forceinline__ static void run(const uint4 (&sc)[NR], const uint4 (&cd)[NR][CROW_STEPS], const void* x,
-                                               size_t x_off, size_t x_stride, int m_rows, int nsteps,
-                                               float (&acc)[NR][M]) {
-        if (S < nsteps) {
-            uint4 c[NR];
-#pragma unroll
-            for (int r = 0; r < NR; r++) c[r] = cd[r][S];
-            step<NR, M, XBF16, S>(sc, c, x, x_off + S * CROW_STEP_COLS, x_stride, m_rows, acc);
-        }
-        Steps<NR, M, XBF16, S + 1>::run(sc, cd, x, x_off, x_stride, m_rows, nsteps, acc);
-    }
-    // a whole panel: no per-step test (see panel_full below)
-};
-template <int NR, int M, bool XBF16>
-struct Steps<NR, M, XBF16, CROW_STEPS> {
-    __device__ __forceinline__ static void run(const uint4 (&)[NR], const uint4 (&)[NR][CROW_STEPS], const void*, size_t,
-                                               size_t, int, int, float (&)[NR][M]) {}
-};
-
-// A whole 256-column panel with the activation chunks software-pipelined: the scalar loads of
-// sub-block H + 1 are issued before the arithmetic of sub-block H, so their latency is covered by
-// 16 * M fused multiply-adds instead of being waited for.
-template <int NR, int M, bool XBF16, int H>
-struct PanelFull {
-    __device__ __forceinline__ static void run(const uint4 (&sc)[NR], const uint4 (&cd)[NR][CROW_STEPS], const void* x, size_t x_off,
-                                               size_t x_stride, int m_rows, XChunk<XBF16> (&cur)[M], float (&acc)[NR][M]) {
-        // first link of every chain: this is where the wave waits for `cur`; only then are the
-        // next sub-block's scalar loads issued (scalar loads return out of order, so a wait covers
-        // everything outstanding - issued any earlier they would be waited for here as well)
-        float part[NR][M];
-#pragma unroll
-        for (int r = 0; r < NR; r++) {
-            const uint4& c = cd[r][H >> 1];
-#pragma unroll
-            for (int m = 0; m < M; m++)
-                if (m < m_rows) part[r][m] = dot_head<XBF16>((H & 1) ? c.z : c.x, cur[m]);
-        }
-        __builtin_amdgcn_sched_barrier(0);
-        XChunk<XBF16> nxt[M];
-        if (H + 1 < 2 * CROW_STEPS) {
-#pragma unroll
-            for (int m = 0; m < M; m++)
-                if (m < m_rows) nxt[m].load(x, (size_t)m * x_stride + x_off + (H + 1) * 16);
-        }
-        __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-        for (int r = 0; r < NR; r++) {
-            const uint4& c = cd[r][H >> 1];
-            const unsigned w0 = (H & 1) ? c.z : c.x, w1 = (H & 1) ? c.w : c.y;
-            const float sf = scale_of<H>(sc[r]);
-#pragma unroll
-            for (int m = 0; m < M; m++)
-                if (m < m_rows) acc[r][m] = __builtin_fmaf(dot_tail<XBF16>(part[r][m], w0, w1, cur[m]), sf, acc[r][m]);
-        }
-        PanelFull<NR, M, XBF16, H + 1>::run(sc, cd, x, x_off, x_stride, m_rows, nxt, acc);
-    }
-};
-template <int NR, int M, bool XBF16>
-struct PanelFull<NR, M, XBF16, 2 * CROW_STEPS> {
-    __device__ __forceinline__ static void run(const uint4 (&)[NR], const uint4 (&)[NR][CROW_STEPS], const void*, size_t, size_t, int,
-                                               XChunk<XBF16> (&)[M], float (&)[NR][M]) {}
-};
-
-// f32 activations with M >= 3 rows: two 16-value chunks per row (current + prefetched) would need 128
-// SGPRs, more than a wave has, and the compiler then parks them in VGPR lanes.  The same chains
-// are therefore fed in 8-value chunks (one code word): chunk C is word C & 3 of step C >> 2, i.e.
-// half C & 1 of sub-block C >> 1.  Operation order per row is unchanged (one 16-long chain per
-// sub-block), so the results are bit-identical to the 16-value form.
-struct XHalf {
-    float v[8];
-    __device__ __forceinline__ void load(const void* x, size_t off) {
-        const float* p = (const float*)x + off;
-#pragma unroll
-        for (int j = 0; j < 8; j++) v[j] = p[j];
-    }
-};
-template <int NR, int M, int C>
-struct PanelFullHalf {
-    __device__ __forceinline__ static void run(const uint4 (&sc)[NR], const uint4 (&cd)[NR][CROW_STEPS], const void* x, size_t x_off,
-                                               size_t x_stride, int m_rows, float (&part)[NR][M], float (&acc)[NR][M]) {
-        // no software prefetch here: M * 8 SGPRs per chunk is all the scalar file affords next to the
-        // addressing; 4 + 8 M instructions per chunk and several waves per SIMD cover the scalar-cache latency
-        XHalf cur[M];
-#pragma unroll
-        for (int m = 0; m < M; m++)
-            if (m < m_rows) cur[m].load(x, (size_t)m * x_stride + x_off + C * 8);
-#pragma unroll
-        for (int r = 0; r < NR; r++) {
-            const unsigned word = u4_get(cd[r][C >> 2], C & 3);
-            const f32x2 a = fp4x2_to_f32<0>(word), b = fp4x2_to_f32<1>(word), c = fp4x2_to_f32<2>(word), d = fp4x2_to_f32<3>(word);
-            const float sf = scale_of<(C >> 1)>(sc[r]);
-#pragma unroll
-            for (int m = 0; m < M; m++) {
-                if (m < m_rows) {
-                    float p = (C & 1) ? __builtin_fmaf(a.x, cur[m].v[0], part[r][m]) : a.x * cur[m].v[0];
-                    p = __builtin_fmaf(a.y, cur[m].v[1], p);
-                    p = __builtin_fmaf(b.x, cur[m].v[2], p);
-                    p = __builtin_fmaf(b.y, cur[m].v[3], p);
-                    p = __builtin_fmaf(c.x, cur[m].v[4], p);
-                    p = __builtin_fmaf(c.y, cur[m].v[5], p);
-                    p = __builtin_fmaf(d.x, cur[m].v[6], p);
-                    p = __builtin_fmaf(d.y, cur[m].v[7], p);
-                    part[r][m] = p;
-                    if (C & 1) acc[r][m] = __builtin_fmaf(p, sf, acc[r][m]);
-                }
-            }
-        }
-        __builtin_amdgcn_sched_barrier(0);
-        PanelFullHalf<NR, M, C + 1>::run(sc, cd, x, x_off, x_stride, m_rows, part, acc);
-    }
-};
-template <int NR, int M>
-struct PanelFullHalf<NR, M, 32> {
-    __device__ __forceinline__ static void run(const uint4 (&)[NR], const uint4 (&)[NR][CROW_STEPS], const void*, size_t, size_t, int,
-                                               float (&)[NR][M], float (&)[NR][M]) {}
-};
 
 template <int NR>
 __device__ __forceinline__ void load_tile(const unsigned char* const (&w)[2], int rt, int panels, int p, int lane,
@@ -281,23 +110,102 @@ __device__ __forceinline__ void load_tile(const unsigned char* const (&w)[2], in
     }
 }
 
-template <int NR, int M, bool XBF16>
-__device__ __forceinline__ void panel_compute(const uint4 (&sc)[NR], const uint4 (&cd)[NR][CROW_STEPS], int p, int k_dim,
-                                              const void* x, size_t x_stride, int m_rows, float (&acc)[NR][M]) {
-    const int left = (k_dim - p * CROW_PANEL_COLS) / CROW_STEP_COLS;
-    if (left >= CROW_STEPS && !XBF16 && M >= 3) {
-        float part[NR][M];
-        PanelFullHalf<NR, M, 0>::run(sc, cd, x, (size_t)p * CROW_PANEL_COLS, x_stride, m_rows, part, acc);
-    } else if (left >= CROW_STEPS) {
-        XChunk<XBF16> first[M];
+// The activation slice of one panel, fetched into registers (before the weight loads are issued, so that its
+// data does not queue behind them) and then written to the wave's LDS rows.
+template <int M, bool XBF16>
+struct XStage;
+template <int M>
+struct XStage<M, true> {
+    uint4 v[(M + 1) / 2];
+    __device__ __forceinline__ void fetch(const void* x, size_t x_stride, int col0, int k_dim, int m_rows, int lane) {
+        const int c = lane & 31, col = col0 + 8 * c;
 #pragma unroll
-        for (int m = 0; m < M; m++)
-            if (m < m_rows) first[m].load(x, (size_t)m * x_stride + (size_t)p * CROW_PANEL_COLS);
-        PanelFull<NR, M, XBF16, 0>::run(sc, cd, x, (size_t)p * CROW_PANEL_COLS, x_stride, m_rows, first, acc);
-    } else {
-        Steps<NR, M, XBF16, 0>::run(sc, cd, x, (size_t)p * CROW_PANEL_COLS, x_stride, m_rows, left, acc);
+        for (int t0 = 0; t0 < M; t0 += 2) {
+            const int tok = t0 + (lane >> 5);
+            v[t0 / 2] = make_uint4(0, 0, 0, 0);
+            if (tok < m_rows && col < k_dim) v[t0 / 2] = *(const uint4*)((const unsigned short*)x + (size_t)tok * x_stride + col);
+        }
     }
-}
+    __device__ __forceinline__ void store(lds_p xw, int lane) const {
+#pragma unroll
+        for (int t0 = 0; t0 < M; t0 += 2) {
+            const int tok = t0 + (lane >> 5);
+            if (tok < M) lds_store16(xw + tok * CROW_GEMV_XROW_BYTES + 16 * (lane & 31), v[t0 / 2].x, v[t0 / 2].y, v[t0 / 2].z, v[t0 / 2].w);
+        }
+    }
+};
+template <int M>
+struct XStage<M, false> {
+    float4 v[M];
+    __device__ __forceinline__ void fetch(const void* x, size_t x_stride, int col0, int k_dim, int m_rows, int lane) {
+        const int col = col0 + 4 * lane;
+#pragma unroll
+        for (int t = 0; t < M; t++) {
+            v[t] = make_float4(0.f, 0.f, 0.f, 0.f);
+            if (t < m_rows && col < k_dim) v[t] = *(const float4*)((const float*)x + (size_t)t * x_stride + col);
+        }
+    }
+    // x = hi + mid + lo exactly: each term keeps the next 8 significant bits (truncation; the subtractions are exact)
+    __device__ __forceinline__ static void split(float f, unsigned& hi, unsigned& mid, unsigned& lo) {
+        hi = __float_as_uint(f) & 0xffff0000u;
+        const float r1 = __fsub_rn(f, __uint_as_float(hi));
+        mid = __float_as_uint(r1) & 0xffff0000u;
+        const float r2 = __fsub_rn(r1, __uint_as_float(mid));
+        lo = __float_as_uint(r2) & 0xffff0000u;
+    }
+    __device__ __forceinline__ void store(lds_p xw, int lane) const {
+#pragma unroll
+        for (int t = 0; t < M; t++) {
+            unsigned h[4], m[4], l[4];
+            split(v[t].x, h[0], m[0], l[0]);
+            split(v[t].y, h[1], m[1], l[1]);
+            split(v[t].z, h[2], m[2], l[2]);
+            split(v[t].w, h[3], m[3], l[3]);
+            // bf16 pairs: high halves of (odd element, even element)
+            lds_p row = xw + (3 * t) * CROW_GEMV_XROW_BYTES + 8 * lane;
+            lds_store8(row, __builtin_amdgcn_perm(h[1], h[0], 0x07060302u), __builtin_amdgcn_perm(h[3], h[2], 0x07060302u));
+            lds_store8(row + CROW_GEMV_XROW_BYTES, __builtin_amdgcn_perm(m[1], m[0], 0x07060302u), __builtin_amdgcn_perm(m[3], m[2], 0x07060302u));
+            lds_store8(row + 2 * CROW_GEMV_XROW_BYTES, __builtin_amdgcn_perm(l[1], l[0], 0x07060302u), __builtin_amdgcn_perm(l[3], l[2], 0x07060302u));
+        }
+    }
+};
+
+// One 32-column segment S of a panel: 4 * NR units.  `a1`, `a2` are this lane's LDS addresses of its A1 / A2 operand
+// for segment 0 of set q (or of the zero area); `acc[r][jp][m]` as described at the top of the file.
+template <int NR, int M, bool XBF16, int S>
+struct Segment {
+    static constexpr int NSET = XBF16 ? 1 : M;
+    __device__ __forceinline__ static void run(const uint4 (&sc)[NR], const uint4 (&cd)[NR][CROW_STEPS], const lds_p (&a1)[NSET],
+                                               const lds_p (&a2)[NSET], float (&acc)[NR][2][M]) {
+        typedef __attribute__((address_space(3))) const u32x4* lds_v4;
+        bf16x8 A1[NSET], A2[NSET];
+#pragma unroll
+        for (int q = 0; q < NSET; q++) {
+            A1[q] = __builtin_bit_cast(bf16x8, *(lds_v4)(a1[q] + 64 * S));
+            A2[q] = __builtin_bit_cast(bf16x8, *(lds_v4)(a2[q] + 64 * S));
+        }
+#pragma unroll
+        for (int jp = 0; jp < 2; jp++) {
+#pragma unroll
+            for (int r = 0; r < NR; r++) {
+                const bf16x8 B0 = decode8(u4_get(cd[r][S], 2 * jp)), B1 = decode8(u4_get(cd[r][S], 2 * jp + 1));
+                const float sv = e4m3_to_f32<S & 3>(u4_get(sc[r], 2 * jp + (S >> 2)));
+#pragma unroll
+                for (int q = 0; q < NSET; q++) {
+                    const f32x4 z = {0.f, 0.f, 0.f, 0.f};
+                    f32x4 D = __builtin_amdgcn_mfma_f32_16x16x32_bf16(A1[q], B0, z, 0, 0, 0);
+                    D = __builtin_amdgcn_mfma_f32_16x16x32_bf16(A2[q], B1, D, 0, 0, 0);
+                    if (XBF16) {
+#pragma unroll
+                        for (int m = 0; m < M; m++) acc[r][jp][m] = __builtin_fmaf(D[m], sv, acc[r][jp][m]);
+                    } else {
+                        acc[r][jp][q] = __builtin_fmaf(__fadd_rn(__fadd_rn(D[0], D[1]), D[2]), sv, acc[r][jp][q]);
+                    }
+                }
+            }
+        }
+    }
+};
 
 // Ordering point of the cross-block hand-over.  Every access to the shared partials and counters
 // is a device-scope atomic (store / load / add carry the device-coherence bits, so each one is
@@ -312,22 +220,64 @@ __device__ __forceinline__ void device_order() {
     asm volatile("" ::: "memory");
 }
 
-// acc[r][m] = sum over panels p = p0, p0 + stride, ... of the 64-row tile `rt` of tensor r against
-// activation row m: the per-lane (= per-row) partial dot product of one wave.  One register buffer
-// per wave; loads and arithmetic of different waves overlap through occupancy (about 52 VGPRs).
+// out[r][m] in lane l = the wave's partial dot product of tile row l (of tensor r) with activation row m, summed
+// over panels p = p0, p0 + stride, ...  `xw` is the wave's own staging area, `zero` the block's zeroed 512 bytes.
 template <int NR, int M, bool XBF16>
-__device__ __forceinline__ void tile_accumulate(const unsigned char* const (&w)[2], int rt, int panels, int p0, int stride,
-                                                int k_dim, const void* x, size_t x_stride, int m_rows, float (&acc)[NR][M]) {
+__device__ __forceinline__ void tile_accumulate(const unsigned char* const (&w)[2], int rt, int panels, int p0, int stride, int k_dim,
+                                                const void* x, size_t x_stride, int m_rows, lds_p xw, lds_p zero, float (&out)[NR][M]) {
+    constexpr int NSET = XBF16 ? 1 : M;
+    constexpr int SET_ROWS = XBF16 ? M : 3;  // live operand rows of a set
     const int lane = lane_id();
+    // this lane as a holder of A operand row i = lane % 16, K group g = lane / 16 (K indices 8 g .. 8 g + 7)
+    const int g = lane >> 4, i = lane & 15, r4 = i & 3;
+    const bool live = ((g >> 1) == (i >> 3)) && r4 < SET_ROWS;  // the row's 16-column half is this K group's half
+    const bool second = ((i >> 2) & 1) != 0;                    // rows 4..7, 12..15 belong to A2
+    lds_p a1[NSET], a2[NSET];
+#pragma unroll
+    for (int q = 0; q < NSET; q++) {
+        lds_p data = xw + (q * SET_ROWS + r4) * CROW_GEMV_XROW_BYTES + 16 * g;
+        a1[q] = (live && !second) ? data : zero + 16 * g;
+        a2[q] = (live && second) ? data : zero + 16 * g;
+    }
+    float acc[NR][2][M];
 #pragma unroll
     for (int r = 0; r < NR; r++)
 #pragma unroll
-        for (int m = 0; m < M; m++) acc[r][m] = 0.0f;
+        for (int jp = 0; jp < 2; jp++)
+#pragma unroll
+            for (int m = 0; m < M; m++) acc[r][jp][m] = 0.0f;
     for (int p = p0; p < panels; p += stride) {
+        XStage<M, XBF16> xs;
+        xs.fetch(x, x_stride, p * CROW_PANEL_COLS, k_dim, m_rows, lane);
         uint4 sc[NR], cd[NR][CROW_STEPS];
         load_tile<NR>(w, rt, panels, p, lane, sc, cd);
-        panel_compute<NR, M, XBF16>(sc, cd, p, k_dim, x, x_stride, m_rows, acc);
+        xs.store(xw, lane);
+        __builtin_amdgcn_wave_barrier();  // the reads below follow the writes above in program order (same wave)
+        Segment<NR, M, XBF16, 0>::run(sc, cd, a1, a2, acc);
+        Segment<NR, M, XBF16, 1>::run(sc, cd, a1, a2, acc);
+        Segment<NR, M, XBF16, 2>::run(sc, cd, a1, a2, acc);
+        Segment<NR, M, XBF16, 3>::run(sc, cd, a1, a2, acc);
+        Segment<NR, M, XBF16, 4>::run(sc, cd, a1, a2, acc);
+        Segment<NR, M, XBF16, 5>::run(sc, cd, a1, a2, acc);
+        Segment<NR, M, XBF16, 6>::run(sc, cd, a1, a2, acc);
+        Segment<NR, M, XBF16, 7>::run(sc, cd, a1, a2, acc);
+        __builtin_amdgcn_wave_barrier();  // ... and the next panel's writes follow these reads
     }
+    // lane (g, n) holds row 16 (2 jp + (g & 1)) + n, sub-block parity g >> 1.  Even + odd sub-blocks (lanes l and l + 32),
+    // then rows 0..31 (jp = 0) stay in lanes 0..31 and rows 32..63 (jp = 1) move to lanes 32..63: lane = tile row.
+#pragma unroll
+    for (int r = 0; r < NR; r++)
+#pragma unroll
+        for (int m = 0; m < M; m++) {
+            float v[2];
+#pragma unroll
+            for (int jp = 0; jp < 2; jp++) {
+                const unsigned a = __float_as_uint(acc[r][jp][m]);
+                const u32x2 sw = __builtin_amdgcn_permlane32_swap(a, a, false, false);  // .x = lanes 0..31 everywhere, .y = 32..63
+                v[jp] = __fadd_rn(__uint_as_float(sw.x), __uint_as_float(sw.y));
+            }
+            out[r][m] = lane < 32 ? v[0] : v[1];
+        }
 }
 
 typedef __attribute__((address_space(1))) float* gfloat_p;
@@ -335,10 +285,11 @@ typedef __attribute__((address_space(1))) unsigned* guint_p;
 typedef __attribute__((address_space(1))) int* gint_p;
 
 // The body every GEMV entry point runs.  The caller has already offset the pointers in `a` for
-// its token group / combo `z`, which only indexes the workspace here.  `red` is the block's LDS
-// hand-over buffer of (W - 1) * NR * M * 64 floats (RED_FLOATS of them are there).
-template <int NR, int M, bool XBF16, int EPI, int RED_FLOATS>
-__device__ __forceinline__ void gemv_body(const GemvArgs& a, unsigned z, float* red, const Workspace& ws) {
+// its token group / combo `z`, which only indexes the workspace here.  `lds` is the block's dynamic
+// LDS, laid out as described at the top of the file for XR_ALLOC staging rows per wave.
+template <int NR, int M, bool XBF16, int EPI, int XR_ALLOC>
+__device__ __forceinline__ void gemv_body(const GemvArgs& a, unsigned z, lds_p lds, const Workspace& ws) {
+    static_assert(XRows<M, XBF16>::value <= XR_ALLOC, "staging rows");
     const int lane = lane_id();
     const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6)), waves = block_threads() >> 6;  // wave-uniform on purpose
     const int slice = (int)blockIdx.x, slices = (int)gridDim.x;
@@ -348,15 +299,19 @@ __device__ __forceinline__ void gemv_body(const GemvArgs& a, unsigned z, float* 
     const int m_rows = a.m < M ? a.m : M;
     const unsigned tile_id = z * (unsigned)row_tiles + (unsigned)rt;
 
+    lds_p zero = lds;
+    lds_p xw = lds + CROW_GEMV_ZERO_BYTES + wave * (XR_ALLOC * CROW_GEMV_XROW_BYTES);
+    __attribute__((address_space(3))) float* red =
+        (__attribute__((address_space(3))) float*)(lds + CROW_GEMV_ZERO_BYTES + waves * (XR_ALLOC * CROW_GEMV_XROW_BYTES));
+    if (threadIdx.x < CROW_GEMV_ZERO_BYTES / 16) lds_store16(zero + 16 * threadIdx.x, 0, 0, 0, 0);
+    if (waves > 1) __syncthreads();
+    else __builtin_amdgcn_wave_barrier();
+
     float acc[NR][M];
-    tile_accumulate<NR, M, XBF16>(a.w, rt, panels, slice * waves + wave, slices * waves, a.k_dim, a.x, a.x_stride, m_rows, acc);
+    tile_accumulate<NR, M, XBF16>(a.w, rt, panels, slice * waves + wave, slices * waves, a.k_dim, a.x, a.x_stride, m_rows, xw, zero, acc);
 
     // waves of the block -> wave 0, in wave order
     if (waves > 1) {
-        if ((waves - 1) * NR * M * 64 > RED_FLOATS) {  // uniform: the launch does not fit this kernel
-            if (threadIdx.x == 0) atomicOr(ws.status, STATUS_BAD_SHAPE);
-            return;
-        }
         if (wave > 0) {
 #pragma unroll
             for (int r = 0; r < NR; r++)

@@ -10,9 +10,9 @@
 
 using namespace crow;
 
-// LDS hand-over buffer of a GEMV block: up to 16 waves, NR tensors, M activation rows
-#define RED_N(NR, M) (15 * (NR) * (M) * 64)
-#define RED(NR, M) __shared__ float red[RED_N(NR, M)]
+// The block's dynamic LDS (zeros, activation staging, wave hand-over: gemv.h); the launcher sizes it.
+extern __shared__ uint4 crow_dyn_lds[];
+#define LDS ((lds_p)crow_dyn_lds)
 // First statement of every GEMV entry point: the workspace descriptor is fetched with the kernel arguments, in the
 // first scalar round trip.  Left alone the compiler issues it after the shape words behind k_dim_p / rows_p have
 // arrived, as a third dependent round trip in front of every wave's first weight load.
@@ -27,7 +27,7 @@ extern "C" __global__ void __launch_bounds__(1024) gemv_nvfp4_w(const unsigned c
                                                                 const int* __restrict__ k_dim_p, const int* __restrict__ rows_p) {
     ENTER(w, x, gs_ptr, y, k_dim_p, rows_p);
     GemvArgs a{{w, nullptr}, {gs_ptr, nullptr}, x, 0, y, 0, *k_dim_p, *rows_p, 1, nullptr};
-    RED(1, 1); gemv_body<1, 1, false, EPI_SCALE, RED_N(1, 1)>(a, 0, red, ws);
+    gemv_body<1, 1, false, EPI_SCALE, XRows<1, false>::value>(a, 0, LDS, ws);
 }
 // the same product on bf16 activations (exact widening; BASELINE configs quote X in bf16)
 extern "C" __global__ void __launch_bounds__(1024) gemv_nvfp4_w_bf16(const unsigned char* __restrict__ w, const unsigned short* __restrict__ x,
@@ -35,7 +35,7 @@ extern "C" __global__ void __launch_bounds__(1024) gemv_nvfp4_w_bf16(const unsig
                                                                      const int* __restrict__ k_dim_p, const int* __restrict__ rows_p) {
     ENTER(w, x, gs_ptr, y, k_dim_p, rows_p);
     GemvArgs a{{w, nullptr}, {gs_ptr, nullptr}, x, 0, y, 0, *k_dim_p, *rows_p, 1, nullptr};
-    RED(1, 1); gemv_body<1, 1, true, EPI_SCALE, RED_N(1, 1)>(a, 0, red, ws);
+    gemv_body<1, 1, true, EPI_SCALE, XRows<1, true>::value>(a, 0, LDS, ws);
 }
 // reference: gemv_fp4, engine/src/kernels.rs:118-151 (+ rows_p: the reference's grid.x is the row count)
 extern "C" __global__ void __launch_bounds__(1024) gemv_fp4(const unsigned char* __restrict__ w, const float* __restrict__ x,
@@ -43,7 +43,7 @@ extern "C" __global__ void __launch_bounds__(1024) gemv_fp4(const unsigned char*
                                                             const int* __restrict__ k_dim_p, const int* __restrict__ rows_p) {
     ENTER(w, x, gs_ptr, y, k_dim_p, rows_p);
     GemvArgs a{{w, nullptr}, {gs_ptr, nullptr}, x, 0, y, 0, *k_dim_p, *rows_p, 1, nullptr};
-    RED(1, 1); gemv_body<1, 1, false, EPI_SCALE, RED_N(1, 1)>(a, 0, red, ws);
+    gemv_body<1, 1, false, EPI_SCALE, XRows<1, false>::value>(a, 0, LDS, ws);
 }
 
 // lm_head with the first stage of the greedy argmax fused in: logits[rows], and one candidate per 64-row
@@ -57,7 +57,7 @@ extern "C" __global__ void __launch_bounds__(1024) gemv_nvfp4_w_argmax(const uns
                                                                        int* __restrict__ out_idx) {
     ENTER(w, x, gs_ptr, y, k_dim_p, rows_p, out_idx);
     GemvArgs a{{w, nullptr}, {gs_ptr, nullptr}, x, 0, y, 0, *k_dim_p, *rows_p, 1, out_idx};
-    RED(1, 1); gemv_body<1, 1, false, EPI_SCALE, RED_N(1, 1)>(a, 0, red, ws);
+    gemv_body<1, 1, false, EPI_SCALE, XRows<1, false>::value>(a, 0, LDS, ws);
 }
 
 // ------------------------------------------------------------------ fused gate/up + SiLU (decode)
@@ -68,18 +68,18 @@ extern "C" __global__ void __launch_bounds__(1024) gemv_nvfp4_gu(const unsigned 
                                                                  const int* __restrict__ k_dim_p, const int* __restrict__ rows_p) {
     ENTER(wg, wu, x, gs_g, gs_u, y, k_dim_p, rows_p);
     GemvArgs a{{wg, wu}, {gs_g, gs_u}, x, 0, y, 0, *k_dim_p, *rows_p, 1, nullptr};
-    RED(2, 1); gemv_body<2, 1, false, EPI_SILU_GU, RED_N(2, 1)>(a, 0, red, ws);
+    gemv_body<2, 1, false, EPI_SILU_GU, XRows<1, false>::value>(a, 0, LDS, ws);
 }
 
 // ------------------------------------------------------------------ M <= 4 rows (MTP verify)
 template <int NR, bool XBF16, int EPI>
-__device__ __forceinline__ void gemv_m_dispatch(GemvArgs& a, unsigned z, float* red, const Workspace& ws) {
+__device__ __forceinline__ void gemv_m_dispatch(GemvArgs& a, unsigned z, lds_p lds, const Workspace& ws) {
     // one body per M keeps each row's operation sequence identical to the one-row kernel
     switch (a.m) {
-        case 1: gemv_body<NR, 1, XBF16, EPI, RED_N(NR, 4)>(a, z, red, ws); break;
-        case 2: gemv_body<NR, 2, XBF16, EPI, RED_N(NR, 4)>(a, z, red, ws); break;
-        case 3: gemv_body<NR, 3, XBF16, EPI, RED_N(NR, 4)>(a, z, red, ws); break;
-        default: gemv_body<NR, 4, XBF16, EPI, RED_N(NR, 4)>(a, z, red, ws); break;
+        case 1: gemv_body<NR, 1, XBF16, EPI, XRows<4, XBF16>::value>(a, z, lds, ws); break;
+        case 2: gemv_body<NR, 2, XBF16, EPI, XRows<4, XBF16>::value>(a, z, lds, ws); break;
+        case 3: gemv_body<NR, 3, XBF16, EPI, XRows<4, XBF16>::value>(a, z, lds, ws); break;
+        default: gemv_body<NR, 4, XBF16, EPI, XRows<4, XBF16>::value>(a, z, lds, ws); break;
     }
 }
 // reference: gemv_nvfp4_wm, engine/src/kernels_p2.rs:472-497
@@ -90,7 +90,7 @@ extern "C" __global__ void __launch_bounds__(1024) gemv_nvfp4_wm(const unsigned 
     ENTER(w, x, gs_ptr, y, k_dim_p, rows_p, m_p);
     const int k = *k_dim_p, rows = *rows_p;
     GemvArgs a{{w, nullptr}, {gs_ptr, nullptr}, x, (size_t)k, y, (size_t)rows, k, rows, *m_p, nullptr};
-    RED(1, 4); gemv_m_dispatch<1, false, EPI_SCALE>(a, 0, red, ws);
+    gemv_m_dispatch<1, false, EPI_SCALE>(a, 0, LDS, ws);
 }
 // reference: gemv_nvfp4_gum, engine/src/kernels_p2.rs:499-530
 extern "C" __global__ void __launch_bounds__(1024) gemv_nvfp4_gum(const unsigned char* __restrict__ wg, const unsigned char* __restrict__ wu,
@@ -101,7 +101,7 @@ extern "C" __global__ void __launch_bounds__(1024) gemv_nvfp4_gum(const unsigned
     ENTER(wg, wu, x, gs_g, gs_u, y, k_dim_p, rows_p, m_p);
     const int k = *k_dim_p, rows = *rows_p;
     GemvArgs a{{wg, wu}, {gs_g, gs_u}, x, (size_t)k, y, (size_t)rows, k, rows, *m_p, nullptr};
-    RED(2, 4); gemv_m_dispatch<2, false, EPI_SILU_GU>(a, 0, red, ws);
+    gemv_m_dispatch<2, false, EPI_SILU_GU>(a, 0, LDS, ws);
 }
 // bf16-activation twins of the two verify kernels (X [M][k_dim] bf16, outputs f32)
 extern "C" __global__ void __launch_bounds__(1024) gemv_nvfp4_wm_bf16(const unsigned char* __restrict__ w, const unsigned short* __restrict__ x,
@@ -111,7 +111,7 @@ extern "C" __global__ void __launch_bounds__(1024) gemv_nvfp4_wm_bf16(const unsi
     ENTER(w, x, gs_ptr, y, k_dim_p, rows_p, m_p);
     const int k = *k_dim_p, rows = *rows_p;
     GemvArgs a{{w, nullptr}, {gs_ptr, nullptr}, x, (size_t)k, y, (size_t)rows, k, rows, *m_p, nullptr};
-    RED(1, 4); gemv_m_dispatch<1, true, EPI_SCALE>(a, 0, red, ws);
+    gemv_m_dispatch<1, true, EPI_SCALE>(a, 0, LDS, ws);
 }
 extern "C" __global__ void __launch_bounds__(1024) gemv_nvfp4_gum_bf16(const unsigned char* __restrict__ wg, const unsigned char* __restrict__ wu,
                                                                        const unsigned short* __restrict__ x, const float* __restrict__ gs_g,
@@ -121,7 +121,7 @@ extern "C" __global__ void __launch_bounds__(1024) gemv_nvfp4_gum_bf16(const uns
     ENTER(wg, wu, x, gs_g, gs_u, y, k_dim_p, rows_p, m_p);
     const int k = *k_dim_p, rows = *rows_p;
     GemvArgs a{{wg, wu}, {gs_g, gs_u}, x, (size_t)k, y, (size_t)rows, k, rows, *m_p, nullptr};
-    RED(2, 4); gemv_m_dispatch<2, true, EPI_SILU_GU>(a, 0, red, ws);
+    gemv_m_dispatch<2, true, EPI_SILU_GU>(a, 0, LDS, ws);
 }
 
 // ------------------------------------------------------------------ batched over token rows
@@ -133,7 +133,7 @@ __device__ __forceinline__ void gemv_tokens(const unsigned char* w, const float*
     if (t0 >= t_total) return;
     GemvArgs a{{w, nullptr}, {gs, nullptr}, x + (size_t)t0 * k, (size_t)k, y + (size_t)t0 * y_stride, y_stride, k, rows,
                t_total - t0 < 4 ? t_total - t0 : 4, nullptr};
-    RED(1, 4); gemv_m_dispatch<1, false, EPI_SCALE>(a, blockIdx.z, red, ws);
+    gemv_m_dispatch<1, false, EPI_SCALE>(a, blockIdx.z, LDS, ws);
 }
 extern "C" __global__ void __launch_bounds__(1024) gemv_fp4_b(const unsigned char* __restrict__ w, const float* __restrict__ x,
                                                               const float* __restrict__ gs_ptr, float* __restrict__ y,
@@ -168,7 +168,7 @@ extern "C" __global__ void __launch_bounds__(1024) gemv_fp4_ptrb(const unsigned 
     const int combo = (int)blockIdx.z, rows = *rows_p;
     const unsigned char* w = (const unsigned char*)ptrs[combo];
     GemvArgs a{{w, nullptr}, {gs_ptr, nullptr}, x + (size_t)(combo / *x_div_p) * *x_stride_p, 0, y + (size_t)combo * rows, 0, *k_dim_p, rows, 1, nullptr};
-    RED(1, 1); gemv_body<1, 1, false, EPI_SCALE, RED_N(1, 1)>(a, blockIdx.z, red, ws);
+    gemv_body<1, 1, false, EPI_SCALE, XRows<1, false>::value>(a, blockIdx.z, LDS, ws);
 }
 // Fused routed gate|up + SwiGLU: the expert's fused tensor [2 I][H] holds gate in rows 0..I and up
 // in rows I..2I (converter/tests/fixtures/cnq45m-index.tsv:351); h[combo][I] = silu(gate x) * up x.
@@ -182,7 +182,7 @@ extern "C" __global__ void __launch_bounds__(1024) moe_gate_up_silu(const unsign
     const unsigned char* w = (const unsigned char*)ptrs[combo];
     const size_t up_off = (size_t)(inter / CROW_TILE_ROWS) * ((k + CROW_PANEL_COLS - 1) / CROW_PANEL_COLS) * CROW_TILE_BYTES;
     GemvArgs a{{w, w + up_off}, {gs_ptr, gs_ptr}, x + (size_t)(combo / *x_div_p) * *x_stride_p, 0, h + (size_t)combo * inter, 0, k, inter, 1, nullptr};
-    RED(2, 1); gemv_body<2, 1, false, EPI_SILU_GU, RED_N(2, 1)>(a, blockIdx.z, red, ws);
+    gemv_body<2, 1, false, EPI_SILU_GU, XRows<1, false>::value>(a, blockIdx.z, LDS, ws);
 }
 
 // Fused routed down projection + weighted combine: y[t][row] += sum_j rw[t][j] * (gs * <down_{e(t,j)} row, h[t K + j]>),
@@ -193,7 +193,6 @@ extern "C" __global__ void __launch_bounds__(1024) moe_down_combine(const unsign
                                                                     const float* __restrict__ gs_ptr, const float* __restrict__ rw,
                                                                     float* __restrict__ y, const int* __restrict__ k_dim_p,
                                                                     const int* __restrict__ rows_p) {
-    __shared__ float red[16 * 64];
     const int k = *k_dim_p, rows = *rows_p, topk = block_threads() >> 6;
     if (topk != g_geo.topk || topk > 16) {
         if (threadIdx.x == 0) atomicOr(g_ws.status, STATUS_BAD_GEO);
@@ -201,9 +200,15 @@ extern "C" __global__ void __launch_bounds__(1024) moe_down_combine(const unsign
     }
     const int t = (int)blockIdx.z, rt = (int)blockIdx.y, j = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6)), lane = lane_id();
     const int combo = t * topk + j;
+    // dynamic LDS: zeros, 3 staging rows per wave (f32 activations, one row), then one float per (wave, lane)
+    lds_p zero = LDS, xw = LDS + CROW_GEMV_ZERO_BYTES + j * (3 * CROW_GEMV_XROW_BYTES);
+    __attribute__((address_space(3))) float* red =
+        (__attribute__((address_space(3))) float*)(LDS + CROW_GEMV_ZERO_BYTES + topk * (3 * CROW_GEMV_XROW_BYTES));
+    if (threadIdx.x < CROW_GEMV_ZERO_BYTES / 16) lds_store16(zero + 16 * threadIdx.x, 0, 0, 0, 0);
+    __syncthreads();
     const unsigned char* const w[2] = {(const unsigned char*)ptrs[combo], nullptr};
     float acc[1][1];
-    tile_accumulate<1, 1, false>(w, rt, (k + CROW_PANEL_COLS - 1) / CROW_PANEL_COLS, 0, 1, k, h + (size_t)combo * k, 0, 1, acc);
+    tile_accumulate<1, 1, false>(w, rt, (k + CROW_PANEL_COLS - 1) / CROW_PANEL_COLS, 0, 1, k, h + (size_t)combo * k, 0, 1, xw, zero, acc);
     red[j * 64 + lane] = rw[combo] * (acc[0][0] * gs_ptr[0]);
     __syncthreads();
     const int row = rt * CROW_TILE_ROWS + lane;

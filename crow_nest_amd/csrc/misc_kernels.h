@@ -7,47 +7,37 @@ using namespace crow;
 #define CROW_STATUS_BAD_SCALE_BYTE 8u
 
 // ------------------------------------------------------------------ container <-> tiled
-// One 64-thread block per tile (blockIdx.x = panel, blockIdx.y = row tile); lane l moves row l.
-// Load-time work: the strided 36-byte reads are not coalesced and need not be.
+// One 64-thread block per tile (blockIdx.x = panel, blockIdx.y = row tile); thread l moves tile row l.
+// Load-time work: neither the strided 36-byte reads nor the scattered 4-byte tile writes are
+// coalesced, and they need not be.
 extern "C" __global__ void __launch_bounds__(64) repack_nvfp4(const unsigned char* __restrict__ src, unsigned char* __restrict__ dst,
                                                               const int* __restrict__ rows_p, const int* __restrict__ k_dim_p) {
     const int rows = *rows_p, k = *k_dim_p;
     const int panels = (k + CROW_PANEL_COLS - 1) / CROW_PANEL_COLS, bpr = k / CROW_BLOCK_VALUES;
     const int p = (int)blockIdx.x, rt = (int)blockIdx.y, lane = lane_id();
     const int row = rt * CROW_TILE_ROWS + lane;
-    unsigned sc[4] = {0, 0, 0, 0};
-    unsigned cd[CROW_STEPS][4];
-#pragma unroll
-    for (int s = 0; s < CROW_STEPS; s++) cd[s][0] = cd[s][1] = cd[s][2] = cd[s][3] = 0;
+    unsigned char* tile = dst + ((size_t)rt * panels + p) * CROW_TILE_BYTES;
     bool bad = false;
-    if (row < rows) {
 #pragma unroll
-        for (int b = 0; b < 4; b++) {
-            const int blk = p * 4 + b;
-            if (blk < bpr) {
-                const unsigned* q = (const unsigned*)(src + ((size_t)row * bpr + blk) * CROW_BLOCK_BYTES);
-                unsigned s4 = q[0], canon = 0;
+    for (int b = 0; b < 4; b++) {
+        const int blk = p * 4 + b;
+        unsigned q[9] = {0, 0, 0, 0, 0, 0, 0, 0, 0};
+        if (row < rows && blk < bpr) {
+            const unsigned* sq = (const unsigned*)(src + ((size_t)row * bpr + blk) * CROW_BLOCK_BYTES);
 #pragma unroll
-                for (int i = 0; i < 4; i++) {
-                    unsigned v = (s4 >> (8 * i)) & 0xFFu;
-                    if (v == 0xFFu) bad = true;
-                    v &= 0x7Fu;
-                    if (v == 0x7Fu) v = 0x7Eu;
-                    canon |= v << (8 * i);
-                }
-                sc[b] = canon;
-#pragma unroll
-                for (int j = 0; j < 4; j++) {
-                    cd[2 * b][j] = q[1 + j];
-                    cd[2 * b + 1][j] = q[5 + j];
-                }
-            }
+            for (int i = 0; i < 9; i++) q[i] = sq[i];
         }
-    }
-    uint4* t = (uint4*)(dst + ((size_t)rt * panels + p) * CROW_TILE_BYTES) + lane;
-    t[0] = make_uint4(sc[0], sc[1], sc[2], sc[3]);
 #pragma unroll
-    for (int s = 0; s < CROW_STEPS; s++) t[64 * (s + 1)] = make_uint4(cd[s][0], cd[s][1], cd[s][2], cd[s][3]);
+        for (int i = 0; i < 4; i++) {
+            unsigned v = (q[0] >> (8 * i)) & 0xFFu;
+            if (v == 0xFFu) bad = true;
+            v &= 0x7Fu;
+            if (v == 0x7Fu) v = 0x7Eu;
+            tile[crow_tile_scale_offset((unsigned)lane, (unsigned)(4 * b + i))] = (unsigned char)v;
+        }
+#pragma unroll
+        for (int wd = 0; wd < 8; wd++) *(unsigned*)(tile + crow_tile_code_offset((unsigned)lane, (unsigned)(8 * b + wd))) = q[1 + wd];
+    }
     if (bad) atomicOr(g_ws.status, CROW_STATUS_BAD_SCALE_BYTE);
 }
 
@@ -60,17 +50,18 @@ extern "C" __global__ void __launch_bounds__(64) unpack_nvfp4(const unsigned cha
     const int p = (int)blockIdx.x, rt = (int)blockIdx.y, lane = lane_id();
     const int row = rt * CROW_TILE_ROWS + lane;
     if (row >= rows) return;
-    const uint4* t = (const uint4*)(src + ((size_t)rt * panels + p) * CROW_TILE_BYTES) + lane;
-    const uint4 sc = t[0];
+    const unsigned char* tile = src + ((size_t)rt * panels + p) * CROW_TILE_BYTES;
 #pragma unroll
     for (int b = 0; b < 4; b++) {
         const int blk = p * 4 + b;
         if (blk < bpr) {
             unsigned* q = (unsigned*)(dst + ((size_t)row * bpr + blk) * CROW_BLOCK_BYTES);
-            q[0] = u4_get(sc, b);
-            const uint4 c0 = t[64 * (2 * b + 1)], c1 = t[64 * (2 * b + 2)];
-            q[1] = c0.x; q[2] = c0.y; q[3] = c0.z; q[4] = c0.w;
-            q[5] = c1.x; q[6] = c1.y; q[7] = c1.z; q[8] = c1.w;
+            unsigned s4 = 0;
+#pragma unroll
+            for (int i = 0; i < 4; i++) s4 |= (unsigned)tile[crow_tile_scale_offset((unsigned)lane, (unsigned)(4 * b + i))] << (8 * i);
+            q[0] = s4;
+#pragma unroll
+            for (int wd = 0; wd < 8; wd++) q[1 + wd] = *(const unsigned*)(tile + crow_tile_code_offset((unsigned)lane, (unsigned)(8 * b + wd)));
         }
     }
 }
@@ -87,24 +78,19 @@ extern "C" __global__ void __launch_bounds__(64) dequant_nvfp4_tiled(const unsig
     const int row = rt * CROW_TILE_ROWS + lane;
     if (row >= rows) return;
     const float gs = gs_ptr[0];
-    const uint4* t = (const uint4*)(w + ((size_t)rt * panels + p) * CROW_TILE_BYTES) + lane;
-    const uint4 sc = t[0];
-    for (int s = 0; s < CROW_STEPS; s++) {
-        const int col0 = p * CROW_PANEL_COLS + s * CROW_STEP_COLS;
+    const unsigned char* tile = w + ((size_t)rt * panels + p) * CROW_TILE_BYTES;
+    for (int sb = 0; sb < 16; sb++) {
+        const int col0 = p * CROW_PANEL_COLS + sb * 16;
         if (col0 >= k) break;
-        const uint4 c = t[64 * (s + 1)];
+        const unsigned byte = tile[crow_tile_scale_offset((unsigned)lane, (unsigned)sb)];
+        const float sf = __builtin_amdgcn_cvt_f32_fp8((int)byte, 0) * gs;
         float* o = out + (size_t)row * k + col0;
-        for (int h = 0; h < 2; h++) {
-            const int sb = 2 * s + h;
-            const unsigned byte = (u4_get(sc, sb >> 2) >> (8 * (sb & 3))) & 0xFFu;
-            const float sf = __builtin_amdgcn_cvt_f32_fp8((int)byte, 0) * gs;
-            for (int d = 0; d < 2; d++) {
-                const unsigned wd = u4_get(c, 2 * h + d);
-                for (int j = 0; j < 8; j++) {
-                    const unsigned nib = (wd >> (4 * j)) & 0xFu;
-                    const f32x2 v = __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(nib, 1.0f, 0);
-                    o[h * 16 + d * 8 + j] = v.x * sf;
-                }
+        for (int d = 0; d < 2; d++) {
+            const unsigned wd = *(const unsigned*)(tile + crow_tile_code_offset((unsigned)lane, (unsigned)(2 * sb + d)));
+            for (int j = 0; j < 8; j++) {
+                const unsigned nib = (wd >> (4 * j)) & 0xFu;
+                const f32x2 v = __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(nib, 1.0f, 0);
+                o[d * 8 + j] = v.x * sf;
             }
         }
     }
