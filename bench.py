@@ -116,9 +116,9 @@ def main() -> int:
     y = torch.empty(K, dtype=torch.float32, device=dev)
     gen_s = time.time() - t0
 
-    gu = Launch(eng, "gemv_nvfp4_gum_bf16", N, K, 1,
+    gu = Launch(eng, "gemv_nvfp4_gu_bf16", N, K, 1,
                 [[s["gate"].data_ptr(), s["up"].data_ptr(), xb.data_ptr(), base["gate"].gs_ptr, base["up"].gs_ptr, h.data_ptr(),
-                  p.i32(K), p.i32(N), p.i32(1)] for s in sets])
+                  p.i32(K), p.i32(N)] for s in sets])
     dn = Launch(eng, "gemv_nvfp4_w", K, N, 1,
                 [[s["down"].data_ptr(), h.data_ptr(), base["down"].gs_ptr, y.data_ptr(), p.i32(N), p.i32(K)] for s in sets])
 
@@ -160,7 +160,7 @@ def main() -> int:
     gu_us = gu.us()
     dn_us = dn.us()
     gu_bytes = alg_bytes_gate_up(1)
-    roof = {"bound": "hbm", "kernel": "gemv_nvfp4_gum_bf16", "achieved": round(gu_bytes / gu_us / 1e3, 1), "peak": PEAK_HBM_GBS,
+    roof = {"bound": "hbm", "kernel": "gemv_nvfp4_gu_bf16", "achieved": round(gu_bytes / gu_us / 1e3, 1), "peak": PEAK_HBM_GBS,
             "unit": "GB/s", "frac": round(gu_bytes / gu_us / 1e3 / PEAK_HBM_GBS, 4), "traffic": TRAFFIC_GATE_UP_M1,
             "us_per_launch": round(gu_us, 2), "algorithmic_bytes": gu_bytes, "grid": list(gu.dims)}
 

@@ -19,15 +19,17 @@ struct FnEntry {
     unsigned lds_fixed, lds_per_wave;  // dynamic LDS of a launch = lds_fixed + lds_per_wave * (block size / 64)
 };
 
-// GEMV blocks (gemv.h): 512 zero bytes, then per wave XR staging rows of 512 bytes and NR * M hand-over rows of 256
+// GEMV blocks (gemv.h): 512 zero bytes, then per wave XR staging rows of 576 bytes and NR * M hand-over rows of 256
+// (NR = 1 for the two-tensor kernels that run one tile per wave: gemv_nvfp4_gu, gemv_nvfp4_gu_bf16, moe_gate_up_silu)
 #define CROW_FN(name, nargs) {#name, (const void*)&name, nargs, 0u, 0u}
-#define CROW_GEMV(name, nargs, NR, M, XR) {#name, (const void*)&name, nargs, 512u, (XR) * 512u + (NR) * (M) * 256u}
+#define CROW_GEMV(name, nargs, NR, M, XR) {#name, (const void*)&name, nargs, 512u, (XR) * 576u + (NR) * (M) * 256u}
 const FnEntry g_table[] = {
     CROW_GEMV(gemv_nvfp4_w, 6, 1, 1, 3),       CROW_GEMV(gemv_nvfp4_w_bf16, 6, 1, 1, 1),  CROW_GEMV(gemv_nvfp4_w_argmax, 7, 1, 1, 3),
-    CROW_GEMV(gemv_nvfp4_gu, 8, 2, 1, 3),      CROW_GEMV(gemv_nvfp4_wm, 7, 1, 4, 12),     CROW_GEMV(gemv_nvfp4_gum, 9, 2, 4, 12),
+    CROW_GEMV(gemv_nvfp4_gu, 8, 1, 1, 3),      CROW_GEMV(gemv_nvfp4_gu_bf16, 8, 1, 1, 1),
+        CROW_GEMV(gemv_nvfp4_wm, 7, 1, 4, 12),     CROW_GEMV(gemv_nvfp4_gum, 9, 2, 4, 12),
     CROW_GEMV(gemv_nvfp4_wm_bf16, 7, 1, 4, 4), CROW_GEMV(gemv_nvfp4_gum_bf16, 9, 2, 4, 4), CROW_GEMV(gemv_fp4, 6, 1, 1, 3),
     CROW_GEMV(gemv_fp4_b, 7, 1, 4, 12),        CROW_GEMV(gemv_fp4_b1k, 7, 1, 4, 12),      CROW_GEMV(gemv_fp4_bs, 8, 1, 4, 12),
-    CROW_GEMV(gemv_fp4_ptrb, 8, 1, 1, 3),      CROW_GEMV(moe_gate_up_silu, 8, 2, 1, 3),   CROW_GEMV(moe_down_combine, 7, 1, 1, 3),
+    CROW_GEMV(gemv_fp4_ptrb, 8, 1, 1, 3),      CROW_GEMV(moe_gate_up_silu, 8, 1, 1, 3),   CROW_GEMV(moe_down_combine, 7, 1, 1, 3),
     CROW_FN(router_top10, 10),     CROW_FN(silu_mul_combo, 3),      CROW_FN(acc_combo, 3),
     CROW_FN(argmax_k, 3),          CROW_FN(argmax_tiles, 2),        CROW_FN(dequant_fp4_flat, 4),    CROW_FN(repack_nvfp4, 4),
     CROW_FN(unpack_nvfp4, 4),      CROW_FN(dequant_nvfp4_tiled, 5), CROW_FN(gemm_nvfp4_bf16, 7),
@@ -240,7 +242,10 @@ int crow_hip_launch_dims(const char* name, uint32_t rows, uint32_t k_dim, uint32
         const long force_s = env_long("CROW_GEMV_S", 0), force_w = env_long("CROW_GEMV_W", 0);
         if (force_s > 0) s = force_s;
         if (force_w > 0) w = force_w;
-        if (w > 16) w = 16;
+        // gate/up kernels for one activation row run one tile per wave: 2 W waves per block (W per tensor), at most 1024 threads
+        const bool thin = strcmp(name, "gemv_nvfp4_gu") == 0 || strcmp(name, "gemv_nvfp4_gu_bf16") == 0 || strcmp(name, "moe_gate_up_silu") == 0;
+        const bool half = thin || strcmp(name, "gemv_nvfp4_gum") == 0;  // (that one is built for blocks of at most 512 threads)
+        if (w > (half ? 8 : 16)) w = half ? 8 : 16;
         if (w < 1) w = 1;
         if (s < 1) s = 1;
         if (s * w > (long)panels) s = (panels + w - 1) / w;
@@ -248,7 +253,7 @@ int crow_hip_launch_dims(const char* name, uint32_t rows, uint32_t k_dim, uint32
         out->gx = (uint32_t)s;
         out->gy = tiles;
         out->gz = gz;
-        out->bx = (uint32_t)(64 * w);
+        out->bx = (uint32_t)(64 * w * (thin ? 2 : 1));
         const unsigned long long need = (unsigned long long)tiles * gz * s * nrm * 64;
         if (s > 1 && (need > PARTIAL_FLOATS || (unsigned long long)tiles * gz > COUNTER_SLOTS)) return CROW_ERR_WORKSPACE;
         if (strcmp(name, "gemv_nvfp4_w_argmax") == 0 && tiles > AM_SLOTS) return CROW_ERR_WORKSPACE;

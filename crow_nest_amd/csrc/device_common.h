@@ -25,7 +25,8 @@ __device__ __forceinline__ int block_threads() {
 // displacing reusable lines in L2 and the memory-side cache (measured on a pure read of the tile pattern:
 // 6.8-6.9 TB/s against 6.1-6.3 TB/s without the hint at 437 MB, 5.8 against 5.5 at 50 MB)
 __device__ __forceinline__ uint4 stream_load(const uint4* p) {
-    const stream_u32x4 v = __builtin_nontemporal_load((const stream_u32x4*)p);
+    // weights are device memory: the explicit address space keeps the load a global one when `p` comes out of a select
+    const stream_u32x4 v = __builtin_nontemporal_load((const __attribute__((address_space(1))) stream_u32x4*)p);
     return make_uint4(v.x, v.y, v.z, v.w);
 }
 

@@ -54,8 +54,8 @@
 //
 // Dynamic LDS of a block (bytes; the launcher sizes it from the block size):
 //   [0, 512)                                   zeros
-//   [512 + (wave * XR + r) * 512, + 512)       activation staging, XR rows per wave
-//   then (W - 1) * NR * M * 64 floats          wave hand-over
+//   [512 + (wave * XR + r) * 576, + 512)       activation staging, XR rows per wave (row stride 576)
+//   then (waves - 1) * NR * M * 64 floats      wave hand-over (one-tile-per-wave two-tensor kernels: waves = 2 W, NR -> 1)
 #pragma once
 #include "device_common.h"
 
@@ -80,7 +80,9 @@ struct XRows {
     static constexpr int value = XBF16 ? M : 3 * M;
 };
 #define CROW_GEMV_ZERO_BYTES 512
-#define CROW_GEMV_XROW_BYTES 512
+// 512 bytes of data per staged row; the 64 bytes of padding put four consecutive rows on four different groups of
+// 16 LDS banks, so that the operand reads of a set's rows do not collide
+#define CROW_GEMV_XROW_BYTES 576
 
 typedef __attribute__((address_space(3))) unsigned char* lds_p;
 __device__ __forceinline__ void lds_store16(lds_p p, unsigned a, unsigned b, unsigned c, unsigned d) {
@@ -175,14 +177,16 @@ struct XStage<M, false> {
 template <int NR, int M, bool XBF16, int S>
 struct Segment {
     static constexpr int NSET = XBF16 ? 1 : M;
-    __device__ __forceinline__ static void run(const uint4 (&sc)[NR], const uint4 (&cd)[NR][CROW_STEPS], const lds_p (&a1)[NSET],
-                                               const lds_p (&a2)[NSET], float (&acc)[NR][2][M]) {
+    // `a1`, `a2`: this lane's LDS address of its A1 / A2 operand of segment 0, set 0; set q is `step` bytes further
+    // (0 for a lane that reads the zero area)
+    __device__ __forceinline__ static void run(const uint4 (&sc)[NR], const uint4 (&cd)[NR][CROW_STEPS], lds_p a1, lds_p a2, int step1,
+                                               int step2, float (&acc)[NR][2][M]) {
         typedef __attribute__((address_space(3))) const u32x4* lds_v4;
         bf16x8 A1[NSET], A2[NSET];
 #pragma unroll
         for (int q = 0; q < NSET; q++) {
-            A1[q] = __builtin_bit_cast(bf16x8, *(lds_v4)(a1[q] + 64 * S));
-            A2[q] = __builtin_bit_cast(bf16x8, *(lds_v4)(a2[q] + 64 * S));
+            A1[q] = __builtin_bit_cast(bf16x8, *(lds_v4)(a1 + q * step1 + 64 * S));
+            A2[q] = __builtin_bit_cast(bf16x8, *(lds_v4)(a2 + q * step2 + 64 * S));
         }
 #pragma unroll
         for (int jp = 0; jp < 2; jp++) {
@@ -227,18 +231,16 @@ __device__ __forceinline__ void tile_accumulate(const unsigned char* const (&w)[
                                                 const void* x, size_t x_stride, int m_rows, lds_p xw, lds_p zero, float (&out)[NR][M]) {
     constexpr int NSET = XBF16 ? 1 : M;
     constexpr int SET_ROWS = XBF16 ? M : 3;  // live operand rows of a set
+    // register-hungry instantiations keep the segments apart: the next segment's operands are not fetched early
+    constexpr bool LEAN = NR * NSET >= 2 && !XBF16;
     const int lane = lane_id();
     // this lane as a holder of A operand row i = lane % 16, K group g = lane / 16 (K indices 8 g .. 8 g + 7)
     const int g = lane >> 4, i = lane & 15, r4 = i & 3;
     const bool live = ((g >> 1) == (i >> 3)) && r4 < SET_ROWS;  // the row's 16-column half is this K group's half
     const bool second = ((i >> 2) & 1) != 0;                    // rows 4..7, 12..15 belong to A2
-    lds_p a1[NSET], a2[NSET];
-#pragma unroll
-    for (int q = 0; q < NSET; q++) {
-        lds_p data = xw + (q * SET_ROWS + r4) * CROW_GEMV_XROW_BYTES + 16 * g;
-        a1[q] = (live && !second) ? data : zero + 16 * g;
-        a2[q] = (live && second) ? data : zero + 16 * g;
-    }
+    lds_p data = xw + r4 * CROW_GEMV_XROW_BYTES + 16 * g;
+    const lds_p a1 = (live && !second) ? data : zero + 16 * g, a2 = (live && second) ? data : zero + 16 * g;
+    const int step1 = (live && !second) ? SET_ROWS * CROW_GEMV_XROW_BYTES : 0, step2 = (live && second) ? SET_ROWS * CROW_GEMV_XROW_BYTES : 0;
     float acc[NR][2][M];
 #pragma unroll
     for (int r = 0; r < NR; r++)
@@ -253,14 +255,22 @@ __device__ __forceinline__ void tile_accumulate(const unsigned char* const (&w)[
         load_tile<NR>(w, rt, panels, p, lane, sc, cd);
         xs.store(xw, lane);
         __builtin_amdgcn_wave_barrier();  // the reads below follow the writes above in program order (same wave)
-        Segment<NR, M, XBF16, 0>::run(sc, cd, a1, a2, acc);
-        Segment<NR, M, XBF16, 1>::run(sc, cd, a1, a2, acc);
-        Segment<NR, M, XBF16, 2>::run(sc, cd, a1, a2, acc);
-        Segment<NR, M, XBF16, 3>::run(sc, cd, a1, a2, acc);
-        Segment<NR, M, XBF16, 4>::run(sc, cd, a1, a2, acc);
-        Segment<NR, M, XBF16, 5>::run(sc, cd, a1, a2, acc);
-        Segment<NR, M, XBF16, 6>::run(sc, cd, a1, a2, acc);
-        Segment<NR, M, XBF16, 7>::run(sc, cd, a1, a2, acc);
+        Segment<NR, M, XBF16, 0>::run(sc, cd, a1, a2, step1, step2, acc);
+        if (LEAN) __builtin_amdgcn_sched_barrier(0);
+        Segment<NR, M, XBF16, 1>::run(sc, cd, a1, a2, step1, step2, acc);
+        if (LEAN) __builtin_amdgcn_sched_barrier(0);
+        Segment<NR, M, XBF16, 2>::run(sc, cd, a1, a2, step1, step2, acc);
+        if (LEAN) __builtin_amdgcn_sched_barrier(0);
+        Segment<NR, M, XBF16, 3>::run(sc, cd, a1, a2, step1, step2, acc);
+        if (LEAN) __builtin_amdgcn_sched_barrier(0);
+        Segment<NR, M, XBF16, 4>::run(sc, cd, a1, a2, step1, step2, acc);
+        if (LEAN) __builtin_amdgcn_sched_barrier(0);
+        Segment<NR, M, XBF16, 5>::run(sc, cd, a1, a2, step1, step2, acc);
+        if (LEAN) __builtin_amdgcn_sched_barrier(0);
+        Segment<NR, M, XBF16, 6>::run(sc, cd, a1, a2, step1, step2, acc);
+        if (LEAN) __builtin_amdgcn_sched_barrier(0);
+        Segment<NR, M, XBF16, 7>::run(sc, cd, a1, a2, step1, step2, acc);
+        if (LEAN) __builtin_amdgcn_sched_barrier(0);
         __builtin_amdgcn_wave_barrier();  // ... and the next panel's writes follow these reads
     }
     // lane (g, n) holds row 16 (2 jp + (g & 1)) + n, sub-block parity g >> 1.  Even + odd sub-blocks (lanes l and l + 32),
@@ -287,7 +297,7 @@ typedef __attribute__((address_space(1))) int* gint_p;
 // The body every GEMV entry point runs.  The caller has already offset the pointers in `a` for
 // its token group / combo `z`, which only indexes the workspace here.  `lds` is the block's dynamic
 // LDS, laid out as described at the top of the file for XR_ALLOC staging rows per wave.
-template <int NR, int M, bool XBF16, int EPI, int XR_ALLOC>
+template <int NR, int M, bool XBF16, int EPI, int XR_ALLOC, bool THIN = false>
 __device__ __forceinline__ void gemv_body(const GemvArgs& a, unsigned z, lds_p lds, const Workspace& ws) {
     static_assert(XRows<M, XBF16>::value <= XR_ALLOC, "staging rows");
     const int lane = lane_id();
@@ -308,25 +318,58 @@ __device__ __forceinline__ void gemv_body(const GemvArgs& a, unsigned z, lds_p l
     else __builtin_amdgcn_wave_barrier();
 
     float acc[NR][M];
-    tile_accumulate<NR, M, XBF16>(a.w, rt, panels, slice * waves + wave, slices * waves, a.k_dim, a.x, a.x_stride, m_rows, xw, zero, acc);
-
-    // waves of the block -> wave 0, in wave order
-    if (waves > 1) {
+    if constexpr (THIN && NR == 2) {
+        // One tile per wave: the block runs 2 W waves, waves 0 .. W - 1 take the panels of tensor 0 and waves W .. 2 W - 1 the
+        // same panels of tensor 1.  This keeps the register count (and so the number of resident waves) of the
+        // one-tensor kernel; the arithmetic per row is that of the two-tiles-per-wave form.
+        const int wpt = waves >> 1;               // waves per tensor (W)
+        const int r_own = wave >= wpt ? 1 : 0;    // wave-uniform
+        const int pw = wave - r_own * wpt;
+        float part[1][M];
+        const unsigned char* const w_own[2] = {r_own != 0 ? a.w[1] : a.w[0], nullptr};  // a select, never an indexed read
+        tile_accumulate<1, M, XBF16>(w_own, rt, panels, slice * wpt + pw, slices * wpt, a.k_dim, a.x, a.x_stride, m_rows, xw, zero, part);
+        // waves of the block -> wave 0, per tensor in wave order
+#pragma unroll
+        for (int m = 0; m < M; m++) acc[0][m] = part[0][m];
         if (wave > 0) {
 #pragma unroll
-            for (int r = 0; r < NR; r++)
-#pragma unroll
-                for (int m = 0; m < M; m++)
-                    if (m < m_rows) red[((wave - 1) * NR * M + r * M + m) * 64 + lane] = acc[r][m];
+            for (int m = 0; m < M; m++)
+                if (m < m_rows) red[((wave - 1) * M + m) * 64 + lane] = part[0][m];
         }
         __syncthreads();
         if (wave > 0) return;
-        for (int w = 1; w < waves; w++) {
+        for (int w = 1; w < wpt; w++) {
 #pragma unroll
-            for (int r = 0; r < NR; r++)
+            for (int m = 0; m < M; m++)
+                if (m < m_rows) acc[0][m] += red[((w - 1) * M + m) * 64 + lane];
+        }
 #pragma unroll
-                for (int m = 0; m < M; m++)
-                    if (m < m_rows) acc[r][m] += red[((w - 1) * NR * M + r * M + m) * 64 + lane];
+        for (int m = 0; m < M; m++) acc[1][m] = m < m_rows ? red[((wpt - 1) * M + m) * 64 + lane] : 0.0f;
+        for (int w = wpt + 1; w < waves; w++) {
+#pragma unroll
+            for (int m = 0; m < M; m++)
+                if (m < m_rows) acc[1][m] += red[((w - 1) * M + m) * 64 + lane];
+        }
+    } else {
+        tile_accumulate<NR, M, XBF16>(a.w, rt, panels, slice * waves + wave, slices * waves, a.k_dim, a.x, a.x_stride, m_rows, xw, zero, acc);
+        // waves of the block -> wave 0, in wave order
+        if (waves > 1) {
+            if (wave > 0) {
+#pragma unroll
+                for (int r = 0; r < NR; r++)
+#pragma unroll
+                    for (int m = 0; m < M; m++)
+                        if (m < m_rows) red[((wave - 1) * NR * M + r * M + m) * 64 + lane] = acc[r][m];
+            }
+            __syncthreads();
+            if (wave > 0) return;
+            for (int w = 1; w < waves; w++) {
+#pragma unroll
+                for (int r = 0; r < NR; r++)
+#pragma unroll
+                    for (int m = 0; m < M; m++)
+                        if (m < m_rows) acc[r][m] += red[((w - 1) * NR * M + r * M + m) * 64 + lane];
+            }
         }
     }
 

@@ -68,7 +68,17 @@ extern "C" __global__ void __launch_bounds__(1024) gemv_nvfp4_gu(const unsigned 
                                                                  const int* __restrict__ k_dim_p, const int* __restrict__ rows_p) {
     ENTER(wg, wu, x, gs_g, gs_u, y, k_dim_p, rows_p);
     GemvArgs a{{wg, wu}, {gs_g, gs_u}, x, 0, y, 0, *k_dim_p, *rows_p, 1, nullptr};
-    gemv_body<2, 1, false, EPI_SILU_GU, XRows<1, false>::value>(a, 0, LDS, ws);
+    gemv_body<2, 1, false, EPI_SILU_GU, XRows<1, false>::value, true>(a, 0, LDS, ws);
+}
+
+// the same on bf16 activations (BASELINE quotes X in bf16; exact widening)
+extern "C" __global__ void __launch_bounds__(1024) gemv_nvfp4_gu_bf16(const unsigned char* __restrict__ wg, const unsigned char* __restrict__ wu,
+                                                                      const unsigned short* __restrict__ x, const float* __restrict__ gs_g,
+                                                                      const float* __restrict__ gs_u, float* __restrict__ y,
+                                                                      const int* __restrict__ k_dim_p, const int* __restrict__ rows_p) {
+    ENTER(wg, wu, x, gs_g, gs_u, y, k_dim_p, rows_p);
+    GemvArgs a{{wg, wu}, {gs_g, gs_u}, x, 0, y, 0, *k_dim_p, *rows_p, 1, nullptr};
+    gemv_body<2, 1, true, EPI_SILU_GU, XRows<1, true>::value, true>(a, 0, LDS, ws);
 }
 
 // ------------------------------------------------------------------ M <= 4 rows (MTP verify)
@@ -93,7 +103,8 @@ extern "C" __global__ void __launch_bounds__(1024) gemv_nvfp4_wm(const unsigned 
     gemv_m_dispatch<1, false, EPI_SCALE>(a, 0, LDS, ws);
 }
 // reference: gemv_nvfp4_gum, engine/src/kernels_p2.rs:499-530
-extern "C" __global__ void __launch_bounds__(1024) gemv_nvfp4_gum(const unsigned char* __restrict__ wg, const unsigned char* __restrict__ wu,
+// (blocks of at most 8 waves: two weight tiles, four sets of split activation rows and their sums need more than 128 registers)
+extern "C" __global__ void __launch_bounds__(512) gemv_nvfp4_gum(const unsigned char* __restrict__ wg, const unsigned char* __restrict__ wu,
                                                                   const float* __restrict__ x, const float* __restrict__ gs_g,
                                                                   const float* __restrict__ gs_u, float* __restrict__ y,
                                                                   const int* __restrict__ k_dim_p, const int* __restrict__ rows_p,
@@ -182,7 +193,7 @@ extern "C" __global__ void __launch_bounds__(1024) moe_gate_up_silu(const unsign
     const unsigned char* w = (const unsigned char*)ptrs[combo];
     const size_t up_off = (size_t)(inter / CROW_TILE_ROWS) * ((k + CROW_PANEL_COLS - 1) / CROW_PANEL_COLS) * CROW_TILE_BYTES;
     GemvArgs a{{w, w + up_off}, {gs_ptr, gs_ptr}, x + (size_t)(combo / *x_div_p) * *x_stride_p, 0, h + (size_t)combo * inter, 0, k, inter, 1, nullptr};
-    gemv_body<2, 1, false, EPI_SILU_GU, XRows<1, false>::value>(a, blockIdx.z, LDS, ws);
+    gemv_body<2, 1, false, EPI_SILU_GU, XRows<1, false>::value, true>(a, blockIdx.z, LDS, ws);
 }
 
 // Fused routed down projection + weighted combine: y[t][row] += sum_j rw[t][j] * (gs * <down_{e(t,j)} row, h[t K + j]>),

@@ -100,9 +100,10 @@ class Engine:
         if h is None:
             h = torch.empty((t, inter), dtype=torch.float32, device=self.dev)
         p = self.p
-        if t == 1 and x.dtype == torch.float32:
-            gx, gy, gz, bx = launch_dims("gemv_nvfp4_gu", inter, k)
-            launch_v(self.k.f("gemv_nvfp4_gu"), gx, gy, gz, bx,
+        if t == 1:
+            name = "gemv_nvfp4_gu" if x.dtype == torch.float32 else "gemv_nvfp4_gu_bf16"
+            gx, gy, gz, bx = launch_dims(name, inter, k)
+            launch_v(self.k.f(name), gx, gy, gz, bx,
                      [mlp.gate.w_ptr, mlp.up.w_ptr, x.data_ptr(), mlp.gate.gs_ptr, mlp.up.gs_ptr, h.data_ptr(), p.i32(k), p.i32(inter)])
         else:
             name = "gemv_nvfp4_gum" if x.dtype == torch.float32 else "gemv_nvfp4_gum_bf16"
