@@ -29,8 +29,8 @@ for p in (ROOT, os.path.join(ROOT, "tests")):
 
 PEAK_HBM_GBS = 8000.0
 # HBM bytes per launch of the dominant kernel, measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE and scaled by
-# a 256 MiB copy kernel in the same run (profiles/gemv_nvfp4_gum_bf16__config1_m1.md): 101,337,112 read + 818,176 written
-TRAFFIC_GATE_UP_M1 = 102155288
+# a 256 MiB copy kernel in the same run (profiles/gemv_nvfp4_gu_bf16__config1_m1.md): 101,142,440 read + 818,176 written
+TRAFFIC_GATE_UP_M1 = 101960616
 N, K = 17408, 5120
 W_BYTES = N * K // 64 * 36  # 50,135,040: container encoding, 4.5 bits per weight
 
@@ -85,7 +85,7 @@ def main() -> int:
     import torch
 
     from crow_nest_amd import lib as L
-    from crow_nest_amd.engine import Engine
+    from crow_nest_amd.engine import Engine, gemm_kernel_for
     from crow_nest_amd.kernels import KernelGeo, status
     from crow_nest_amd.weights import Nvfp4Matrix, load_fp4, tiled_bytes
     from oracle import oracle as orc  # only for the synthetic inputs' encoder and the cpu_baseline leg
@@ -221,7 +221,7 @@ def main() -> int:
         for m in (16, 128, 512):
             xm = torch.randn(m, K, device=dev).to(torch.bfloat16)
             ym = torch.empty(m, N, dtype=torch.float32, device=dev)
-            nm = "gemm_nvfp4_bf16_m32" if m <= 32 else ("gemm_nvfp4_bf16_m64" if m <= 64 else "gemm_nvfp4_bf16")
+            nm = gemm_kernel_for(m)
             l4 = Launch(eng, nm, N, K, m, [[s["gate"].data_ptr(), xm.data_ptr(), gs1.data_ptr(), ym.data_ptr(), p.i32(K), p.i32(N), p.i32(m)] for s in sets])
             us = l4.us(iters=50)
             e = entry(us, W_BYTES + m * K * 2 + m * N * 4)

@@ -263,8 +263,7 @@ int crow_hip_launch_dims(const char* name, uint32_t rows, uint32_t k_dim, uint32
         if (k_dim == 0 || k_dim % CROW_BLOCK_VALUES != 0) return CROW_ERR_SHAPE;
         const uint32_t mt = strcmp(name, "gemm_nvfp4_bf16_m32") == 0 ? 32 : (strcmp(name, "gemm_nvfp4_bf16_m64") == 0 ? 64 : 128);
         if (mt == 32) {
-            if (z > 32) return CROW_ERR_SHAPE;
-            *out = crow_dims{rt, 1, 1, 256};
+            *out = crow_dims{rt, (z + 31) / 32, 1, 256};
         } else {
             *out = crow_dims{(rt + 3) / 4, (z + mt - 1) / mt, 1, 256};
         }

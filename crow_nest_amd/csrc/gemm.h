@@ -154,9 +154,9 @@ __device__ __forceinline__ void gemm_body(const unsigned char* __restrict__ w, c
     gemm_store<TBK>(acc, gs_ptr[0], y, rt, m0, rows, m_total, lane);
 }
 
-// M <= 32 token rows: the product is bandwidth-bound and needs every CU streaming, so a block is ONE row
-// tile whose panels are dealt to its 4 waves (wave w: panels w, w + 4, ...).  Each wave stages its
-// own X panel in its own LDS region and reads it back itself: no block barrier in the loop.  The
+// Token blocks of 32 rows: a block is ONE row tile and one token block (blockIdx.y) whose panels are dealt to
+// its 4 waves (wave w: panels w, w + 4, ...), so that even a small M puts every SIMD to work.  Each wave stages
+// its own X panel in its own LDS region and reads it back itself: no block barrier in the loop.  The
 // four partial tiles are added in wave order through LDS at the end (deterministic).
 __device__ __forceinline__ void gemm_small_body(const unsigned char* __restrict__ w, const unsigned short* __restrict__ x,
                                                 const float* __restrict__ gs_ptr, float* __restrict__ y, int k_dim, int rows,
@@ -164,7 +164,7 @@ __device__ __forceinline__ void gemm_small_body(const unsigned char* __restrict_
     constexpr int TBK = 2;
     const int lane = lane_id();
     const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
-    const int rt = (int)blockIdx.x;
+    const int rt = (int)blockIdx.x, m0 = 32 * (int)blockIdx.y;
     const int panels = (k_dim + CROW_PANEL_COLS - 1) / CROW_PANEL_COLS;
     __bf16* xs = xs_all + wave * (32 * CROW_GEMM_XS_STRIDE);
     const __bf16* xs_lane = xs + (lane & 15) * CROW_GEMM_XS_STRIDE + (lane >> 4) * 8;
@@ -185,7 +185,7 @@ __device__ __forceinline__ void gemm_small_body(const unsigned char* __restrict_
             const int c = i * 64 + lane, r = c >> 5, q = c & 31;
             const int k = p * CROW_PANEL_COLS + q * 8;
             xv[i] = make_uint4(0, 0, 0, 0);
-            if (r < m_total && k < k_dim) xv[i] = *(const uint4*)(x + (size_t)r * k_dim + k);
+            if (m0 + r < m_total && k < k_dim) xv[i] = *(const uint4*)(x + (size_t)(m0 + r) * k_dim + k);
         }
         uint4 sc, cd[CROW_STEPS];
         const uint4* t = wt + (size_t)p * (CROW_TILE_BYTES / 16);
@@ -222,7 +222,7 @@ __device__ __forceinline__ void gemm_small_body(const unsigned char* __restrict_
 #pragma unroll
                 for (int r = 0; r < 4; r++) acc[tb][j][r] += q[((tb * 4 + j) * 4 + r) * 64 + lane];
     }
-    gemm_store<TBK>(acc, gs_ptr[0], y, rt, 0, rows, m_total, lane);
+    gemm_store<TBK>(acc, gs_ptr[0], y, rt, m0, rows, m_total, lane);
 }
 
 }  // namespace crow
@@ -238,7 +238,7 @@ __device__ __forceinline__ void gemm_small_body(const unsigned char* __restrict_
         __shared__ __attribute__((aligned(16))) __bf16 xs[16 * TBK * CROW_GEMM_XS_STRIDE];                                     \
         crow::gemm_body<TBK>(w, x, gs_ptr, y, *k_dim_p, *rows_p, *m_p, xs);                                                    \
     }
-// M <= 32: grid (row_tiles), block 256
+// token blocks of 32: grid (row_tiles, ceil(M / 32)), block 256
 extern "C" __global__ void __launch_bounds__(256, 2) gemm_nvfp4_bf16_m32(const unsigned char* __restrict__ w, const unsigned short* __restrict__ x,
                                                                          const float* __restrict__ gs_ptr, float* __restrict__ y,
                                                                          const int* __restrict__ k_dim_p, const int* __restrict__ rows_p,

@@ -190,14 +190,22 @@ class Engine:
         return ids, wts, y
 
     # ------------------------------------------------------------------ prefill GEMM (M >= 16)
-    def gemm(self, w: Fp4, m: int, x: torch.Tensor, y: torch.Tensor | None = None) -> torch.Tensor:
-        """Y[m][rows] = X[m][cols] W^T on the matrix cores (bf16 X, exact bf16 weight tiles, f32 accumulate)."""
+    def gemm(self, w: Fp4, m: int, x: torch.Tensor, y: torch.Tensor | None = None, kernel: str | None = None) -> torch.Tensor:
+        """Y[m][rows] = X[m][cols] W^T on the matrix cores (bf16 X, exact bf16 weight tiles, f32 accumulate).
+        `kernel` forces one of the three entry points (all take any m); default: gemm_kernel_for(m)."""
         rows, k = w.rows, w.cols
         assert x.is_cuda and x.is_contiguous() and x.dtype == torch.bfloat16 and x.numel() == m * k
         if y is None:
             y = torch.empty((m, rows), dtype=torch.float32, device=self.dev)
-        name = "gemm_nvfp4_bf16_m32" if m <= 32 else ("gemm_nvfp4_bf16_m64" if m <= 64 else "gemm_nvfp4_bf16")
+        name = kernel or gemm_kernel_for(m)
         gx, gy, gz, bx = launch_dims(name, rows, k, m)
         p = self.p
         launch_v(self.k.f(name), gx, gy, gz, bx, [w.w_ptr, x.data_ptr(), w.gs_ptr, y.data_ptr(), p.i32(k), p.i32(rows), p.i32(m)])
         return y
+
+
+def gemm_kernel_for(m: int) -> str:
+    """Which GEMM entry point serves m token rows.  Up to 256 rows the K-split body (one row tile per block, its panels
+    dealt to the block's four waves, 32-token blocks on grid.y) keeps every SIMD busy; beyond that the body that shares
+    one staged X tile between four row tiles (64 tokens per wave) decodes the weights fewer times."""
+    return "gemm_nvfp4_bf16_m32" if m <= 256 else "gemm_nvfp4_bf16_m64"

@@ -295,16 +295,17 @@ def test_config0_full_size(eng):
 
 # ---------------------------------------------------------------- batched GEMM on the matrix cores (config 4)
 
+@pytest.mark.parametrize("kernel", ["gemm_nvfp4_bf16_m32", "gemm_nvfp4_bf16_m64", "gemm_nvfp4_bf16"])
 @pytest.mark.parametrize("m,rows,cols", [(16, 320, 1024), (17, 100, 320), (33, 256, 512), (128, 512, 2048), (200, 192, 5120)])
-def test_gemm_bf16_against_the_cpu_path(eng, m, rows, cols):
+def test_gemm_bf16_against_the_cpu_path(eng, m, rows, cols, kernel):
     """Weights decode to exact bf16, X is bf16, products are exact in f32: only the summation order
     differs from the CPU path (which gets the exactly widened X)."""
-    print(f"case m={m} rows={rows} cols={cols}", flush=True)
+    print(f"case m={m} rows={rows} cols={cols} {kernel}", flush=True)
     w = random_nvfp4(m * 7 + rows, rows, cols)
     gs = 6.0e-4
     f = _load(w, rows, cols, gs)
     xb, xw = _bf16_dev(normal_f32(7, m, m * cols))
-    y = eng.gemm(f, m, xb.reshape(m, cols).contiguous()).cpu().numpy()
+    y = eng.gemm(f, m, xb.reshape(m, cols).contiguous(), kernel=kernel).cpu().numpy()
     eng.check()
     ref = orc.gemv(w, rows, cols, gs, xw.reshape(m, cols), threads=8)
     assert rel_err(y, ref) <= TOL
