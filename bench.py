@@ -78,7 +78,7 @@ def main() -> int:
     a = ap.parse_args()
     if a.gpus != 1:
         print(f"bench.py: this build runs on ONE GPU (every box here has one); --gpus {a.gpus} is not supported. "
-              "DESIGN.md says how the path would shard.", file=sys.stderr)
+              "The path would shard by output rows, with no exchange inside the product.", file=sys.stderr)
         return 2
 
     import numpy as np

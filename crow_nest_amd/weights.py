@@ -8,6 +8,7 @@ Mirrors, for the NVFP4 path only:
   * the loader's scale rule 0x7F -> 0x7E (engine/src/gen.rs:2178-2187, residency.rs:126-137), which the
     library's repacker applies while it re-tiles (``crow_hip_repack_nvfp4``);
   * ``Params`` (engine/src/gen.rs:2913-2925): the 4-byte device words kernels read their scalars from.
+  * ``load_fp4(cnq, name, sec)`` from an open container (``crow_nest_amd/cnq.py``): ``load_fp4_cnq``.
 PyTorch tensors are used as device allocations only.
 """
 from __future__ import annotations
@@ -93,6 +94,38 @@ def load_fp4(m: Nvfp4Matrix) -> Fp4:
     repack_into(raw, m.rows, m.cols, w)
     gs = torch.tensor([m.global_scale], dtype=torch.float32, device=dev)
     return Fp4(w, gs, m.rows, m.cols)
+
+
+def nvfp4_matrix_of(cnq, name: str, sec: str) -> Nvfp4Matrix:
+    """The container bytes of one 2-D NVFP4 tensor of an open CNQ1 container as an ``Nvfp4Matrix`` (host side).
+    The dtype check and its text are ``weights::load_fp4``'s (engine/src/weights.rs:26-28); rows and cols come from the
+    index entry's shape, and the byte length is checked against it as ``Nvfp4Matrix::new`` does."""
+    t = cnq.find(name, sec)
+    if t.dtype in ("bf16", "f32"):
+        raise AssertionError(f"{name}: expected NVFP4, got {t.dtype}")
+    if len(t.shape) != 2 or t.shape[0] * t.shape[1] != t.n_values:
+        raise ValueError(f"{name}: shape {list(t.shape)} is not a matrix of {t.n_values} values")
+    return Nvfp4Matrix.new(cnq.read_bytes(t), t.shape[0], t.shape[1], t.global_scale)
+
+
+def load_fp4_cnq(cnq, name: str, sec: str) -> Fp4:
+    """``weights::load_fp4(cnq, name, sec)`` (engine/src/weights.rs:26-33): read the tensor's bytes from the container,
+    upload, re-tile on the device (the scale rule is applied there), keep (w, gs)."""
+    return load_fp4(nvfp4_matrix_of(cnq, name, sec))
+
+
+def load_expert_slabs_cnq(cnq, name: str, sec: str) -> ExpertSlabs:
+    """An expert tensor [E][rows][cols] of a container, read slab by slab with ``read_range`` (row-aligned reads, as
+    engine/src/residency.rs:108-117 cuts them) and re-tiled per expert."""
+    t = cnq.find(name, sec)
+    if t.dtype in ("bf16", "f32"):
+        raise AssertionError(f"{name}: expected NVFP4, got {t.dtype}")
+    if len(t.shape) != 3 or t.shape[0] * t.shape[1] * t.shape[2] != t.n_values:
+        raise ValueError(f"{name}: shape {list(t.shape)} is not [experts][rows][cols] of {t.n_values} values")
+    e, rows, cols = t.shape
+    per = Nvfp4Matrix.byte_len(rows, cols)
+    data = np.concatenate([cnq.read_range(t, i * per, per) for i in range(e)])
+    return load_expert_slabs(data, e, rows, cols, t.global_scale)
 
 
 def unpack(w: Fp4) -> np.ndarray:

@@ -328,3 +328,43 @@ def test_gemm_full_size_sampled_rows(eng):
     x2 = (xb.reshape(m, cols).float() * 4.0).to(torch.bfloat16).contiguous()
     y2 = eng.gemm(f, m, x2).cpu().numpy()
     assert np.array_equal(y2.view(np.uint32), (y * np.float32(4.0)).view(np.uint32))
+
+
+# ---------------------------------------------------------------- a real container through the load path
+
+def test_container_tensors_load_dequantise_and_multiply(eng):
+    """Every NVFP4 tensor of the reference's container fixture: read from the file, repacked at load, dequantised
+    bit-exactly, multiplied within tolerance; its gate / down pair run as one dense FFN."""
+    import os
+
+    from conftest import GOLDEN
+    from crow_nest_amd.cnq import Cnq
+    from crow_nest_amd.weights import dequant, load_fp4_cnq, unpack
+    c = Cnq.open(os.path.join(GOLDEN, "synthetic-v2.cnq"))
+    loaded = {}
+    for t in c.tensors:
+        if t.dtype != "nvfp4":
+            continue
+        print(f"case {t.name} {t.shape}", flush=True)
+        raw = c.read_bytes(t)
+        rows, cols = t.shape
+        f = load_fp4_cnq(c, t.name, t.section)
+        assert np.array_equal(unpack(f), raw)  # no 0x7F scale byte in this container: the round trip is the identity
+        want = orc.dequant(raw, t.global_scale)
+        assert np.array_equal(dequant(f).cpu().numpy().reshape(-1).view(np.uint32), want.view(np.uint32))
+        x = normal_f32(11, len(loaded), 3 * cols).reshape(3, cols)
+        y = eng.proj_m(f, 3, _dev(x)).cpu().numpy()
+        assert rel_err(y, orc.gemv(raw, rows, cols, t.global_scale, x)) <= TOL
+        loaded[t.name] = (f, raw, t)
+    assert len(loaded) == 6
+    # layers.0 gate_proj [128, 64] as gate AND up, layers.1 down_proj [64, 128] as down: a small dense FFN from the file
+    from crow_nest_amd.engine import MlpW
+    g, graw, gt = loaded["model.language_model.layers.0.mlp.gate_proj.weight"]
+    u, uraw, ut = loaded["model.language_model.layers.0.linear_attn.in_proj_qkv.weight"]
+    d, draw, dt = loaded["model.language_model.layers.1.mlp.down_proj.weight"]
+    x = normal_f32(12, 0, 2 * 64).reshape(2, 64) * np.float32(40.0)
+    y = eng.dense_ffn_w(MlpW(g, u, d), _dev(x), 2).cpu().numpy()
+    ref = orc.ffn(graw, gt.global_scale, uraw, ut.global_scale, draw, dt.global_scale, 64, 128, x)
+    assert rel_err(y, ref) <= TOL
+    eng.check()
+    c.close()
