@@ -156,6 +156,16 @@ def main() -> int:
     parity_h = rel_err(h.cpu().numpy(), ref_h)
     parity_y = rel_err(y.cpu().numpy(), orc.gemv(host["down"][0], K, N, host["down"][1], ref_h, threads=8)[0])
 
+    # ---------------- the same step as a captured graph (10 steps, one per weight copy, in one graph)
+    from crow_nest_amd.kernels import Graph
+    gr = Graph()
+    with gr.capture():
+        for i in range(copies):
+            step(i)
+    gr.time(3)
+    graph_us_per_step = min(gr.time(40) for _ in range(3)) / copies
+    gr.close()
+
     # ---------------- roofline of the dominant kernel (gate/up + SiLU), HIP events on the launch stream
     gu_us = gu.us()
     dn_us = dn.us()
@@ -172,6 +182,9 @@ def main() -> int:
         "config": {"workload": "BASELINE config 1 at M=1: fused gate/up+SiLU GEMV (W_gate,W_up [17408,5120] NVFP4, X bf16) + down "
                                "projection (W_down [5120,17408] on f32 H), batch 1; 10 rotating weight copies (1.5 GB)",
                    "algorithmic_bytes_per_step": step_bytes, "pct_of_peak": round(100 * value / PEAK_HBM_GBS, 1),
+                   "arithmetic": "exact bf16 x bf16 products on the matrix cores (weights decode exactly, f32 activations split "
+                                 "into three exact bf16 terms), f32 accumulation and scales",
+                   "graph_replay_us_per_step": round(graph_us_per_step, 2),
                    "us_per_call": {"gate_up_silu": round(gu_us, 2), "down": round(dn_us, 2)},
                    "parity_max_rel_err": {"h": float(f"{parity_h:.3g}"), "y": float(f"{parity_y:.3g}")},
                    "device": name_buf.value.decode(), "input_generation_s": round(gen_s, 1)},

@@ -413,6 +413,66 @@ int crow_hip_time_sequence(uint32_t n_kernels, const crow_fn_t* fns, const crow_
     return out;
 }
 
+int crow_hip_stream_create(void** out) {
+    if (!g.ready) return CROW_ERR_NOT_INITIALIZED;
+    if (!out) return CROW_ERR_BAD_ARGUMENT;
+    hipStream_t s = nullptr;
+    const int rc = hip_rc(hipStreamCreateWithFlags(&s, hipStreamNonBlocking));
+    *out = (void*)s;
+    return rc;
+}
+int crow_hip_stream_destroy(void* stream) {
+    if (!stream) return CROW_OK;
+    if (g.stream == (hipStream_t)stream) g.stream = nullptr;
+    return hip_rc(hipStreamDestroy((hipStream_t)stream));
+}
+int crow_hip_begin_capture(void* stream) {
+    if (!g.ready) return CROW_ERR_NOT_INITIALIZED;
+    if (!stream) return CROW_ERR_BAD_ARGUMENT;  // the legacy default stream cannot be captured
+    g.stream = (hipStream_t)stream;
+    return hip_rc(hipStreamBeginCapture((hipStream_t)stream, hipStreamCaptureModeGlobal));
+}
+int crow_hip_end_capture_instantiate(void* stream, void** graph_exec_out) {
+    if (!g.ready) return CROW_ERR_NOT_INITIALIZED;
+    if (!stream || !graph_exec_out) return CROW_ERR_BAD_ARGUMENT;
+    hipGraph_t graph = nullptr;
+    hipError_t e = hipStreamEndCapture((hipStream_t)stream, &graph);
+    if (e != hipSuccess) return (int)e;
+    hipGraphExec_t exec = nullptr;
+    e = hipGraphInstantiate(&exec, graph, nullptr, nullptr, 0);
+    (void)hipGraphDestroy(graph);  // the executable graph is independent of its template
+    if (e != hipSuccess) return (int)e;
+    *graph_exec_out = (void*)exec;
+    return CROW_OK;
+}
+int crow_hip_launch_graph(void* graph_exec, void* stream) {
+    if (!g.ready) return CROW_ERR_NOT_INITIALIZED;
+    if (!graph_exec) return CROW_ERR_BAD_ARGUMENT;
+    return hip_rc(hipGraphLaunch((hipGraphExec_t)graph_exec, (hipStream_t)stream));
+}
+int crow_hip_graph_exec_destroy(void* graph_exec) {
+    if (!graph_exec) return CROW_OK;
+    return hip_rc(hipGraphExecDestroy((hipGraphExec_t)graph_exec));
+}
+int crow_hip_time_graph(void* graph_exec, void* stream, uint32_t iters, float* us_per_replay) {
+    if (!g.ready) return CROW_ERR_NOT_INITIALIZED;
+    if (!graph_exec || !us_per_replay || iters == 0) return CROW_ERR_BAD_ARGUMENT;
+    hipEvent_t a, b;
+    hipError_t rc;
+    if ((rc = hipEventCreate(&a)) != hipSuccess) return (int)rc;
+    if ((rc = hipEventCreate(&b)) != hipSuccess) return (int)rc;
+    int out = hip_rc(hipEventRecord(a, (hipStream_t)stream));
+    for (uint32_t i = 0; i < iters && out == CROW_OK; i++) out = hip_rc(hipGraphLaunch((hipGraphExec_t)graph_exec, (hipStream_t)stream));
+    if (out == CROW_OK) out = hip_rc(hipEventRecord(b, (hipStream_t)stream));
+    if (out == CROW_OK) out = hip_rc(hipEventSynchronize(b));
+    float ms = 0.0f;
+    if (out == CROW_OK) out = hip_rc(hipEventElapsedTime(&ms, a, b));
+    (void)hipEventDestroy(a);
+    (void)hipEventDestroy(b);
+    *us_per_replay = ms * 1000.0f / (float)iters;
+    return out;
+}
+
 size_t crow_hip_container_bytes(uint32_t rows, uint32_t cols) { return crow_container_bytes(rows, cols); }
 size_t crow_hip_tiled_bytes(uint32_t rows, uint32_t cols) { return crow_tiled_bytes(rows, cols); }
 

@@ -143,6 +143,62 @@ def time_sequence(kernels, n_sets: int, iters: int) -> float:
     return float(us.value)
 
 
+class Graph:
+    """A captured launch sequence (the reference's CROW_GRAPH path, engine/src/cuda.rs:113-203):
+
+        g = Graph()
+        with g.capture():           # begin_capture on the graph's own non-blocking stream; launch_v records
+            launch_v(...); launch_v(...)
+        g.launch()                  # launch_graph on that stream
+    """
+
+    def __init__(self):
+        _l.ensure_init()
+        s = C.c_void_p()
+        _l.check(_l.lib().crow_hip_stream_create(C.byref(s)), "crow_hip_stream_create")
+        self.stream = s
+        self.exec = C.c_void_p()
+
+    class _Capture:
+        def __init__(self, g):
+            self.g = g
+
+        def __enter__(self):
+            self.prev = _l.lib().crow_hip_cur_stream()
+            _l.check(_l.lib().crow_hip_begin_capture(self.g.stream), "crow_hip_begin_capture")
+            return self.g
+
+        def __exit__(self, et, ev, tb):
+            rc = _l.lib().crow_hip_end_capture_instantiate(self.g.stream, C.byref(self.g.exec))
+            _l.lib().crow_hip_set_stream(self.prev)
+            if et is None:
+                _l.check(rc, "crow_hip_end_capture_instantiate")
+            return False
+
+    def capture(self):
+        return Graph._Capture(self)
+
+    def launch(self) -> None:
+        _l.check(_l.lib().crow_hip_launch_graph(self.exec, self.stream), "crow_hip_launch_graph")
+
+    def sync(self) -> None:
+        import torch
+        torch.cuda.synchronize()
+
+    def time(self, iters: int) -> float:
+        us = C.c_float()
+        _l.check(_l.lib().crow_hip_time_graph(self.exec, self.stream, iters, C.byref(us)), "crow_hip_time_graph")
+        return float(us.value)
+
+    def close(self) -> None:
+        if self.exec:
+            _l.lib().crow_hip_graph_exec_destroy(self.exec)
+            self.exec = C.c_void_p()
+        if self.stream:
+            _l.lib().crow_hip_stream_destroy(self.stream)
+            self.stream = C.c_void_p()
+
+
 class Event:
     """A HIP event on the library's current stream (the stream every launch_v goes to)."""
 

@@ -74,6 +74,13 @@ def lib():
         "crow_hip_event_destroy": (C.c_int, [vp]),
         "crow_hip_time_launches": (C.c_int, [vp, u32, u32, u32, u32, u64p, u32, u32, u32, C.POINTER(C.c_float)]),
         "crow_hip_time_sequence": (C.c_int, [u32, C.POINTER(vp), C.POINTER(Dims), C.POINTER(u32), u64p, u32, u32, C.POINTER(C.c_float)]),
+        "crow_hip_stream_create": (C.c_int, [C.POINTER(vp)]),
+        "crow_hip_stream_destroy": (C.c_int, [vp]),
+        "crow_hip_begin_capture": (C.c_int, [vp]),
+        "crow_hip_end_capture_instantiate": (C.c_int, [vp, C.POINTER(vp)]),
+        "crow_hip_launch_graph": (C.c_int, [vp, vp]),
+        "crow_hip_graph_exec_destroy": (C.c_int, [vp]),
+        "crow_hip_time_graph": (C.c_int, [vp, vp, u32, C.POINTER(C.c_float)]),
         "crow_hip_container_bytes": (sz, [u32, u32]),
         "crow_hip_tiled_bytes": (sz, [u32, u32]),
         "crow_hip_repack_nvfp4": (C.c_int, [vp, u32, u32, vp]),
@@ -94,6 +101,8 @@ EXPORTS = [
     "crow_hip_function_name", "crow_hip_function_arg_count", "crow_hip_set_geo", "crow_hip_launch",
     "crow_hip_launch_dims", "crow_hip_status", "crow_hip_reset_workspace", "crow_hip_set_stream", "crow_hip_cur_stream",
     "crow_hip_sync", "crow_hip_event_create", "crow_hip_event_record", "crow_hip_event_elapsed_ms", "crow_hip_event_destroy", "crow_hip_time_launches", "crow_hip_time_sequence", "crow_hip_alloc", "crow_hip_free", "crow_hip_upload", "crow_hip_download",
+    "crow_hip_stream_create", "crow_hip_stream_destroy", "crow_hip_begin_capture", "crow_hip_end_capture_instantiate",
+    "crow_hip_launch_graph", "crow_hip_graph_exec_destroy", "crow_hip_time_graph",
     "crow_hip_container_bytes", "crow_hip_tiled_bytes", "crow_hip_repack_nvfp4", "crow_hip_unpack_nvfp4",
     "crow_hip_dequant_tiled",
 ]

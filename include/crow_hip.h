@@ -103,6 +103,20 @@ int crow_hip_time_launches(crow_fn_t f, uint32_t gx, uint32_t gy, uint32_t gz, u
 int crow_hip_time_sequence(uint32_t n_kernels, const crow_fn_t* fns, const crow_dims* dims, const uint32_t* n_vals,
                            const uint64_t* vals, uint32_t n_sets, uint32_t iters, float* us_per_iteration);
 
+/* ---- graph capture: cuda::stream_create_non_blocking / begin_capture / end_capture_instantiate / launch_graph /
+ * graph_exec_destroy / stream_destroy, engine/src/cuda.rs:113-203.  A launch sequence issued with crow_hip_launch
+ * between begin and end on a created stream is recorded, not run (no host read, no synchronisation, no allocation and
+ * no memset happens inside crow_hip_launch); the instantiated graph replays it.  Capture mode is global, as the
+ * reference's.  Default stream priority only. ---- */
+int crow_hip_stream_create(void** out);         /* non-blocking stream */
+int crow_hip_stream_destroy(void* stream);
+int crow_hip_begin_capture(void* stream);       /* also makes `stream` the current stream, as the reference's capture path does */
+int crow_hip_end_capture_instantiate(void* stream, void** graph_exec_out); /* the template graph is destroyed */
+int crow_hip_launch_graph(void* graph_exec, void* stream);
+int crow_hip_graph_exec_destroy(void* graph_exec);
+/* `iters` back-to-back replays on `stream` between two events; mean microseconds per replay */
+int crow_hip_time_graph(void* graph_exec, void* stream, uint32_t iters, float* us_per_replay);
+
 /* ---- load-time repack (the one call the reference does not have) ---- */
 size_t crow_hip_container_bytes(uint32_t rows, uint32_t cols);
 size_t crow_hip_tiled_bytes(uint32_t rows, uint32_t cols);

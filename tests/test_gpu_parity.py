@@ -368,3 +368,53 @@ def test_container_tensors_load_dequantise_and_multiply(eng):
     assert rel_err(y, ref) <= TOL
     eng.check()
     c.close()
+
+
+# ---------------------------------------------------------------- captured launch sequences
+
+def test_captured_sequence_replays_match_eager_launches(eng):
+    """The decode sequence gate/up+SiLU -> down -> lm_head + argmax stage 1 -> argmax stage 2, captured once and replayed
+    with new inputs, eager work and synchronisations in between: every replay equals the eager result bit for bit."""
+    from crow_nest_amd.kernels import Graph, launch_dims, launch_v, sync
+    H, I, V = 1024, 2816, 4000
+    wg, wu, wd, wh = random_nvfp4(31, I, H), random_nvfp4(32, I, H), random_nvfp4(33, H, I), random_nvfp4(34, V, H)
+    g_, u_, d_, h_ = _load(wg, I, H, 2e-3), _load(wu, I, H, 1.5e-3), _load(wd, H, I, 1.1e-3), _load(wh, V, H, 9e-4)
+    p = eng.p
+    x = torch.zeros(H, dtype=torch.float32, device="cuda")
+    hbuf = torch.empty(I, dtype=torch.float32, device="cuda")
+    y = torch.empty(H, dtype=torch.float32, device="cuda")
+    logits = torch.empty(V, dtype=torch.float32, device="cuda")
+    tok = torch.zeros(1, dtype=torch.int32, device="cuda")
+    seq = [("gemv_nvfp4_gu", launch_dims("gemv_nvfp4_gu", I, H), [g_.w_ptr, u_.w_ptr, x.data_ptr(), g_.gs_ptr, u_.gs_ptr, hbuf.data_ptr(), p.i32(H), p.i32(I)]),
+           ("gemv_nvfp4_w", launch_dims("gemv_nvfp4_w", H, I), [d_.w_ptr, hbuf.data_ptr(), d_.gs_ptr, y.data_ptr(), p.i32(I), p.i32(H)]),
+           ("gemv_nvfp4_w_argmax", launch_dims("gemv_nvfp4_w_argmax", V, H), [h_.w_ptr, y.data_ptr(), h_.gs_ptr, logits.data_ptr(), p.i32(H), p.i32(V), tok.data_ptr()]),
+           ("argmax_tiles", (1, 1, 1, 256), [tok.data_ptr(), p.i32(V)])]
+
+    def eager():
+        for name, dims, vals in seq:
+            launch_v(eng.k.f(name), *dims, vals)
+        sync()
+        torch.cuda.synchronize()
+        return y.cpu().numpy().copy(), logits.cpu().numpy().copy(), int(tok.item())
+
+    torch.cuda.synchronize()
+    gr = Graph()
+    with gr.capture():
+        for name, dims, vals in seq:
+            launch_v(eng.k.f(name), *dims, vals)
+    for r in range(4):
+        x.copy_(_dev(normal_f32(50, r, H) * np.float32(0.05)))
+        ye, le, te = eager()
+        y.zero_(); logits.zero_(); tok.zero_()  # eager work of the program's own between the replays
+        torch.cuda.synchronize()
+        gr.launch()
+        gr.sync()
+        assert np.array_equal(y.cpu().numpy().view(np.uint32), ye.view(np.uint32)), r
+        assert np.array_equal(logits.cpu().numpy().view(np.uint32), le.view(np.uint32)), r
+        assert int(tok.item()) == te == int(orc.argmax_ref(le)), r
+    # and the replayed result is the CPU path's
+    xr = normal_f32(50, 3, H) * np.float32(0.05)
+    ref = orc.ffn(wg, 2e-3, wu, 1.5e-3, wd, 1.1e-3, H, I, xr.reshape(1, H))[0]
+    assert rel_err(y.cpu().numpy(), ref) <= TOL
+    gr.close()
+    eng.check()
