@@ -84,6 +84,10 @@ extern "C" __global__ void __launch_bounds__(1024) gemv_nvfp4_gu_bf16(const unsi
 // ------------------------------------------------------------------ M <= 4 rows (MTP verify)
 template <int NR, bool XBF16, int EPI>
 __device__ __forceinline__ void gemv_m_dispatch(GemvArgs& a, unsigned z, lds_p lds, const Workspace& ws) {
+    if (a.m < 1 || a.m > 4) {  // the reference's NVFP4_MMAX (engine/src/kernels_p2.rs:397-400); uniform over the launch
+        if (threadIdx.x == 0) atomicOr(ws.status, STATUS_BAD_SHAPE);
+        return;
+    }
     // one body per M keeps each row's operation sequence identical to the one-row kernel
     switch (a.m) {
         case 1: gemv_body<NR, 1, XBF16, EPI, XRows<4, XBF16>::value>(a, z, lds, ws); break;

@@ -418,3 +418,21 @@ def test_captured_sequence_replays_match_eager_launches(eng):
     assert rel_err(y.cpu().numpy(), ref) <= TOL
     gr.close()
     eng.check()
+
+
+def test_verify_kernels_refuse_more_than_four_rows(eng):
+    """The reference's verify kernels take at most NVFP4_MMAX = 4 rows (kernels_p2.rs:397-400); a launch with m = 5 writes
+    nothing and reports a shape error through the status word instead of computing four rows silently."""
+    from crow_nest_amd.kernels import launch_dims, launch_v, status
+    from crow_nest_amd.lib import CrowHipError
+    rows, cols = 128, 512
+    f = _load(random_nvfp4(61, rows, cols), rows, cols, 1e-3)
+    x = torch.zeros(5 * cols, dtype=torch.float32, device="cuda")
+    y = torch.full((5 * rows,), 7.0, dtype=torch.float32, device="cuda")
+    p = eng.p
+    launch_v(eng.k.f("gemv_nvfp4_wm"), *launch_dims("gemv_nvfp4_wm", rows, cols), [f.w_ptr, x.data_ptr(), f.gs_ptr, y.data_ptr(), p.i32(cols), p.i32(rows), p.i32(5)])
+    with pytest.raises(CrowHipError) as ei:
+        status()
+    assert ei.value.code == -7  # CROW_ERR_SHAPE
+    assert bool((y == 7.0).all())
+    eng.check()
