@@ -241,6 +241,14 @@ def main() -> int:
             e["TFLOP/s"] = round(2.0 * m * N * K / us / 1e6, 1)
             e["pct_mfma_peak_bf16"] = round(2.0 * m * N * K / us / 1e6 / 2500 * 100, 1)
             others[f"config4_gemm_M{m}"] = e
+        # BF16 keeps (the tensors the container leaves in bf16): router [256, 2048] and a [10240, 2560] projection, f32 x
+        for rows_b, k_b in ((256, 2048), (10240, 2560)):
+            n_b = max(2, int(6e8 // (rows_b * k_b * 2)))
+            wbs = [torch.randn(rows_b, k_b, device=dev).to(torch.bfloat16) for _ in range(min(n_b, 16))]
+            xb_ = torch.randn(k_b, device=dev)
+            lb = Launch(eng, "gemv_bf16_w", rows_b, k_b, 1, [[w_.data_ptr(), xb_.data_ptr(), ybuf.data_ptr(), p.i32(k_b), p.i32(rows_b)] for w_ in wbs])
+            others[f"bf16_keep_gemv_{rows_b}x{k_b}"] = entry(lb.us(), rows_b * k_b * 2 + k_b * 4 + rows_b * 4)
+            del wbs
         # config 2: one MoE layer, 256 experts top-8, H 2048, I 512 (router + fused gate|up+SiLU + fused down+combine)
         from crow_nest_amd.engine import MoeW, expert_table
         from crow_nest_amd.weights import ExpertSlabs

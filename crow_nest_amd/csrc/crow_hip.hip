@@ -33,7 +33,7 @@ const FnEntry g_table[] = {
     CROW_FN(router_top10, 10),     CROW_FN(silu_mul_combo, 3),      CROW_FN(acc_combo, 3),
     CROW_FN(argmax_k, 3),          CROW_FN(argmax_tiles, 2),        CROW_FN(dequant_fp4_flat, 4),    CROW_FN(repack_nvfp4, 4),
     CROW_FN(unpack_nvfp4, 4),      CROW_FN(dequant_nvfp4_tiled, 5), CROW_FN(gemm_nvfp4_bf16, 7),
-    CROW_FN(gemm_nvfp4_bf16_m64, 7), CROW_FN(gemm_nvfp4_bf16_m32, 7),
+    CROW_FN(gemm_nvfp4_bf16_m64, 7), CROW_FN(gemm_nvfp4_bf16_m32, 7), CROW_FN(gemv_bf16_w, 5),
 };
 const int g_table_n = (int)(sizeof(g_table) / sizeof(g_table[0]));
 
@@ -219,6 +219,11 @@ int crow_hip_launch_dims(const char* name, uint32_t rows, uint32_t k_dim, uint32
     if (!e) return CROW_ERR_KERNEL_MISSING;
     const uint32_t rt = (rows + CROW_TILE_ROWS - 1) / CROW_TILE_ROWS;
     const uint32_t panels = (k_dim + CROW_PANEL_COLS - 1) / CROW_PANEL_COLS;
+    if (strcmp(name, "gemv_bf16_w") == 0) {  // z = T activation rows
+        if (k_dim == 0 || k_dim % 8 != 0) return CROW_ERR_SHAPE;
+        *out = crow_dims{(rows + 3) / 4, z, 1, 256};
+        return CROW_OK;
+    }
     if (strncmp(name, "gemv_", 5) == 0 || strncmp(name, "moe_gate_up", 11) == 0) {
         if (k_dim == 0 || k_dim % CROW_BLOCK_VALUES != 0) return CROW_ERR_SHAPE;
         const bool moe = strcmp(name, "gemv_fp4_ptrb") == 0 || strncmp(name, "moe_", 4) == 0;

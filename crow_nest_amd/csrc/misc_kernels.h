@@ -286,3 +286,48 @@ extern "C" __global__ void __launch_bounds__(256) argmax_tiles(int* __restrict__
         out[0] = b.i;
     }
 }
+
+// ------------------------------------------------------------------ BF16 keeps
+// reference: gemv_bf16_w, engine/src/kernels.rs:1130-1157 - y[t][row] = sum_k bf16(w[row][k]) * x[t][k] for the tensors the
+// container keeps in bf16 (router, q/k, MTP head), f32 activations, f32 accumulation; k_dim % 8 == 0.
+// One wavefront per (row, t): grid (ceil(rows / 4), T), block 256 = 4 rows; 16-byte non-temporal weight loads (8 bf16 per
+// lane per step, 1024 contiguous bytes per instruction), x through the vector cache (it is re-read by every row).
+// Order: a lane adds its products in column order with one FMA each (columns 8 lane + 512 j + 0..7), then the 64 lane sums
+// are added by halving (lane l += lane l + 32, + 16, ... + 1).
+extern "C" __global__ void __launch_bounds__(256) gemv_bf16_w(const unsigned short* __restrict__ w, const float* __restrict__ x,
+                                                              float* __restrict__ y, const int* __restrict__ k_dim_p,
+                                                              const int* __restrict__ rows_p) {
+    const int k = *k_dim_p, rows = *rows_p;
+    const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6)), lane = lane_id();
+    const int row = (int)blockIdx.x * 4 + wave, t = (int)blockIdx.y;
+    if (row >= rows) return;
+    const unsigned short* wp = w + (size_t)row * k;
+    const float* xp = x + (size_t)t * k;
+    float acc = 0.0f;
+    for (int i0 = lane * 8; i0 < k; i0 += 4 * 512) {
+        uint4 v[4];
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            const int i = i0 + j * 512;
+            v[j] = make_uint4(0, 0, 0, 0);
+            if (i < k) v[j] = stream_load((const uint4*)(wp + i));
+        }
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            const int i = i0 + j * 512;
+            if (i < k) {
+                const float4 a = *(const float4*)(xp + i), b = *(const float4*)(xp + i + 4);
+                acc = __builtin_fmaf(__uint_as_float(v[j].x << 16), a.x, acc);
+                acc = __builtin_fmaf(__uint_as_float(v[j].x & 0xffff0000u), a.y, acc);
+                acc = __builtin_fmaf(__uint_as_float(v[j].y << 16), a.z, acc);
+                acc = __builtin_fmaf(__uint_as_float(v[j].y & 0xffff0000u), a.w, acc);
+                acc = __builtin_fmaf(__uint_as_float(v[j].z << 16), b.x, acc);
+                acc = __builtin_fmaf(__uint_as_float(v[j].z & 0xffff0000u), b.y, acc);
+                acc = __builtin_fmaf(__uint_as_float(v[j].w << 16), b.z, acc);
+                acc = __builtin_fmaf(__uint_as_float(v[j].w & 0xffff0000u), b.w, acc);
+            }
+        }
+    }
+    for (int o = 32; o > 0; o >>= 1) acc += __shfl_down(acc, o);
+    if (lane == 0) y[(size_t)t * rows + row] = acc;
+}

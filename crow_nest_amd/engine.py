@@ -189,6 +189,18 @@ class Engine:
             launch_v(self.k.f("acc_combo"), (hdim + 255) // 256, t, 1, 256, [eo.data_ptr(), wts.data_ptr(), y.data_ptr()])
         return ids, wts, y
 
+    # ------------------------------------------------------------------ BF16 keeps (router, q/k, MTP head)
+    def bf16_proj(self, w: torch.Tensor, t: int, x: torch.Tensor, y: torch.Tensor | None = None) -> torch.Tensor:
+        """y[t][rows] = bf16 W [rows][k] times f32 x [t][k]: ``gemv_bf16_w`` (engine/src/kernels.rs:1130-1157)."""
+        assert w.is_cuda and w.dtype == torch.bfloat16 and w.dim() == 2 and w.is_contiguous()
+        rows, k = w.shape
+        assert x.is_cuda and x.dtype == torch.float32 and x.is_contiguous() and x.numel() == t * k
+        if y is None:
+            y = torch.empty((t, rows), dtype=torch.float32, device=self.dev)
+        p = self.p
+        launch_v(self.k.f("gemv_bf16_w"), *launch_dims("gemv_bf16_w", rows, k, t), [w.data_ptr(), x.data_ptr(), y.data_ptr(), p.i32(k), p.i32(rows)])
+        return y
+
     # ------------------------------------------------------------------ prefill GEMM (M >= 16)
     def gemm(self, w: Fp4, m: int, x: torch.Tensor, y: torch.Tensor | None = None, kernel: str | None = None) -> torch.Tensor:
         """Y[m][rows] = X[m][cols] W^T on the matrix cores (bf16 X, exact bf16 weight tiles, f32 accumulate).

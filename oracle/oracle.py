@@ -204,3 +204,14 @@ def f32_to_bf16_bits(v) -> np.ndarray:
 
 def bf16_bits_to_f32(b) -> np.ndarray:
     return (np.asarray(b, np.uint16).astype(np.uint32) << 16).view(np.float32)
+
+
+def gemv_bf16(w_bits, rows: int, cols: int, x) -> np.ndarray:
+    """BF16-keep GEMV of the reference (engine/src/kernels.rs:1130-1157): y[t][r] = sum_k bf16(w[r][k]) * x[t][k].  The product
+    is defined by the real-number sum; this restatement evaluates it in f64 (every bf16 * f32 product is exact in f64, the
+    sum of K <= 2^20 of them carries a relative error below 2^-32) and rounds once to f32.  Device results are held to
+    that value within the f32 dot-product bound gamma(K + 6) * sum |w x| and to the 1e-3 tolerance."""
+    w = bf16_bits_to_f32(np.asarray(w_bits, np.uint16).reshape(rows, cols)).astype(np.float64)
+    xv = _f32(x).reshape(-1, cols).astype(np.float64)
+    return (xv @ w.T).astype(np.float32)
+

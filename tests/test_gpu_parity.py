@@ -436,3 +436,22 @@ def test_verify_kernels_refuse_more_than_four_rows(eng):
     assert ei.value.code == -7  # CROW_ERR_SHAPE
     assert bool((y == 7.0).all())
     eng.check()
+
+
+# ---------------------------------------------------------------- BF16 keeps
+
+@pytest.mark.parametrize("rows,cols,t", [(256, 2048, 1), (256, 2048, 4), (37, 320, 3), (1000, 2560, 1), (64, 10240, 2), (5, 8, 1)])
+def test_bf16_keep_gemv(eng, rows, cols, t):
+    print(f"case rows={rows} cols={cols} t={t}", flush=True)
+    w32 = normal_f32(70, rows, rows * cols) * np.float32(0.05)
+    w_bits = orc.f32_to_bf16_bits(w32).reshape(rows, cols)
+    x = normal_f32(71, t, t * cols).reshape(t, cols)
+    wd = torch.from_numpy(w_bits.view(np.int16)).cuda().view(torch.bfloat16)
+    y = eng.bf16_proj(wd, t, _dev(x)).cpu().numpy()
+    ref = orc.gemv_bf16(w_bits, rows, cols, x)
+    assert rel_err(y, ref) <= TOL
+    wf = orc.bf16_bits_to_f32(w_bits).astype(np.float64)
+    bound = orc.gamma(16 * (cols + 6)) * (np.abs(x.astype(np.float64)) @ np.abs(wf).T)  # gamma(n) of the oracle counts n / 16 + 10 steps
+    assert np.all(np.abs(y.astype(np.float64) - ref.astype(np.float64)) <= bound + 1e-30)
+    eng.check()
+

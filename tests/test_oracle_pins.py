@@ -435,3 +435,23 @@ def test_moe_layer_is_the_staged_composition():
             acc = (acc + w[t, j] * eo).astype(np.float32)
         want[t] = acc
     assert np.array_equal(want.view(np.uint32), y.view(np.uint32))
+
+
+def test_bf16_keep_gemv_is_the_exact_rational_dot_product():
+    """gemv_bf16's f64 evaluation against exact rational arithmetic on small inputs (a transposed operand, a dropped
+    column or a wrong widening of the bf16 bits would show)."""
+    from fractions import Fraction
+    rng = np.random.default_rng(5)
+    rows, cols, t = 5, 24, 2
+    w_bits = rng.integers(0, 1 << 16, size=(rows, cols), dtype=np.uint16)
+    w_bits[(w_bits & 0x7F80) == 0x7F80] = 0x3F80  # no inf / nan
+    w_bits = (w_bits & 0x8FFF) | 0x3000           # exponents near 1: no overflow in the exact sum
+    x = rng.standard_normal((t, cols)).astype(np.float32)
+    y = orc.gemv_bf16(w_bits, rows, cols, x)
+    wf = orc.bf16_bits_to_f32(w_bits)
+    assert np.array_equal(wf.view(np.uint32), w_bits.astype(np.uint32) << 16)
+    for ti in range(t):
+        for r in range(rows):
+            exact = sum(Fraction(float(wf[r, k])) * Fraction(float(x[ti, k])) for k in range(cols))
+            assert y[ti, r] == np.float32(float(exact)), (ti, r)
+
