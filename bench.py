@@ -115,6 +115,9 @@ def main() -> int:
     h = torch.empty(N, dtype=torch.float32, device=dev)
     y = torch.empty(K, dtype=torch.float32, device=dev)
     gen_s = time.time() - t0
+    import hashlib
+    input_sha256 = {nm: hashlib.sha256(host[nm][0].tobytes()).hexdigest()[:16] for nm in host}
+    input_sha256["x_bf16"] = hashlib.sha256(xb_bits.tobytes()).hexdigest()[:16]
 
     gu = Launch(eng, "gemv_nvfp4_gu_bf16", N, K, 1,
                 [[s["gate"].data_ptr(), s["up"].data_ptr(), xb.data_ptr(), base["gate"].gs_ptr, base["up"].gs_ptr, h.data_ptr(),
@@ -187,6 +190,9 @@ def main() -> int:
                    "graph_replay_us_per_step": round(graph_us_per_step, 2),
                    "us_per_call": {"gate_up_silu": round(gu_us, 2), "down": round(dn_us, 2)},
                    "parity_max_rel_err": {"h": float(f"{parity_h:.3g}"), "y": float(f"{parity_y:.3g}")},
+                   "inputs": {"generator": "splitmix64 + Box-Muller, seed 0, one stream per tensor; W ~ N(0, 0.02^2) through the ceil encoder, "
+                                           "x ~ N(0, 1) rounded to bf16", "sha256_16": input_sha256,
+                              "global_scales": {nm: float(np.float32(host[nm][1])) for nm in host}},
                    "device": name_buf.value.decode(), "input_generation_s": round(gen_s, 1)},
         "roofline": roof,
     }
@@ -288,7 +294,7 @@ def main() -> int:
 
     # ---------------- CPU baseline: the C port of the reference's CPU path on this host (rank 0, N = 1 only)
     if not a.no_cpu:
-        threads = max(1, min(os.cpu_count() or 1, 64))
+        threads = max(1, min(os.cpu_count() or 1, int(os.environ.get("OMP_NUM_THREADS", "16") or 16), 16))  # the box's CPU share
         units = []
         g = np.random.default_rng(0)
         for u in range(8):  # 8 distinct units of 150 MB: larger than any L3 (the reference's method, cpu_nvfp4.rs:729-777)
@@ -305,8 +311,21 @@ def main() -> int:
             ts.append(time.perf_counter() - c0)
         ts.sort()
         med = ts[len(ts) // 2]
+        by_threads = {}
+        for th in (1, 4, 8):  # the reference reports 1 / 4 / 8 / all threads (cpu_nvfp4.rs:729-777); 8 calls each here
+            if th >= threads:
+                continue
+            tt = []
+            for rep in range(8):
+                u = units[rep % 8]
+                c0 = time.perf_counter()
+                orc.ffn(u[0], gsv[0], u[1], gsv[1], u[2], gsv[2], K, N, xs, threads=th, path=1)
+                tt.append(time.perf_counter() - c0)
+            tt.sort()
+            by_threads[str(th)] = round(3 * W_BYTES / tt[len(tt) // 2] / 1e9, 2)
+        by_threads[str(threads)] = round(3 * W_BYTES / med / 1e9, 2)
         out["cpu_baseline"] = {"value": round(3 * W_BYTES / med / 1e9, 2), "unit": "GB/s", "cores": threads, "kind": "port",
-                               "ms_per_step": round(med * 1e3, 3),
+                               "ms_per_step": round(med * 1e3, 3), "GB/s_by_threads": by_threads,
                                "sample": "same step (gate/up + SiLU + down, one token, f32 x) on 8 rotating 150 MB weight units, median of 24 calls "
                                          "after a warm-up pass; AVX2 path of the C restatement of engine/src/cpu_nvfp4.rs (OpenMP row split)"}
     print(json.dumps(out))
