@@ -480,6 +480,8 @@ int crow_hip_time_graph(void* graph_exec, void* stream, uint32_t iters, float* u
 
 size_t crow_hip_container_bytes(uint32_t rows, uint32_t cols) { return crow_container_bytes(rows, cols); }
 size_t crow_hip_tiled_bytes(uint32_t rows, uint32_t cols) { return crow_tiled_bytes(rows, cols); }
+uint32_t crow_hip_tile_code_offset(uint32_t row, uint32_t wp) { return row < 64 && wp < 32 ? crow_tile_code_offset(row, wp) : UINT32_MAX; }
+uint32_t crow_hip_tile_scale_offset(uint32_t row, uint32_t sb) { return row < 64 && sb < 16 ? crow_tile_scale_offset(row, sb) : UINT32_MAX; }
 
 static int layout_launch(const char* name, const void* a, const void* b, const void* c, uint32_t rows, uint32_t cols) {
     if (!g.ready) return CROW_ERR_NOT_INITIALIZED;

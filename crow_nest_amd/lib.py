@@ -83,6 +83,8 @@ def lib():
         "crow_hip_time_graph": (C.c_int, [vp, vp, u32, C.POINTER(C.c_float)]),
         "crow_hip_container_bytes": (sz, [u32, u32]),
         "crow_hip_tiled_bytes": (sz, [u32, u32]),
+        "crow_hip_tile_code_offset": (u32, [u32, u32]),
+        "crow_hip_tile_scale_offset": (u32, [u32, u32]),
         "crow_hip_repack_nvfp4": (C.c_int, [vp, u32, u32, vp]),
         "crow_hip_unpack_nvfp4": (C.c_int, [vp, u32, u32, vp]),
         "crow_hip_dequant_tiled": (C.c_int, [vp, vp, u32, u32, vp]),
@@ -103,7 +105,7 @@ EXPORTS = [
     "crow_hip_sync", "crow_hip_event_create", "crow_hip_event_record", "crow_hip_event_elapsed_ms", "crow_hip_event_destroy", "crow_hip_time_launches", "crow_hip_time_sequence", "crow_hip_alloc", "crow_hip_free", "crow_hip_upload", "crow_hip_download",
     "crow_hip_stream_create", "crow_hip_stream_destroy", "crow_hip_begin_capture", "crow_hip_end_capture_instantiate",
     "crow_hip_launch_graph", "crow_hip_graph_exec_destroy", "crow_hip_time_graph",
-    "crow_hip_container_bytes", "crow_hip_tiled_bytes", "crow_hip_repack_nvfp4", "crow_hip_unpack_nvfp4",
+    "crow_hip_container_bytes", "crow_hip_tiled_bytes", "crow_hip_tile_code_offset", "crow_hip_tile_scale_offset", "crow_hip_repack_nvfp4", "crow_hip_unpack_nvfp4",
     "crow_hip_dequant_tiled",
 ]
 

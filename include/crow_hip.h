@@ -120,6 +120,11 @@ int crow_hip_time_graph(void* graph_exec, void* stream, uint32_t iters, float* u
 /* ---- load-time repack (the one call the reference does not have) ---- */
 size_t crow_hip_container_bytes(uint32_t rows, uint32_t cols);
 size_t crow_hip_tiled_bytes(uint32_t rows, uint32_t cols);
+/* where the repacker puts things inside a 9216-byte tile (host arithmetic, no device needed): the byte offset of the code
+ * dword of tile row `row` (0..63), tile columns 8 wp .. 8 wp + 7 (wp 0..31), and of the scale byte of tile row `row`,
+ * 16-column sub-block sb (0..15).  UINT32_MAX for an argument out of range. */
+uint32_t crow_hip_tile_code_offset(uint32_t row, uint32_t wp);
+uint32_t crow_hip_tile_scale_offset(uint32_t row, uint32_t sb);
 /* src_dev: container bytes [rows][cols/64][36] already on the device; dst_dev: crow_hip_tiled_bytes.
  * Applies the scale rule (0x7F -> 0x7E).  Expert tensors [E][rows][cols]: call once per expert
  * slab, the tiled slabs are then contiguous per expert. */

@@ -82,3 +82,30 @@ def test_product_does_not_import_the_oracle():
             if f.endswith((".py", ".h", ".hip", ".cpp", "Makefile")):
                 text = open(os.path.join(dirpath, f)).read()
                 assert "oracle" not in text.lower(), (dirpath, f)
+
+
+def test_tile_layout_is_a_bijection_and_matches_the_matrix_operand_shape():
+    """Every byte of a 9216-byte tile is owned by exactly one (row, column) item, and the placement is the one the kernels
+    assume: a lane's dword d of code segment s is row 16 d + lane % 16, columns 32 s + 8 (lane / 16) .. + 7; a lane's scale byte
+    8 jp + s is row 16 (2 jp + (g & 1)) + n, sub-block 2 s + (g >> 1)."""
+    lib = L.lib()
+    seen = set()
+    for row in range(64):
+        for wp in range(32):
+            o = lib.crow_hip_tile_code_offset(row, wp)
+            s_, g = wp >> 2, wp & 3
+            lane, d = 16 * g + (row & 15), row >> 4
+            assert o == 1024 * (s_ + 1) + 16 * lane + 4 * d and o % 4 == 0
+            for b in range(4):
+                assert o + b not in seen
+                seen.add(o + b)
+        for sb in range(16):
+            o = lib.crow_hip_tile_scale_offset(row, sb)
+            j, n = row >> 4, row & 15
+            g, jp, s_ = 2 * (sb & 1) + (j & 1), j >> 1, sb >> 1
+            assert o == 16 * (16 * g + n) + 8 * jp + s_ and o < 1024
+            assert o not in seen
+            seen.add(o)
+    assert seen == set(range(9216))
+    assert lib.crow_hip_tile_code_offset(64, 0) == 0xFFFFFFFF and lib.crow_hip_tile_scale_offset(0, 16) == 0xFFFFFFFF
+
