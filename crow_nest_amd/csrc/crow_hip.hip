@@ -24,12 +24,12 @@ struct FnEntry {
 #define CROW_FN(name, nargs) {#name, (const void*)&name, nargs, 0u, 0u}
 #define CROW_GEMV(name, nargs, NR, M, XR) {#name, (const void*)&name, nargs, 512u, (XR) * 576u + (NR) * (M) * 256u}
 const FnEntry g_table[] = {
-    CROW_GEMV(gemv_nvfp4_w, 6, 1, 1, 3),       CROW_GEMV(gemv_nvfp4_w_bf16, 6, 1, 1, 1),  CROW_GEMV(gemv_nvfp4_w_argmax, 7, 1, 1, 3),
-    CROW_GEMV(gemv_nvfp4_gu, 8, 1, 1, 3),      CROW_GEMV(gemv_nvfp4_gu_bf16, 8, 1, 1, 1),
+    CROW_GEMV(gemv_nvfp4_w, 6, 1, 1, 4),       CROW_GEMV(gemv_nvfp4_w_bf16, 6, 1, 1, 1),  CROW_GEMV(gemv_nvfp4_w_argmax, 7, 1, 1, 4),
+    CROW_GEMV(gemv_nvfp4_gu, 8, 1, 1, 4),      CROW_GEMV(gemv_nvfp4_gu_bf16, 8, 1, 1, 1),
         CROW_GEMV(gemv_nvfp4_wm, 7, 1, 4, 12),     CROW_GEMV(gemv_nvfp4_gum, 9, 2, 4, 12),
-    CROW_GEMV(gemv_nvfp4_wm_bf16, 7, 1, 4, 4), CROW_GEMV(gemv_nvfp4_gum_bf16, 9, 2, 4, 4), CROW_GEMV(gemv_fp4, 6, 1, 1, 3),
+    CROW_GEMV(gemv_nvfp4_wm_bf16, 7, 1, 4, 4), CROW_GEMV(gemv_nvfp4_gum_bf16, 9, 2, 4, 4), CROW_GEMV(gemv_fp4, 6, 1, 1, 4),
     CROW_GEMV(gemv_fp4_b, 7, 1, 4, 12),        CROW_GEMV(gemv_fp4_b1k, 7, 1, 4, 12),      CROW_GEMV(gemv_fp4_bs, 8, 1, 4, 12),
-    CROW_GEMV(gemv_fp4_ptrb, 8, 1, 1, 3),      CROW_GEMV(moe_gate_up_silu, 8, 1, 1, 3),   CROW_GEMV(moe_down_combine, 7, 1, 1, 3),
+    CROW_GEMV(gemv_fp4_ptrb, 8, 1, 1, 4),      CROW_GEMV(moe_gate_up_silu, 8, 1, 1, 4),   CROW_GEMV(moe_down_combine, 7, 1, 1, 4),
     CROW_FN(router_top10, 10),     CROW_FN(silu_mul_combo, 3),      CROW_FN(acc_combo, 3),
     CROW_FN(argmax_k, 3),          CROW_FN(argmax_tiles, 2),        CROW_FN(dequant_fp4_flat, 4),    CROW_FN(repack_nvfp4, 4),
     CROW_FN(unpack_nvfp4, 4),      CROW_FN(dequant_nvfp4_tiled, 5), CROW_FN(gemm_nvfp4_bf16, 7),

@@ -21,9 +21,9 @@
 // so one FMA per activation row serves two matrix instructions (1024 weights), and the decode costs
 // half an instruction per weight.  bf16 activations ride as they are (r = token).  f32 activations are
 // split exactly into three bf16 terms (x = hi + mid + lo, 8 + 8 + 8 significant bits by truncation);
-// the three terms of ONE token are the rows r = 0..2 of a matrix instruction pair and their results are
-// added as (hi + mid) + lo before the scale FMA: every product w * term is exact in f32, so the only
-// roundings are the f32 additions, as in any f32 dot product.
+// token t's three terms are operand rows 3 t, 3 t + 1, 3 t + 2 (four rows per matrix instruction pair, so M tokens take
+// ceil(3 M / 4) pairs per unit pair) and their results are added as (hi + mid) + lo before the scale FMA: every product
+// w * term is exact in f32, so the only roundings are the f32 additions, as in any f32 dot product.
 //
 // Each wave stages its own activation slice (M rows x 256 columns, 512 bytes per bf16 row) in LDS and
 // reads its A operands from there with one 16-byte read per lane; lanes whose operand row is zero read
@@ -74,10 +74,11 @@ struct GemvArgs {
     int* argmax_out;     // not null: also write the greedy argmax of y row 0 (fused lm_head head)
 };
 
-// staging rows per wave: one bf16 row per token, or three (hi, mid, lo) per f32 token
+// staging rows per wave: one bf16 row per token, or three (hi, mid, lo) per f32 token, rounded up to whole sets of four
+// operand rows (the padding rows are staged as zeros)
 template <int M, bool XBF16>
 struct XRows {
-    static constexpr int value = XBF16 ? M : 3 * M;
+    static constexpr int value = XBF16 ? M : 4 * ((3 * M + 3) / 4);
 };
 #define CROW_GEMV_ZERO_BYTES 512
 // 512 bytes of data per staged row; the 64 bytes of padding put four consecutive rows on four different groups of
@@ -169,6 +170,8 @@ struct XStage<M, false> {
             lds_store8(row + CROW_GEMV_XROW_BYTES, __builtin_amdgcn_perm(m[1], m[0], 0x07060302u), __builtin_amdgcn_perm(m[3], m[2], 0x07060302u));
             lds_store8(row + 2 * CROW_GEMV_XROW_BYTES, __builtin_amdgcn_perm(l[1], l[0], 0x07060302u), __builtin_amdgcn_perm(l[3], l[2], 0x07060302u));
         }
+#pragma unroll
+        for (int r = 3 * M; r < XRows<M, false>::value; r++) lds_store8(xw + r * CROW_GEMV_XROW_BYTES + 8 * lane, 0u, 0u);
     }
 };
 
@@ -176,7 +179,8 @@ struct XStage<M, false> {
 // for segment 0 of set q (or of the zero area); `acc[r][jp][m]` as described at the top of the file.
 template <int NR, int M, bool XBF16, int S>
 struct Segment {
-    static constexpr int NSET = XBF16 ? 1 : M;
+    // f32: the 3 M split rows (token t: rows 3 t, 3 t + 1, 3 t + 2 = hi, mid, lo) fill sets of four operand rows in order
+    static constexpr int NSET = XBF16 ? 1 : (3 * M + 3) / 4;
     // `a1`, `a2`: this lane's LDS address of its A1 / A2 operand of segment 0, set 0; set q is `step` bytes further
     // (0 for a lane that reads the zero area)
     __device__ __forceinline__ static void run(const uint4 (&sc)[NR], const uint4 (&cd)[NR][CROW_STEPS], lds_p a1, lds_p a2, int step1,
@@ -194,16 +198,20 @@ struct Segment {
             for (int r = 0; r < NR; r++) {
                 const bf16x8 B0 = decode8(u4_get(cd[r][S], 2 * jp)), B1 = decode8(u4_get(cd[r][S], 2 * jp + 1));
                 const float sv = e4m3_to_f32<S & 3>(u4_get(sc[r], 2 * jp + (S >> 2)));
+                f32x4 D[NSET];
 #pragma unroll
                 for (int q = 0; q < NSET; q++) {
                     const f32x4 z = {0.f, 0.f, 0.f, 0.f};
-                    f32x4 D = __builtin_amdgcn_mfma_f32_16x16x32_bf16(A1[q], B0, z, 0, 0, 0);
-                    D = __builtin_amdgcn_mfma_f32_16x16x32_bf16(A2[q], B1, D, 0, 0, 0);
-                    if (XBF16) {
+                    D[q] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(A1[q], B0, z, 0, 0, 0);
+                    D[q] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(A2[q], B1, D[q], 0, 0, 0);
+                }
 #pragma unroll
-                        for (int m = 0; m < M; m++) acc[r][jp][m] = __builtin_fmaf(D[m], sv, acc[r][jp][m]);
+                for (int m = 0; m < M; m++) {
+                    if (XBF16) {
+                        acc[r][jp][m] = __builtin_fmaf(D[0][m], sv, acc[r][jp][m]);
                     } else {
-                        acc[r][jp][q] = __builtin_fmaf(__fadd_rn(__fadd_rn(D[0], D[1]), D[2]), sv, acc[r][jp][q]);
+                        const float hi = D[(3 * m) / 4][(3 * m) % 4], mid = D[(3 * m + 1) / 4][(3 * m + 1) % 4], lo = D[(3 * m + 2) / 4][(3 * m + 2) % 4];
+                        acc[r][jp][m] = __builtin_fmaf(__fadd_rn(__fadd_rn(hi, mid), lo), sv, acc[r][jp][m]);
                     }
                 }
             }
@@ -229,8 +237,8 @@ __device__ __forceinline__ void device_order() {
 template <int NR, int M, bool XBF16>
 __device__ __forceinline__ void tile_accumulate(const unsigned char* const (&w)[2], int rt, int panels, int p0, int stride, int k_dim,
                                                 const void* x, size_t x_stride, int m_rows, lds_p xw, lds_p zero, float (&out)[NR][M]) {
-    constexpr int NSET = XBF16 ? 1 : M;
-    constexpr int SET_ROWS = XBF16 ? M : 3;  // live operand rows of a set
+    constexpr int NSET = XBF16 ? 1 : (3 * M + 3) / 4;
+    constexpr int SET_ROWS = XBF16 ? M : 4;  // live operand rows of a set (f32: padding rows are staged as zeros)
     // register-hungry instantiations keep the segments apart: the next segment's operands are not fetched early
     constexpr bool LEAN = NR * NSET >= 2 && !XBF16;
     const int lane = lane_id();

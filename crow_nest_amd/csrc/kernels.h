@@ -215,10 +215,10 @@ extern "C" __global__ void __launch_bounds__(1024) moe_down_combine(const unsign
     }
     const int t = (int)blockIdx.z, rt = (int)blockIdx.y, j = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6)), lane = lane_id();
     const int combo = t * topk + j;
-    // dynamic LDS: zeros, 3 staging rows per wave (f32 activations, one row), then one float per (wave, lane)
-    lds_p zero = LDS, xw = LDS + CROW_GEMV_ZERO_BYTES + j * (3 * CROW_GEMV_XROW_BYTES);
+    // dynamic LDS: zeros, 4 staging rows per wave (f32 activations, one token: hi, mid, lo, zero), then one float per (wave, lane)
+    lds_p zero = LDS, xw = LDS + CROW_GEMV_ZERO_BYTES + j * (4 * CROW_GEMV_XROW_BYTES);
     __attribute__((address_space(3))) float* red =
-        (__attribute__((address_space(3))) float*)(LDS + CROW_GEMV_ZERO_BYTES + topk * (3 * CROW_GEMV_XROW_BYTES));
+        (__attribute__((address_space(3))) float*)(LDS + CROW_GEMV_ZERO_BYTES + topk * (4 * CROW_GEMV_XROW_BYTES));
     if (threadIdx.x < CROW_GEMV_ZERO_BYTES / 16) lds_store16(zero + 16 * threadIdx.x, 0, 0, 0, 0);
     __syncthreads();
     const unsigned char* const w[2] = {(const unsigned char*)ptrs[combo], nullptr};
