@@ -455,3 +455,20 @@ def test_bf16_keep_gemv(eng, rows, cols, t):
     assert np.all(np.abs(y.astype(np.float64) - ref.astype(np.float64)) <= bound + 1e-30)
     eng.check()
 
+
+
+# ---------------------------------------------------------------- the ABI from plain C
+
+def test_c_abi_from_a_plain_c_program():
+    """tests/c_abi/c_abi_gemv.c (gcc, no Python or torch in the process): init, lookup, alloc, upload, repack, launch with the
+    library's dims, status, download - and the result within tolerance of the CPU oracle."""
+    import os
+    import subprocess
+
+    from conftest import ROOT
+    exe = os.path.join(ROOT, "tests", "c_abi", "c_abi_gemv")
+    if not os.path.exists(exe):
+        subprocess.run(["make", "-C", os.path.dirname(exe)], check=True, capture_output=True)
+    r = subprocess.run([exe], capture_output=True, text=True, timeout=100)
+    print(r.stdout, r.stderr, flush=True)
+    assert r.returncode == 0 and "c_abi ok" in r.stdout
