@@ -154,19 +154,21 @@ __device__ __forceinline__ void gemm_body(const unsigned char* __restrict__ w, c
     gemm_store<TBK>(acc, gs_ptr[0], y, rt, m0, rows, m_total, lane);
 }
 
-// Token blocks of 32 rows: a block is ONE row tile and one token block (blockIdx.y) whose panels are dealt to
-// its 4 waves (wave w: panels w, w + 4, ...), so that even a small M puts every SIMD to work.  Each wave stages
+// Token blocks of 16 TBK rows: a block is ONE row tile and one token block (blockIdx.y) whose panels are dealt to
+// its W waves (wave w: panels w, w + W, ...; W = 4 as launched: 8 measured slower at M = 16), so that even a small M puts
+// every SIMD to work.  Each wave stages
 // its own X panel in its own LDS region and reads it back itself: no block barrier in the loop.  The
 // four partial tiles are added in wave order through LDS at the end (deterministic).
+template <int TBK>
 __device__ __forceinline__ void gemm_small_body(const unsigned char* __restrict__ w, const unsigned short* __restrict__ x,
                                                 const float* __restrict__ gs_ptr, float* __restrict__ y, int k_dim, int rows,
                                                 int m_total, __bf16* xs_all) {
-    constexpr int TBK = 2;
     const int lane = lane_id();
     const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
     const int rt = (int)blockIdx.x, m0 = 32 * (int)blockIdx.y;
     const int panels = (k_dim + CROW_PANEL_COLS - 1) / CROW_PANEL_COLS;
-    __bf16* xs = xs_all + wave * (32 * CROW_GEMM_XS_STRIDE);
+    const int waves = block_threads() >> 6;  // 16 TBK staged rows per wave; the static LDS holds 128 rows
+    __bf16* xs = xs_all + wave * (16 * TBK * CROW_GEMM_XS_STRIDE);
     const __bf16* xs_lane = xs + (lane & 15) * CROW_GEMM_XS_STRIDE + (lane >> 4) * 8;
 
     f32x4 acc[TBK][4];
@@ -176,12 +178,12 @@ __device__ __forceinline__ void gemm_small_body(const unsigned char* __restrict_
         for (int j = 0; j < 4; j++) acc[tb][j] = f32x4{0.f, 0.f, 0.f, 0.f};
 
     const uint4* wt = (const uint4*)(w + (size_t)rt * panels * CROW_TILE_BYTES) + lane;
-    for (int p = wave; p < panels; p += 4) {
-        // 32 tokens x 256 columns = 1024 chunks of 16 bytes, 16 per lane; wave-private.  Fetched before the weight
+    for (int p = wave; p < panels; p += waves) {
+        // 16 TBK tokens x 256 columns = 512 TBK chunks of 16 bytes, 8 TBK per lane; wave-private.  Fetched before the weight
         // loads are issued so that they do not queue behind them.
-        uint4 xv[16];
+        uint4 xv[8 * TBK];
 #pragma unroll
-        for (int i = 0; i < 16; i++) {
+        for (int i = 0; i < 8 * TBK; i++) {
             const int c = i * 64 + lane, r = c >> 5, q = c & 31;
             const int k = p * CROW_PANEL_COLS + q * 8;
             xv[i] = make_uint4(0, 0, 0, 0);
@@ -193,7 +195,7 @@ __device__ __forceinline__ void gemm_small_body(const unsigned char* __restrict_
 #pragma unroll
         for (int s = 0; s < CROW_STEPS; s++) cd[s] = stream_load(t + 64 * (s + 1));
 #pragma unroll
-        for (int i = 0; i < 16; i++) {
+        for (int i = 0; i < 8 * TBK; i++) {
             const int c = i * 64 + lane, r = c >> 5, q = c & 31;
             *(uint4*)(xs + r * CROW_GEMM_XS_STRIDE + q * 8) = xv[i];
         }
@@ -201,7 +203,7 @@ __device__ __forceinline__ void gemm_small_body(const unsigned char* __restrict_
         gemm_panel<TBK>(sc, cd, xs_lane, acc);
         __builtin_amdgcn_wave_barrier();  // the tile is read before the next stage overwrites it
     }
-    // waves 1..3 -> wave 0 through LDS (each wave's own region is free now), added in wave order
+    // the other waves -> wave 0 through LDS (each wave's own region is free now), added in wave order
     float* red = (float*)xs;
     if (wave > 0) {
 #pragma unroll
@@ -213,8 +215,8 @@ __device__ __forceinline__ void gemm_small_body(const unsigned char* __restrict_
     }
     __syncthreads();
     if (wave > 0) return;
-    for (int ww = 1; ww < 4; ww++) {
-        const float* q = (const float*)(xs_all + ww * (32 * CROW_GEMM_XS_STRIDE));
+    for (int ww = 1; ww < waves; ww++) {
+        const float* q = (const float*)(xs_all + ww * (16 * TBK * CROW_GEMM_XS_STRIDE));
 #pragma unroll
         for (int tb = 0; tb < TBK; tb++)
 #pragma unroll
@@ -238,13 +240,15 @@ __device__ __forceinline__ void gemm_small_body(const unsigned char* __restrict_
         __shared__ __attribute__((aligned(16))) __bf16 xs[16 * TBK * CROW_GEMM_XS_STRIDE];                                     \
         crow::gemm_body<TBK>(w, x, gs_ptr, y, *k_dim_p, *rows_p, *m_p, xs);                                                    \
     }
-// token blocks of 32: grid (row_tiles, ceil(M / 32)), block 256
-extern "C" __global__ void __launch_bounds__(256, 2) gemm_nvfp4_bf16_m32(const unsigned char* __restrict__ w, const unsigned short* __restrict__ x,
+// token blocks of 32: grid (row_tiles, ceil(M / 32)), block 256 (any multiple of 64 up to 512 works: the waves deal the panels)
+extern "C" __global__ void __launch_bounds__(512) gemm_nvfp4_bf16_m32(const unsigned char* __restrict__ w, const unsigned short* __restrict__ x,
                                                                          const float* __restrict__ gs_ptr, float* __restrict__ y,
                                                                          const int* __restrict__ k_dim_p, const int* __restrict__ rows_p,
                                                                          const int* __restrict__ m_p) {
     __shared__ __attribute__((aligned(16))) __bf16 xs[4 * 32 * CROW_GEMM_XS_STRIDE];
-    crow::gemm_small_body(w, x, gs_ptr, y, *k_dim_p, *rows_p, *m_p, xs);
+    const int m = *m_p;
+    if (m <= 16) crow::gemm_small_body<1>(w, x, gs_ptr, y, *k_dim_p, *rows_p, m, xs);  // one 16-token block: half the matrix work and staging
+    else crow::gemm_small_body<2>(w, x, gs_ptr, y, *k_dim_p, *rows_p, m, xs);
 }
 CROW_GEMM_ENTRY(gemm_nvfp4_bf16_m64, 4, 3)
 CROW_GEMM_ENTRY(gemm_nvfp4_bf16, 8, 2)
