@@ -33,7 +33,7 @@ const FnEntry g_table[] = {
     CROW_FN(router_top10, 10),     CROW_FN(silu_mul_combo, 3),      CROW_FN(acc_combo, 3),
     CROW_FN(argmax_k, 3),          CROW_FN(argmax_tiles, 2),        CROW_FN(dequant_fp4_flat, 4),    CROW_FN(repack_nvfp4, 4),
     CROW_FN(unpack_nvfp4, 4),      CROW_FN(dequant_nvfp4_tiled, 5), CROW_FN(gemm_nvfp4_bf16, 7),
-    CROW_FN(gemm_nvfp4_bf16_m64, 7), CROW_FN(gemm_nvfp4_bf16_m32, 7), CROW_FN(gemv_bf16_w, 5),
+    CROW_FN(gemm_nvfp4_bf16_m64, 7), CROW_FN(gemm_nvfp4_bf16_m32, 7), CROW_FN(gemm_nvfp4_bf16_m16, 7), CROW_FN(gemv_bf16_w, 5),
 };
 const int g_table_n = (int)(sizeof(g_table) / sizeof(g_table[0]));
 
@@ -266,6 +266,14 @@ int crow_hip_launch_dims(const char* name, uint32_t rows, uint32_t k_dim, uint32
     }
     if (strncmp(name, "gemm_nvfp4_bf16", 15) == 0) {  // z = M token rows
         if (k_dim == 0 || k_dim % CROW_BLOCK_VALUES != 0) return CROW_ERR_SHAPE;
+        if (strcmp(name, "gemm_nvfp4_bf16_m16") == 0) {  // one panel per wave where the workspace allows it
+            if (z > 16) return CROW_ERR_SHAPE;
+            uint32_t s = (panels + 3) / 4;
+            if (s > 16) s = 16;
+            while (s > 1 && ((unsigned long long)rt * s * 16 * 64 > PARTIAL_FLOATS || rt > COUNTER_SLOTS)) s--;
+            *out = crow_dims{rt, 1, s, 256};
+            return CROW_OK;
+        }
         const uint32_t mt = strcmp(name, "gemm_nvfp4_bf16_m32") == 0 ? 32 : (strcmp(name, "gemm_nvfp4_bf16_m64") == 0 ? 64 : 128);
         if (mt == 32) {
             *out = crow_dims{rt, (z + 31) / 32, 1, 256};

@@ -17,7 +17,7 @@
 // The weight rows ride on the N side and the tokens on the M side, so a lane's 4 results of an instruction are
 // 4 tokens of one weight row and a store instruction writes four 64-byte runs of Y.
 #pragma once
-#include "device_common.h"
+#include "gemv.h"
 
 namespace crow {
 
@@ -167,7 +167,8 @@ __device__ __forceinline__ void gemm_small_body(const unsigned char* __restrict_
     const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
     const int rt = (int)blockIdx.x, m0 = 32 * (int)blockIdx.y;
     const int panels = (k_dim + CROW_PANEL_COLS - 1) / CROW_PANEL_COLS;
-    const int waves = block_threads() >> 6;  // 16 TBK staged rows per wave; the static LDS holds 128 rows
+    const int waves = block_threads() >> 6;  // 16 TBK staged rows per wave
+    const int slice = (int)blockIdx.z, slices = (int)gridDim.z;  // the panels may also be dealt over blocks (workspace hand-over)
     __bf16* xs = xs_all + wave * (16 * TBK * CROW_GEMM_XS_STRIDE);
     const __bf16* xs_lane = xs + (lane & 15) * CROW_GEMM_XS_STRIDE + (lane >> 4) * 8;
 
@@ -178,7 +179,7 @@ __device__ __forceinline__ void gemm_small_body(const unsigned char* __restrict_
         for (int j = 0; j < 4; j++) acc[tb][j] = f32x4{0.f, 0.f, 0.f, 0.f};
 
     const uint4* wt = (const uint4*)(w + (size_t)rt * panels * CROW_TILE_BYTES) + lane;
-    for (int p = wave; p < panels; p += waves) {
+    for (int p = slice * waves + wave; p < panels; p += slices * waves) {
         // 16 TBK tokens x 256 columns = 512 TBK chunks of 16 bytes, 8 TBK per lane; wave-private.  Fetched before the weight
         // loads are issued so that they do not queue behind them.
         uint4 xv[8 * TBK];
@@ -224,6 +225,22 @@ __device__ __forceinline__ void gemm_small_body(const unsigned char* __restrict_
 #pragma unroll
                 for (int r = 0; r < 4; r++) acc[tb][j][r] += q[((tb * 4 + j) * 4 + r) * 64 + lane];
     }
+    if (slices > 1) {  // slices of the row tile -> the block that arrives last, in slice order (the GEMV's protocol)
+        float v[16 * TBK];
+#pragma unroll
+        for (int tb = 0; tb < TBK; tb++)
+#pragma unroll
+            for (int j = 0; j < 4; j++)
+#pragma unroll
+                for (int r = 0; r < 4; r++) v[(tb * 4 + j) * 4 + r] = acc[tb][j][r];
+        if (!slice_hand_over<16 * TBK>(v, (unsigned)blockIdx.y * gridDim.x + blockIdx.x, slice, slices, g_ws, lane)) return;
+#pragma unroll
+        for (int tb = 0; tb < TBK; tb++)
+#pragma unroll
+            for (int j = 0; j < 4; j++)
+#pragma unroll
+                for (int r = 0; r < 4; r++) acc[tb][j][r] = v[(tb * 4 + j) * 4 + r];
+    }
     gemm_store<TBK>(acc, gs_ptr[0], y, rt, m0, rows, m_total, lane);
 }
 
@@ -249,6 +266,19 @@ extern "C" __global__ void __launch_bounds__(512) gemm_nvfp4_bf16_m32(const unsi
     const int m = *m_p;
     if (m <= 16) crow::gemm_small_body<1>(w, x, gs_ptr, y, *k_dim_p, *rows_p, m, xs);  // one 16-token block: half the matrix work and staging
     else crow::gemm_small_body<2>(w, x, gs_ptr, y, *k_dim_p, *rows_p, m, xs);
+}
+// M <= 16: one 16-token block, its panels dealt over grid.z blocks of 4 waves (one panel per wave at K = 5120): grid (row_tiles, 1, S)
+extern "C" __global__ void __launch_bounds__(256) gemm_nvfp4_bf16_m16(const unsigned char* __restrict__ w, const unsigned short* __restrict__ x,
+                                                                       const float* __restrict__ gs_ptr, float* __restrict__ y,
+                                                                       const int* __restrict__ k_dim_p, const int* __restrict__ rows_p,
+                                                                       const int* __restrict__ m_p) {
+    __shared__ __attribute__((aligned(16))) __bf16 xs[4 * 16 * CROW_GEMM_XS_STRIDE];
+    const int m = *m_p;
+    if (m > 16 || block_threads() > 256) {  // uniform over the launch
+        if (threadIdx.x == 0) atomicOr(crow::g_ws.status, crow::STATUS_BAD_SHAPE);
+        return;
+    }
+    crow::gemm_small_body<1>(w, x, gs_ptr, y, *k_dim_p, *rows_p, m, xs);
 }
 CROW_GEMM_ENTRY(gemm_nvfp4_bf16_m64, 4, 3)
 CROW_GEMM_ENTRY(gemm_nvfp4_bf16, 8, 2)

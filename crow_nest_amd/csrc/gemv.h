@@ -232,6 +232,50 @@ __device__ __forceinline__ void device_order() {
     asm volatile("" ::: "memory");
 }
 
+// The cross-block hand-over for any per-lane vector of NV partial sums (all of them live): the protocol the GEMV body uses,
+// for callers outside it.  Returns true in the block that arrived last, with `v` = the sum over slices in slice order;
+// false in every other block (which must not touch the output).  Wave-uniform control flow; call from one wave.
+template <int NV>
+__device__ __forceinline__ bool slice_hand_over(float (&v)[NV], unsigned tile_id, int slice, int slices, const Workspace& ws, int lane) {
+    const size_t need = ((size_t)tile_id + 1) * slices * NV * 64;
+    if (need > ws.partial_floats || tile_id >= ws.counter_slots) {
+        if (lane == 0) atomicOr(ws.status, STATUS_WORKSPACE_TOO_SMALL);
+        return false;
+    }
+    typedef __attribute__((address_space(1))) float* gf_p;
+    typedef __attribute__((address_space(1))) unsigned* gu_p;
+    gf_p base = (gf_p)ws.partials + (size_t)tile_id * slices * NV * 64;
+    gf_p mine = base + (size_t)slice * NV * 64;
+    gu_p counter = (gu_p)ws.counters + tile_id;
+#pragma unroll
+    for (int i = 0; i < NV; i++) __hip_atomic_store(mine + i * 64 + lane, v[i], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    device_order();
+    unsigned arrived = 0;
+    if (lane == 0) arrived = __hip_atomic_fetch_add(counter, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    arrived = __builtin_amdgcn_readfirstlane(arrived);
+    if (arrived != (unsigned)slices - 1) return false;
+    device_order();
+#pragma unroll
+    for (int i = 0; i < NV; i++) v[i] = 0.0f;
+    constexpr int PB = NV >= 32 ? 1 : (NV >= 16 ? 2 : 4);
+    for (int s0 = 0; s0 < slices; s0 += PB) {
+        float t[PB][NV];
+#pragma unroll
+        for (int j = 0; j < PB; j++)
+#pragma unroll
+            for (int i = 0; i < NV; i++)
+                t[j][i] = s0 + j < slices ? __hip_atomic_load(base + ((size_t)(s0 + j) * NV + i) * 64 + lane, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) : 0.0f;
+#pragma unroll
+        for (int j = 0; j < PB; j++)
+            if (s0 + j < slices) {
+#pragma unroll
+                for (int i = 0; i < NV; i++) v[i] += t[j][i];
+            }
+    }
+    if (lane == 0) __hip_atomic_store(counter, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    return true;
+}
+
 // out[r][m] in lane l = the wave's partial dot product of tile row l (of tensor r) with activation row m, summed
 // over panels p = p0, p0 + stride, ...  `xw` is the wave's own staging area, `zero` the block's zeroed 512 bytes.
 template <int NR, int M, bool XBF16>

@@ -204,7 +204,7 @@ class Engine:
     # ------------------------------------------------------------------ prefill GEMM (M >= 16)
     def gemm(self, w: Fp4, m: int, x: torch.Tensor, y: torch.Tensor | None = None, kernel: str | None = None) -> torch.Tensor:
         """Y[m][rows] = X[m][cols] W^T on the matrix cores (bf16 X, exact bf16 weight tiles, f32 accumulate).
-        `kernel` forces one of the three entry points (all take any m); default: gemm_kernel_for(m)."""
+        `kernel` forces one entry point (gemm_nvfp4_bf16_m16 takes m <= 16, the other three any m); default: gemm_kernel_for(m)."""
         rows, k = w.rows, w.cols
         assert x.is_cuda and x.is_contiguous() and x.dtype == torch.bfloat16 and x.numel() == m * k
         if y is None:
@@ -218,6 +218,9 @@ class Engine:
 
 def gemm_kernel_for(m: int) -> str:
     """Which GEMM entry point serves m token rows.  Up to 256 rows the K-split body (one row tile per block, its panels
-    dealt to the block's four waves, 32-token blocks on grid.y) keeps every SIMD busy; beyond that the body that shares
-    one staged X tile between four row tiles (64 tokens per wave) decodes the weights fewer times."""
+    dealt to the block's four waves, 32-token blocks on grid.y) keeps every SIMD busy; up to 16 rows the same body also
+    deals the panels over grid.z blocks (one panel per wave, partial tiles handed over through the workspace); beyond
+    256 the body that shares one staged X tile between four row tiles (64 tokens per wave) decodes the weights fewer times."""
+    if m <= 16:
+        return "gemm_nvfp4_bf16_m16"
     return "gemm_nvfp4_bf16_m32" if m <= 256 else "gemm_nvfp4_bf16_m64"
