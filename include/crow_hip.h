@@ -17,6 +17,7 @@
  * Kernel arguments keep the reference convention: every value handed to crow_hip_launch is a
  * 64-bit device address; scalars live in 4-byte device words.  Weight pointers are to tensors in
  * the library's tiled layout (crow_hip_repack_nvfp4), not to raw container bytes.
+ * crow_kernels.h lists every kernel name with its value list and the reference kernel it stands for.
  *
  * Threading: like the reference engine (one engine thread, one process-global current stream)
  * the library keeps one workspace per process; launches that use it must be ordered on one stream.

@@ -1,0 +1,101 @@
+/*
+ * The kernel table of libcrow_hip.so: every name crow_hip_module_get / crow_hip_get_function resolves, the values
+ * crow_hip_launch expects for it (in order, each a 64-bit device address; `*_p` = address of a 4-byte device word, as the
+ * reference's Params words), and the reference kernel whose call sites it serves.
+ *
+ * This header declares no C symbols: the kernels are reached by name through crow_hip_launch, exactly as the reference
+ * reaches its kernels through Kernels::f(name) + launch_v (engine/src/kernels.rs:5234,5296).  Include it with CROW_KERNEL
+ * defined to walk the table:
+ *     #define CROW_KERNEL(name, n_values) ...
+ *     #include "crow_kernels.h"
+ * Without a definition every line expands to nothing.  Grid and block sizes always come from crow_hip_launch_dims.
+ *
+ * Conventions shared by all entries:
+ *   w, wg, wu   NVFP4 tensors in the library's tiled layout (crow_hip_repack_nvfp4), never raw container bytes
+ *   gs, gs_*    one f32 per tensor: the global scale (PW::Fp4's second word, engine/src/gen.rs:234-237)
+ *   x           activations, row-major [tokens][k_dim]: f32 unless the entry is a *_bf16 twin (then bf16)
+ *   y           f32 outputs, row-major [tokens][rows]
+ *   A shape a kernel cannot serve sets a bit of the device status word (read by crow_hip_status) and the launch
+ *   writes nothing; no kernel traps.
+ */
+#ifndef CROW_KERNEL
+#define CROW_KERNEL(name, n_values)
+#define CROW_KERNEL_DEFAULTED_
+#endif
+
+/* ---- dense GEMV, one token ------------------------------------------------------------------------------------------ */
+/* w, x, gs, y, k_dim_p, rows_p.  gemv_nvfp4_w of engine/src/kernels_p2.rs:304-368 (rows_p appended: the reference reads
+ * the row count off its grid). */
+CROW_KERNEL(gemv_nvfp4_w, 6)
+CROW_KERNEL(gemv_nvfp4_w_bf16, 6) /* the same on bf16 x */
+/* w, x, gs, y, k_dim_p, rows_p.  gemv_fp4 of engine/src/kernels.rs:118-152 (the older one-block-per-row entry point the
+ * engine still calls for some tensors); same arithmetic as gemv_nvfp4_w here. */
+CROW_KERNEL(gemv_fp4, 6)
+/* w, x, gs, y(logits), k_dim_p, rows_p, out_idx.  lm_head_row (engine/src/gen.rs:4766-4784) with the first stage of
+ * argmax_k (engine/src/kernels.rs:4238-4260) fused: leaves one (value, index) candidate per 64-row tile in the library's
+ * workspace; argmax_tiles then writes the winner to out_idx[0].  Same tie order as argmax_k. */
+CROW_KERNEL(gemv_nvfp4_w_argmax, 7)
+CROW_KERNEL(argmax_tiles, 2) /* out_idx, rows_p */
+CROW_KERNEL(argmax_k, 3)     /* logits, out_idx, n_p.  engine/src/kernels.rs:4238-4260 */
+
+/* ---- fused gate / up + SiLU ----------------------------------------------------------------------------------------- */
+/* wg, wu, x, gs_g, gs_u, y, k_dim_p, rows_p.  gemv_nvfp4_gu of kernels_p2.rs:372-389: y = silu(gate x) * (up x). */
+CROW_KERNEL(gemv_nvfp4_gu, 8)
+CROW_KERNEL(gemv_nvfp4_gu_bf16, 8)
+
+/* ---- M <= 4 token rows (speculative verify) ----------------------------------------------------------------------- */
+/* w, x, gs, y, k_dim_p, rows_p, m_p.  gemv_nvfp4_wm of kernels_p2.rs:397-497; *m_p in 1..4 (NVFP4_MMAX), else the status
+ * word gets the bad-shape bit.  Row m of the result is bit-identical to a one-token launch on row m of x. */
+CROW_KERNEL(gemv_nvfp4_wm, 7)
+CROW_KERNEL(gemv_nvfp4_wm_bf16, 7)
+/* wg, wu, x, gs_g, gs_u, y, k_dim_p, rows_p, m_p.  gemv_nvfp4_gum of kernels_p2.rs:499-530. */
+CROW_KERNEL(gemv_nvfp4_gum, 9)
+CROW_KERNEL(gemv_nvfp4_gum_bf16, 9)
+/* w, x, gs, y, k_dim_p, rows_p, t_p.  gemv_fp4_b / gemv_fp4_b1k of kernels.rs:154-189,1302-1337: any token count t,
+ * four tokens per grid.z slice (rows_p and t_p appended). */
+CROW_KERNEL(gemv_fp4_b, 7)
+CROW_KERNEL(gemv_fp4_b1k, 7)
+/* w, x, gs, y, k_dim_p, y_stride_p, rows_p, t_p.  gemv_fp4_bs of kernels.rs:1022-1058: as gemv_fp4_b with a row stride
+ * on y. */
+CROW_KERNEL(gemv_fp4_bs, 8)
+
+/* ---- routed experts ------------------------------------------------------------------------------------------------- */
+/* logits, bitmap, ids, wts, gu_ptrs, dn_ptrs, table, cold_mask, counters, sel_counts.  router_top10 of
+ * kernels.rs:3109-3184: softmax, top-k with ties to the lowest id, renormalised weights, per-combo slab addresses gathered
+ * from table[E][2].  Geometry (experts, top-k) from crow_hip_set_geo. */
+CROW_KERNEL(router_top10, 10)
+/* ptrs, x, gs, y, k_dim_p, x_div_p, x_stride_p, rows_p.  gemv_fp4_ptrb of kernels.rs:195-233: combo c multiplies the slab
+ * at ptrs[c] by row c / *x_div_p of x (rows_p appended). */
+CROW_KERNEL(gemv_fp4_ptrb, 8)
+CROW_KERNEL(silu_mul_combo, 3) /* h1, h2, n_p.  kernels.rs:1562-1581 */
+CROW_KERNEL(acc_combo, 3)      /* x, rw, y.     kernels.rs:1583-1592 */
+/* ptrs, x, gs, h, k_dim_p, x_div_p, x_stride_p, inter_p.  gemv_fp4_ptrb on a fused gate_up slab + silu_mul_combo in one
+ * launch: h[c][i] = silu(gate_c x)[i] * (up_c x)[i]. */
+CROW_KERNEL(moe_gate_up_silu, 8)
+/* ptrs, h, gs, rw, y, k_dim_p, rows_p.  gemv_fp4_ptrb on the down slabs + acc_combo in one launch: y[t] = sum over the
+ * token's combos j, in j order, of rw[t][j] * (down_j h_j). */
+CROW_KERNEL(moe_down_combine, 7)
+
+/* ---- batched GEMM on the matrix cores (bf16 x, f32 y) ------------------------------------------------------------- */
+/* w, x, gs, y, k_dim_p, rows_p, m_p.  The dense NVFP4 GEMM of kernels_glm5_moe.cu:310-543 (gemm_fp4_dense's list minus
+ * the quantised-activation buffer: x is bf16).  gemm_nvfp4_bf16_m16 serves *m_p <= 16 only; the other three take any m
+ * and differ in tiling (32, 64, 128 tokens per block). */
+CROW_KERNEL(gemm_nvfp4_bf16, 7)
+CROW_KERNEL(gemm_nvfp4_bf16_m64, 7)
+CROW_KERNEL(gemm_nvfp4_bf16_m32, 7)
+CROW_KERNEL(gemm_nvfp4_bf16_m16, 7)
+
+/* ---- BF16 weights the container keeps unquantised (router, MTP head) ---------------------------------------------- */
+/* w(bf16 [rows][k_dim]), x, y, k_dim_p, rows_p.  gemv_bf16_w of kernels.rs:1130-1157; tokens on grid.y. */
+CROW_KERNEL(gemv_bf16_w, 5)
+
+/* ---- layout and decode ---------------------------------------------------------------------------------------------- */
+CROW_KERNEL(repack_nvfp4, 4)        /* src(container bytes), dst(tiled), rows_p, k_dim_p: what crow_hip_repack_nvfp4 launches */
+CROW_KERNEL(unpack_nvfp4, 4)        /* src(tiled), dst(container bytes), rows_p, k_dim_p */
+CROW_KERNEL(dequant_nvfp4_tiled, 5) /* w, gs, out(f32 [rows][k_dim]), rows_p, k_dim_p: bit-exact decode (cnq.rs:1298-1308) */
+CROW_KERNEL(dequant_fp4_flat, 4)    /* w(raw container bytes), gs, out, n_p.  dequant_fp4_flat of kernels.rs:1460, same list */
+
+#ifdef CROW_KERNEL_DEFAULTED_
+#undef CROW_KERNEL
+#undef CROW_KERNEL_DEFAULTED_
+#endif

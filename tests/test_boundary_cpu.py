@@ -45,6 +45,22 @@ def test_kernel_table_names_without_a_device():
     assert lib.crow_hip_tiled_bytes(1, 64) == 9216  # one padded tile
 
 
+def test_kernel_header_is_the_library_table():
+    """include/crow_kernels.h lists every kernel name with the number of values its launch takes: same set, same counts."""
+    import ctypes as C
+    text = open(os.path.join(ROOT, "include", "crow_kernels.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    listed = {m.group(1): int(m.group(2)) for m in re.finditer(r"^CROW_KERNEL\((\w+),\s*(\d+)\)", text, flags=re.M)}
+    lib = L.lib()
+    table = {}
+    for i in range(lib.crow_hip_function_count()):
+        name = lib.crow_hip_function_name(i)
+        f = C.c_void_p()
+        assert lib.crow_hip_get_function(name, C.byref(f)) == 0
+        table[name.decode()] = lib.crow_hip_function_arg_count(f)
+    assert listed == table
+
+
 def test_launch_dims_depend_on_the_matrix_only():
     import ctypes as C
     lib = L.lib()
