@@ -114,68 +114,85 @@ extern "C" __global__ void dequant_fp4_flat(const unsigned char* __restrict__ w,
 }
 
 // ------------------------------------------------------------------ router
-// reference: router_top10, engine/src/kernels.rs:3109-3184.  grid (T), block 64: one wavefront per
-// token, expert e lives in lane e % 64, slot e / 64.  The softmax denominator is added in the
-// reference's halving-tree order (slots first, then lanes), so weights match an E-thread tree.
-// Ties go to the lowest expert id.  E = g_geo.experts (power of two, 64..1024), K = g_geo.topk <= 16.
-// bitmap / cold_mask / counters / sel_counts / table / *_ptrs may be null (skipped).
-extern "C" __global__ void __launch_bounds__(64) router_top10(const float* __restrict__ logits, const unsigned int* __restrict__ bitmap,
-                                                              int* __restrict__ ids, float* __restrict__ wts,
-                                                              unsigned long long* __restrict__ gu_ptrs, unsigned long long* __restrict__ dn_ptrs,
-                                                              const unsigned long long* __restrict__ table, unsigned int* __restrict__ cold_mask,
-                                                              unsigned long long* __restrict__ counters, unsigned long long* __restrict__ sel_counts) {
-    const int E = g_geo.experts, K = g_geo.topk;
-    if (E < 64 || E > 1024 || (E & (E - 1)) != 0 || K < 1 || K > 16 || K > E) {
-        if (threadIdx.x == 0) atomicOr(g_ws.status, STATUS_BAD_GEO);
-        return;
-    }
-    const int t = (int)blockIdx.x, lane = lane_id(), slots = E >> 6;
-    float l[16], p[16];
+// Wave-wide maximum of an unsigned key through the data-parallel lane moves (an inclusive scan along the rows of 16
+// lanes, then the two row broadcasts; lane 63 ends with the maximum): six dependent vector instructions where a
+// butterfly of lane shuffles takes six round trips through the LDS crossbar.  All 64 lanes must be active.
+template <int CTRL, int ROW_MASK>
+__device__ __forceinline__ unsigned dpp_umax_step(unsigned v) {
+    const unsigned o = (unsigned)__builtin_amdgcn_update_dpp(0, (int)v, CTRL, ROW_MASK, 0xf, false);
+    return o > v ? o : v;
+}
+__device__ __forceinline__ unsigned wave_umax(unsigned v) {
+    v = dpp_umax_step<0x111, 0xf>(v);  // row_shr:1
+    v = dpp_umax_step<0x112, 0xf>(v);  // row_shr:2
+    v = dpp_umax_step<0x114, 0xf>(v);  // row_shr:4
+    v = dpp_umax_step<0x118, 0xf>(v);  // row_shr:8
+    v = dpp_umax_step<0x142, 0xa>(v);  // row_bcast:15 into rows 1 and 3
+    v = dpp_umax_step<0x143, 0xc>(v);  // row_bcast:31 into rows 2 and 3
+    return (unsigned)__builtin_amdgcn_readlane((int)v, 63);
+}
+
+// One token's routing on one wavefront, SLOTS = E / 64 experts per lane: expert e lives in lane e % 64, slot e / 64.
+template <int SLOTS>
+__device__ __forceinline__ void router_body(const float* __restrict__ logits, const unsigned int* __restrict__ bitmap, int* __restrict__ ids,
+                                            float* __restrict__ wts, unsigned long long* __restrict__ gu_ptrs,
+                                            unsigned long long* __restrict__ dn_ptrs, const unsigned long long* __restrict__ table,
+                                            unsigned int* __restrict__ cold_mask, unsigned long long* __restrict__ counters,
+                                            unsigned long long* __restrict__ sel_counts, int K) {
+    constexpr int E = SLOTS * 64;
+    const int t = (int)blockIdx.x, lane = lane_id();
+    float l[SLOTS], red[SLOTS];
     float mx = -INFINITY;
-    for (int j = 0; j < 16; j++) {
-        l[j] = j < slots ? logits[(size_t)t * E + j * 64 + lane] : -INFINITY;
+#pragma unroll
+    for (int j = 0; j < SLOTS; j++) {
+        l[j] = logits[(size_t)t * E + j * 64 + lane];
         mx = fmaxf(mx, l[j]);
     }
     for (int o = 32; o > 0; o >>= 1) mx = fmaxf(mx, __shfl_xor(mx, o));
-    float red[16];
-    for (int j = 0; j < 16; j++) red[j] = p[j] = j < slots ? expf(l[j] - mx) : 0.0f;
+#pragma unroll
+    for (int j = 0; j < SLOTS; j++) red[j] = l[j] = expf(l[j] - mx);
     // tree over E slots: strides E/2 .. 64 pair slots inside a lane, strides 32 .. 1 pair lanes
 #pragma unroll
-    for (int st = 8; st > 0; st >>= 1) {
-        if (st <= (slots >> 1)) {
+    for (int st = SLOTS / 2; st > 0; st >>= 1)
 #pragma unroll
-            for (int j = 0; j < st; j++) red[j] += red[j + st];
-        }
-    }
+        for (int j = 0; j < st; j++) red[j] += red[j + st];
     float den = red[0];
     for (int o = 32; o > 0; o >>= 1) den += __shfl_down(den, o);
     den = __shfl(den, 0);
-    for (int j = 0; j < 16; j++) p[j] = j < slots ? p[j] / den : -2.0f;
+    // keys: probabilities are >= 0, so their bit patterns order like the values; + 1 keeps 0 for "already picked"
+    unsigned key[SLOTS];
+#pragma unroll
+    for (int j = 0; j < SLOTS; j++) key[j] = __float_as_uint(l[j] / den) + 1u;
     float sum = 0.0f, my_w = 0.0f;
     int my_id = 0;
     for (int k = 0; k < K; k++) {
-        // key = (probability bits, inverted expert id): the maximum is the best probability, lowest id on ties
-        unsigned long long best = 0;
-        for (int j = 0; j < 16; j++) {
-            if (j < slots && p[j] >= 0.0f) {
-                const unsigned long long key = ((unsigned long long)__float_as_uint(p[j]) << 32) | (unsigned)(0xFFFFFFFFu - (unsigned)(j * 64 + lane));
-                best = key > best ? key : best;
+        unsigned best = key[0];
+        int best_id = lane;  // the lane's best: lowest slot (= lowest id in this lane) on ties
+#pragma unroll
+        for (int j = 1; j < SLOTS; j++)
+            if (key[j] > best) {
+                best = key[j];
+                best_id = j * 64 + lane;
             }
+        const unsigned top = wave_umax(best);
+        const unsigned long long tied = __ballot(best == top);
+        int pick;
+        if (__popcll(tied) == 1) {
+            pick = __builtin_amdgcn_readlane(best_id, (int)__builtin_ctzll(tied));
+        } else {  // equal probabilities in several lanes: the lowest expert id
+            const unsigned inv = best == top ? ~(unsigned)best_id : 0u;
+            pick = (int)~wave_umax(inv);
         }
-        for (int o = 32; o > 0; o >>= 1) {
-            const unsigned long long other = __shfl_xor(best, o);
-            best = other > best ? other : best;
-        }
-        const int pick = (int)(0xFFFFFFFFu - (unsigned)(best & 0xFFFFFFFFull));
-        const float pw = __uint_as_float((unsigned)(best >> 32));
+        const float pw = __uint_as_float(top - 1u);
         sum += pw;
         if (lane == k) {
             my_w = pw;
             my_id = pick;
         }
         if ((pick & 63) == lane) {
-            for (int j = 0; j < 16; j++)
-                if (j == (pick >> 6)) p[j] = -1.0f;
+#pragma unroll
+            for (int j = 0; j < SLOTS; j++)
+                if (j == (pick >> 6)) key[j] = 0u;
         }
     }
     unsigned cold = 0;
@@ -189,13 +206,39 @@ extern "C" __global__ void __launch_bounds__(64) router_top10(const float* __res
         if (sel_counts) atomicAdd(&sel_counts[my_id], 1ull);
         if (bitmap && !((bitmap[my_id >> 5] >> (my_id & 31)) & 1u)) cold = 1u << lane;
     }
-    for (int o = 32; o > 0; o >>= 1) cold |= __shfl_xor(cold, o);
-    if (lane == 0) {
-        if (cold_mask) cold_mask[t] = cold;
-        if (counters) {
-            atomicAdd(&counters[0], (unsigned long long)K);
-            atomicAdd(&counters[1], (unsigned long long)__popc(cold));
+    if (cold_mask || counters) {
+        for (int o = 32; o > 0; o >>= 1) cold |= __shfl_xor(cold, o);
+        if (lane == 0) {
+            if (cold_mask) cold_mask[t] = cold;
+            if (counters) {
+                atomicAdd(&counters[0], (unsigned long long)K);
+                atomicAdd(&counters[1], (unsigned long long)__popc(cold));
+            }
         }
+    }
+}
+
+// reference: router_top10, engine/src/kernels.rs:3109-3184.  grid (T), block 64: one wavefront per
+// token.  The softmax denominator is added in the reference's halving-tree order (slots first, then
+// lanes), so weights match an E-thread tree.  Ties go to the lowest expert id.
+// E = g_geo.experts (power of two, 64..1024), K = g_geo.topk <= 16.
+// bitmap / cold_mask / counters / sel_counts / table / *_ptrs may be null (skipped).
+extern "C" __global__ void __launch_bounds__(64) router_top10(const float* __restrict__ logits, const unsigned int* __restrict__ bitmap,
+                                                              int* __restrict__ ids, float* __restrict__ wts,
+                                                              unsigned long long* __restrict__ gu_ptrs, unsigned long long* __restrict__ dn_ptrs,
+                                                              const unsigned long long* __restrict__ table, unsigned int* __restrict__ cold_mask,
+                                                              unsigned long long* __restrict__ counters, unsigned long long* __restrict__ sel_counts) {
+    const int E = g_geo.experts, K = g_geo.topk;
+    if (E < 64 || E > 1024 || (E & (E - 1)) != 0 || K < 1 || K > 16 || K > E || block_threads() != 64) {
+        if (threadIdx.x == 0) atomicOr(g_ws.status, STATUS_BAD_GEO);
+        return;
+    }
+    switch (E >> 6) {
+        case 1: router_body<1>(logits, bitmap, ids, wts, gu_ptrs, dn_ptrs, table, cold_mask, counters, sel_counts, K); break;
+        case 2: router_body<2>(logits, bitmap, ids, wts, gu_ptrs, dn_ptrs, table, cold_mask, counters, sel_counts, K); break;
+        case 4: router_body<4>(logits, bitmap, ids, wts, gu_ptrs, dn_ptrs, table, cold_mask, counters, sel_counts, K); break;
+        case 8: router_body<8>(logits, bitmap, ids, wts, gu_ptrs, dn_ptrs, table, cold_mask, counters, sel_counts, K); break;
+        default: router_body<16>(logits, bitmap, ids, wts, gu_ptrs, dn_ptrs, table, cold_mask, counters, sel_counts, K); break;
     }
 }
 

@@ -253,6 +253,33 @@ def test_router_small_kernels(eng):
     eng.check()
 
 
+@pytest.mark.parametrize("experts,topk", [(64, 4), (128, 8), (512, 10), (1024, 16)])
+def test_router_other_geometries_and_ties(eng, experts, topk):
+    """Expert counts from one to sixteen per lane; equal logits in several lanes and inside one lane (ties go to the
+    lowest expert id); a whole row of equal logits."""
+    from crow_nest_amd.kernels import KernelGeo, launch_v, set_geo
+    print(f"case experts={experts} topk={topk}", flush=True)
+    g = np.random.default_rng(experts)
+    logits = g.standard_normal((6, experts)).astype(np.float32)
+    logits[1, [5, 5 + 64 % experts, experts - 1, 17]] = 3.5  # same lane (where experts > 64) and other lanes
+    logits[2, :] = 0.25                                       # everything ties: ids 0 .. topk-1
+    logits[3, experts // 2:] = logits[3, : experts // 2]     # every value twice, 'experts / 2' apart
+    logits[4, [experts - 1, experts - 2]] = 9.0
+    try:
+        set_geo(KernelGeo(experts=experts, topk=topk, hidden=2048, inter=512))
+        ld = _dev(logits)
+        ids = torch.empty((6, topk), dtype=torch.int32, device="cuda")
+        wts = torch.empty((6, topk), dtype=torch.float32, device="cuda")
+        launch_v(eng.k.f("router_top10"), 6, 1, 1, 64, [ld.data_ptr(), 0, ids.data_ptr(), wts.data_ptr(), 0, 0, 0, 0, 0, 0])
+        eng.check()
+    finally:
+        set_geo(eng.geo)
+    ids_ref, w_ref = orc.router_topk(logits, topk)
+    assert np.array_equal(ids.cpu().numpy(), ids_ref)
+    assert np.allclose(wts.cpu().numpy(), w_ref, rtol=2e-6, atol=0)
+    assert ids_ref[2].tolist() == list(range(topk))
+
+
 @pytest.mark.parametrize("t", [1, 4])
 def test_moe_layer_both_launch_sequences(eng, t):
     from crow_nest_amd.engine import MoeW, expert_table
