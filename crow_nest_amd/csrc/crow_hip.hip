@@ -45,6 +45,7 @@ struct State {
     crow::Workspace ws{};
     int* scalars = nullptr;  // two device words for the library's own launches (rows, k_dim)
     char name[256] = {0};
+    int geo_topk = 0;  // host copy of the routed geometry (crow_hip_set_geo), for launch shapes
 } g;
 
 const unsigned long long PARTIAL_FLOATS = 16ull << 20;  // 64 MiB of split-K partial sums
@@ -198,7 +199,9 @@ int crow_hip_set_geo(int experts, int topk, int hidden, int inter) {
     crow::Geo geo{experts, topk, hidden, inter};
     hipError_t e = hipMemcpyToSymbolAsync(HIP_SYMBOL(crow::g_geo), &geo, sizeof geo, 0, hipMemcpyHostToDevice, g.stream);
     if (e != hipSuccess) return (int)e;
-    return hip_rc(hipStreamSynchronize(g.stream));
+    if ((e = hipStreamSynchronize(g.stream)) != hipSuccess) return (int)e;
+    g.geo_topk = topk;
+    return CROW_OK;
 }
 
 int crow_hip_launch(crow_fn_t f, uint32_t gx, uint32_t gy, uint32_t gz, uint32_t bx, const uint64_t* vals, uint32_t n_vals,
@@ -282,8 +285,9 @@ int crow_hip_launch_dims(const char* name, uint32_t rows, uint32_t k_dim, uint32
         }
         return CROW_OK;
     }
-    if (strcmp(name, "moe_down_combine") == 0) {
-        out->gx = 1; out->gy = rt; out->gz = z; out->bx = 64 * (g.ready ? 1 : 1);
+    if (strcmp(name, "moe_down_combine") == 0) {  // rows = hidden; one wave per picked expert
+        if (g.geo_topk < 1 || g.geo_topk > 16) return CROW_ERR_GEO;
+        *out = crow_dims{1, rt, z, 64u * (uint32_t)g.geo_topk};
         return CROW_OK;
     }
     if (strcmp(name, "repack_nvfp4") == 0 || strcmp(name, "unpack_nvfp4") == 0 || strcmp(name, "dequant_nvfp4_tiled") == 0) {

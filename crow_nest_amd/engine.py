@@ -173,7 +173,7 @@ class Engine:
             gx, gy, gz, bx = launch_dims("moe_gate_up_silu", inter, hdim, combos)
             launch_v(self.k.f("moe_gate_up_silu"), gx, gy, gz, bx,
                      [gu.data_ptr(), x.data_ptr(), gs_gu, h2.data_ptr(), p.i32(hdim), p.i32(topk), p.i32(hdim), p.i32(inter)])
-            launch_v(self.k.f("moe_down_combine"), 1, (hdim + 63) // 64, t, 64 * topk,
+            launch_v(self.k.f("moe_down_combine"), *launch_dims("moe_down_combine", hdim, inter, t),
                      [dn.data_ptr(), h2.data_ptr(), gs_dn, wts.data_ptr(), y.data_ptr(), p.i32(inter), p.i32(hdim)])
         else:
             h1 = torch.empty((combos, 2 * inter), dtype=torch.float32, device=self.dev)

@@ -294,7 +294,9 @@ def test_moe_layer_both_launch_sequences(eng, t):
     logits = normal_f32(6, t, t * E).reshape(t, E)
     ids_ref, w_ref, y_ref = orc.moe_layer(gu, gs_gu, dn, gs_dn, E, H, I, x, logits, K, threads=8)
     for fused in (False, True):
+        print(f"case moe t={t} fused={fused}", flush=True)
         ids, wts, y = eng.moe_run(moe, _dev(x), _dev(logits), fused=fused)
+        eng.check()
         assert np.array_equal(ids.cpu().numpy(), ids_ref)
         assert np.allclose(wts.cpu().numpy(), w_ref, rtol=2e-6, atol=0)
         assert rel_err(y.cpu().numpy(), y_ref) <= TOL, fused
