@@ -32,8 +32,11 @@ const FnEntry g_table[] = {
     CROW_GEMV(gemv_fp4_ptrb, 8, 1, 1, 4),      CROW_GEMV(moe_gate_up_silu, 8, 1, 1, 4),   CROW_GEMV(moe_down_combine, 7, 1, 1, 4),
     CROW_FN(router_top10, 10),     CROW_FN(silu_mul_combo, 3),      CROW_FN(acc_combo, 3),
     CROW_FN(argmax_k, 3),          CROW_FN(argmax_tiles, 2),        CROW_FN(dequant_fp4_flat, 4),    CROW_FN(repack_nvfp4, 4),
-    CROW_FN(unpack_nvfp4, 4),      CROW_FN(dequant_nvfp4_tiled, 5), CROW_FN(gemm_nvfp4_bf16, 7),
-    CROW_FN(gemm_nvfp4_bf16_m64, 7), CROW_FN(gemm_nvfp4_bf16_m32, 7), CROW_FN(gemm_nvfp4_bf16_m16, 7), CROW_FN(gemv_bf16_w, 5),
+    CROW_FN(unpack_nvfp4, 4),      CROW_FN(dequant_nvfp4_tiled, 5),
+    // shared-X GEMM blocks: two staged X tiles of MT rows x 528 bytes
+    {"gemm_nvfp4_bf16", (const void*)&gemm_nvfp4_bf16, 7, 2u * 128u * 528u, 0u},
+    {"gemm_nvfp4_bf16_m64", (const void*)&gemm_nvfp4_bf16_m64, 7, 2u * 64u * 528u, 0u},
+    CROW_FN(gemm_nvfp4_bf16_m32, 7), CROW_FN(gemm_nvfp4_bf16_m16, 7), CROW_FN(gemv_bf16_w, 5),
 };
 const int g_table_n = (int)(sizeof(g_table) / sizeof(g_table[0]));
 

@@ -105,55 +105,6 @@ __device__ __forceinline__ void gemm_store(const f32x4 (&acc)[TBK][4], float gs,
     }
 }
 
-// Block = 4 waves; wave w owns row tile 4 * blockIdx.x + w and all of the block's MT = 16 * TBK token rows.
-template <int TBK>
-__device__ __forceinline__ void gemm_body(const unsigned char* __restrict__ w, const unsigned short* __restrict__ x,
-                                          const float* __restrict__ gs_ptr, float* __restrict__ y, int k_dim, int rows, int m_total,
-                                          __bf16* xs) {
-    constexpr int MT = 16 * TBK;
-    const int lane = lane_id();
-    const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
-    const int row_tiles = (rows + CROW_TILE_ROWS - 1) / CROW_TILE_ROWS;
-    const int rt = (int)blockIdx.x * 4 + wave;
-    const bool has_rows = rt < row_tiles;  // wave-uniform; idle waves still join the barriers
-    const int m0 = (int)blockIdx.y * MT;
-    const int panels = (k_dim + CROW_PANEL_COLS - 1) / CROW_PANEL_COLS;
-
-    f32x4 acc[TBK][4];
-#pragma unroll
-    for (int tb = 0; tb < TBK; tb++)
-#pragma unroll
-        for (int j = 0; j < 4; j++) acc[tb][j] = f32x4{0.f, 0.f, 0.f, 0.f};
-
-    // this lane's fixed read position in the staged X tile: token lane % 16, columns 8 * (lane / 16) .. of a segment
-    const __bf16* xs_lane = xs + (lane & 15) * CROW_GEMM_XS_STRIDE + (lane >> 4) * 8;
-    const uint4* wt = (const uint4*)(w + (size_t)rt * panels * CROW_TILE_BYTES) + lane;
-    for (int p = 0; p < panels; p++) {
-        uint4 sc = make_uint4(0, 0, 0, 0), cd[CROW_STEPS];
-#pragma unroll
-        for (int s = 0; s < CROW_STEPS; s++) cd[s] = make_uint4(0, 0, 0, 0);
-        if (has_rows) {
-            const uint4* t = wt + (size_t)p * (CROW_TILE_BYTES / 16);
-            sc = stream_load(t);
-#pragma unroll
-            for (int s = 0; s < CROW_STEPS; s++) cd[s] = stream_load(t + 64 * (s + 1));
-        }
-        // X[m0 .. m0 + MT][256 p .. 256 p + 255] (zero beyond M and K): MT * 32 chunks of 16 bytes
-        __syncthreads();  // the previous panel's reads are done
-        for (int c = (int)threadIdx.x; c < MT * 32; c += 256) {
-            const int r = c >> 5, q = c & 31;
-            const int m = m0 + r, k = p * CROW_PANEL_COLS + q * 8;
-            uint4 v = make_uint4(0, 0, 0, 0);
-            if (m < m_total && k < k_dim) v = *(const uint4*)(x + (size_t)m * k_dim + k);
-            *(uint4*)(xs + r * CROW_GEMM_XS_STRIDE + q * 8) = v;
-        }
-        __syncthreads();
-        gemm_panel<TBK>(sc, cd, xs_lane, acc);
-    }
-    if (!has_rows) return;
-    gemm_store<TBK>(acc, gs_ptr[0], y, rt, m0, rows, m_total, lane);
-}
-
 // Token blocks of 16 TBK rows: a block is ONE row tile and one token block (blockIdx.y) whose panels are dealt to
 // its W waves (wave w: panels w, w + W, ...; W = 4 as launched: 8 measured slower at M = 16), so that even a small M puts
 // every SIMD to work.  Each wave stages
@@ -244,19 +195,88 @@ __device__ __forceinline__ void gemm_small_body(const unsigned char* __restrict_
     gemm_store<TBK>(acc, gs_ptr[0], y, rt, m0, rows, m_total, lane);
 }
 
+// Shared X: block = 4 waves; wave w owns row tile 4 * blockIdx.x + w and all of the block's MT = 16 * TBK token rows, staged
+// once in LDS for the four row tiles.  The memory traffic of panel p + 1 is in flight while panel p is computed: the next
+// weight tile waits in a second register set and the next X tile in registers, written to the OTHER LDS buffer after the
+// compute, so one block barrier per panel (these kernels run one or two waves per SIMD: nothing else hides the latency).
+template <int TBK>
+__device__ __forceinline__ void gemm_pipe_body(const unsigned char* __restrict__ w, const unsigned short* __restrict__ x,
+                                               const float* __restrict__ gs_ptr, float* __restrict__ y, int k_dim, int rows, int m_total,
+                                               __bf16* xs2) {
+    constexpr int MT = 16 * TBK;
+    constexpr int XCH = MT * 32 / 256;  // 16-byte chunks of an X tile per thread
+    constexpr int XBUF = MT * CROW_GEMM_XS_STRIDE;
+    const int lane = lane_id();
+    const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
+    const int row_tiles = (rows + CROW_TILE_ROWS - 1) / CROW_TILE_ROWS;
+    const int rt = (int)blockIdx.x * 4 + wave;
+    const bool has_rows = rt < row_tiles;  // wave-uniform; idle waves still stage X and join the barriers
+    const int m0 = (int)blockIdx.y * MT;
+    const int panels = (k_dim + CROW_PANEL_COLS - 1) / CROW_PANEL_COLS;
+
+    f32x4 acc[TBK][4];
+#pragma unroll
+    for (int tb = 0; tb < TBK; tb++)
+#pragma unroll
+        for (int j = 0; j < 4; j++) acc[tb][j] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+    const uint4* wt = (const uint4*)(w + (size_t)(has_rows ? rt : 0) * panels * CROW_TILE_BYTES) + lane;
+    auto load_w = [&](int p, uint4& sc, uint4 (&cd)[CROW_STEPS]) {
+        const uint4* t = wt + (size_t)p * (CROW_TILE_BYTES / 16);
+        sc = stream_load(t);
+#pragma unroll
+        for (int s = 0; s < CROW_STEPS; s++) cd[s] = stream_load(t + 64 * (s + 1));
+    };
+    // chunk c = i * 256 + thread: token row c / 32, 8 columns from 8 (c % 32)
+    auto load_x = [&](int p, uint4 (&xv)[XCH]) {
+#pragma unroll
+        for (int i = 0; i < XCH; i++) {
+            const int c = i * 256 + (int)threadIdx.x, r = c >> 5, q = c & 31;
+            const int m = m0 + r, k = p * CROW_PANEL_COLS + q * 8;
+            xv[i] = make_uint4(0, 0, 0, 0);
+            if (m < m_total && k < k_dim) xv[i] = *(const uint4*)(x + (size_t)m * k_dim + k);
+        }
+    };
+    auto store_x = [&](__bf16* xs, const uint4 (&xv)[XCH]) {
+#pragma unroll
+        for (int i = 0; i < XCH; i++) {
+            const int c = i * 256 + (int)threadIdx.x, r = c >> 5, q = c & 31;
+            *(uint4*)(xs + r * CROW_GEMM_XS_STRIDE + q * 8) = xv[i];
+        }
+    };
+    const int lane_off = (lane & 15) * CROW_GEMM_XS_STRIDE + (lane >> 4) * 8;
+
+    uint4 sc[2], cd[2][CROW_STEPS], xv[XCH];
+    load_x(0, xv);
+    load_w(0, sc[0], cd[0]);
+    store_x(xs2, xv);
+    __syncthreads();
+    // two panels per trip so that the register sets swap roles without copies
+    for (int p = 0; p < panels; p += 2) {
+#pragma unroll
+        for (int h = 0; h < 2; h++) {
+            const int pp = p + h;
+            if (pp < panels) {
+                const bool more = pp + 1 < panels;
+                if (more) {
+                    load_x(pp + 1, xv);
+                    load_w(pp + 1, sc[h ^ 1], cd[h ^ 1]);
+                }
+                gemm_panel<TBK>(sc[h], cd[h], xs2 + h * XBUF + lane_off, acc);
+                if (more) store_x(xs2 + (h ^ 1) * XBUF, xv);
+                __syncthreads();  // the other buffer is written, and this one read, by every wave
+            }
+        }
+    }
+    if (!has_rows) return;
+    gemm_store<TBK>(acc, gs_ptr[0], y, rt, m0, rows, m_total, lane);
+}
+
 }  // namespace crow
 
 // Y[M][rows] f32 = X[M][k_dim] bf16 times the tiled NVFP4 tensor, times gs.  The argument list is
 // gemm_fp4_dense's (engine/src/kernels.rs:533-541) without the quantised-activation buffer: x is bf16.
 // grid (ceil(row_tiles / 4), ceil(M / MT)), block 256, MT = 64 / 128 for the two general entry points.
-#define CROW_GEMM_ENTRY(NAME, TBK, OCC)                                                                                       \
-    extern "C" __global__ void __launch_bounds__(256, OCC) NAME(const unsigned char* __restrict__ w, const unsigned short* __restrict__ x, \
-                                                           const float* __restrict__ gs_ptr, float* __restrict__ y,            \
-                                                           const int* __restrict__ k_dim_p, const int* __restrict__ rows_p,    \
-                                                           const int* __restrict__ m_p) {                                      \
-        __shared__ __attribute__((aligned(16))) __bf16 xs[16 * TBK * CROW_GEMM_XS_STRIDE];                                     \
-        crow::gemm_body<TBK>(w, x, gs_ptr, y, *k_dim_p, *rows_p, *m_p, xs);                                                    \
-    }
 // token blocks of 32: grid (row_tiles, ceil(M / 32)), block 256 (any multiple of 64 up to 512 works: the waves deal the panels)
 extern "C" __global__ void __launch_bounds__(512) gemm_nvfp4_bf16_m32(const unsigned char* __restrict__ w, const unsigned short* __restrict__ x,
                                                                          const float* __restrict__ gs_ptr, float* __restrict__ y,
@@ -280,5 +300,17 @@ extern "C" __global__ void __launch_bounds__(256) gemm_nvfp4_bf16_m16(const unsi
     }
     crow::gemm_small_body<1>(w, x, gs_ptr, y, *k_dim_p, *rows_p, m, xs);
 }
-CROW_GEMM_ENTRY(gemm_nvfp4_bf16_m64, 4, 3)
-CROW_GEMM_ENTRY(gemm_nvfp4_bf16, 8, 2)
+// the shared-X body: grid (ceil(row_tiles / 4), ceil(M / MT)), block 256, MT = 16 TBK = 64 / 128 tokens; dynamic LDS = two X tiles
+#define CROW_GEMM_PIPE_ENTRY(NAME, TBK, OCC)                                                                                   \
+    extern "C" __global__ void __launch_bounds__(256, OCC) NAME(const unsigned char* __restrict__ w, const unsigned short* __restrict__ x, \
+                                                           const float* __restrict__ gs_ptr, float* __restrict__ y,            \
+                                                           const int* __restrict__ k_dim_p, const int* __restrict__ rows_p,    \
+                                                           const int* __restrict__ m_p) {                                      \
+        if (block_threads() != 256 || *m_p < 1) {                                                                              \
+            if (threadIdx.x == 0) atomicOr(crow::g_ws.status, crow::STATUS_BAD_SHAPE);                                         \
+            return;                                                                                                            \
+        }                                                                                                                      \
+        crow::gemm_pipe_body<TBK>(w, x, gs_ptr, y, *k_dim_p, *rows_p, *m_p, (__bf16*)crow_dyn_lds);                            \
+    }
+CROW_GEMM_PIPE_ENTRY(gemm_nvfp4_bf16_m64, 4, 2)
+CROW_GEMM_PIPE_ENTRY(gemm_nvfp4_bf16, 8, 1)

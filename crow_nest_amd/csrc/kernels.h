@@ -29,7 +29,7 @@ extern "C" __global__ void __launch_bounds__(1024) gemv_nvfp4_w(const unsigned c
     GemvArgs a{{w, nullptr}, {gs_ptr, nullptr}, x, 0, y, 0, *k_dim_p, *rows_p, 1, nullptr};
     gemv_body<1, 1, false, EPI_SCALE, XRows<1, false>::value>(a, 0, LDS, ws);
 }
-// the same product on bf16 activations (exact widening; BASELINE configs quote X in bf16)
+// the same product on bf16 activations (exact widening), for models that keep their activations in bf16
 extern "C" __global__ void __launch_bounds__(1024) gemv_nvfp4_w_bf16(const unsigned char* __restrict__ w, const unsigned short* __restrict__ x,
                                                                      const float* __restrict__ gs_ptr, float* __restrict__ y,
                                                                      const int* __restrict__ k_dim_p, const int* __restrict__ rows_p) {
@@ -71,7 +71,7 @@ extern "C" __global__ void __launch_bounds__(1024) gemv_nvfp4_gu(const unsigned 
     gemv_body<2, 1, false, EPI_SILU_GU, XRows<1, false>::value, true>(a, 0, LDS, ws);
 }
 
-// the same on bf16 activations (BASELINE quotes X in bf16; exact widening)
+// the same on bf16 activations (exact widening)
 extern "C" __global__ void __launch_bounds__(1024) gemv_nvfp4_gu_bf16(const unsigned char* __restrict__ wg, const unsigned char* __restrict__ wu,
                                                                       const unsigned short* __restrict__ x, const float* __restrict__ gs_g,
                                                                       const float* __restrict__ gs_u, float* __restrict__ y,

@@ -217,10 +217,10 @@ class Engine:
 
 
 def gemm_kernel_for(m: int) -> str:
-    """Which GEMM entry point serves m token rows.  Up to 256 rows the K-split body (one row tile per block, its panels
+    """Which GEMM entry point serves m token rows.  Up to 128 rows the K-split body (one row tile per block, its panels
     dealt to the block's four waves, 32-token blocks on grid.y) keeps every SIMD busy; up to 16 rows the same body also
     deals the panels over grid.z blocks (one panel per wave, partial tiles handed over through the workspace); beyond
-    256 the body that shares one staged X tile between four row tiles (64 tokens per wave) decodes the weights fewer times."""
+    128 the body that shares one staged X tile between four row tiles (64 tokens per wave) decodes the weights fewer times."""
     if m <= 16:
         return "gemm_nvfp4_bf16_m16"
-    return "gemm_nvfp4_bf16_m32" if m <= 256 else "gemm_nvfp4_bf16_m64"
+    return "gemm_nvfp4_bf16_m32" if m <= 128 else "gemm_nvfp4_bf16_m64"
