@@ -322,6 +322,65 @@ def test_config0_full_size(eng):
     assert np.array_equal(d.view(np.uint32), orc.dequant(w[:256 * cols // 64 * 36], gs).view(np.uint32))
 
 
+# ---------------------------------------------------------------- BASELINE config 1 at full size
+
+def test_config1_full_size_properties(eng):
+    """[17408, 5120] gate / up and [5120, 17408] down, BASELINE's weights and bf16 X, four token rows: sampled row slabs
+    against the CPU path, every row of the four-row launch bit-identical to its own one-row launch, and the down
+    projection exactly linear under power-of-two scaling."""
+    from crow_nest_amd.engine import MlpW
+    H, I, T = 5120, 17408, 4
+    (wg, gg), (wu, gu), (wd, gd) = quantized_normal(0, 0, I, H), quantized_normal(0, 1, I, H), quantized_normal(0, 2, H, I)
+    mlp = MlpW(_load(wg, I, H, gg), _load(wu, I, H, gu), _load(wd, H, I, gd))
+    xb, xw = _bf16_dev(normal_f32(0, 3, T * H))
+    xb, xw = xb.reshape(T, H).contiguous(), xw.reshape(T, H)
+    h4 = eng.gate_up(mlp, T, xb)
+    eng.check()
+    h = h4.cpu().numpy()
+    rb = H // 64 * 36
+    for r0 in (0, 8704 - 64, I - 128):
+        g_ref = orc.gemv(wg[r0 * rb:(r0 + 128) * rb], 128, H, gg, xw, threads=8)
+        u_ref = orc.gemv(wu[r0 * rb:(r0 + 128) * rb], 128, H, gu, xw, threads=8)
+        assert rel_err(h[:, r0:r0 + 128], orc.silu_mul(g_ref, u_ref)) <= TOL, r0
+    for t in range(T):
+        h1 = eng.gate_up(mlp, 1, xb[t:t + 1].contiguous()).cpu().numpy()
+        assert np.array_equal(h1.view(np.uint32)[0], h.view(np.uint32)[t]), t
+    y = eng.dense_proj(mlp.down, T, h4).cpu().numpy()
+    eng.check()
+    rbd = I // 64 * 36
+    for r0 in (0, H - 256):
+        assert rel_err(y[:, r0:r0 + 256], orc.gemv(wd[r0 * rbd:(r0 + 256) * rbd], 256, I, gd, h, threads=8)) <= TOL, r0
+    y8 = eng.dense_proj(mlp.down, T, (h4 * 8.0).contiguous()).cpu().numpy()
+    assert np.array_equal(y8.view(np.uint32), (y * np.float32(8.0)).view(np.uint32))
+    for t in (0, 3):
+        y1 = eng.dense_proj(mlp.down, 1, h4[t:t + 1].contiguous()).cpu().numpy()
+        assert np.array_equal(y1.view(np.uint32)[0], y.view(np.uint32)[t]), t
+
+
+# ---------------------------------------------------------------- BASELINE config 3 at full size
+
+def test_config3_full_size_head(eng):
+    """[151936, 5120] head (random codes and scales: the encoder is not what is tested here): sampled row slabs against the
+    CPU path, the fused argmax against the argmax of the logits the device wrote, fused and two-kernel forms equal."""
+    rows, cols = 151936, 5120
+    w = random_nvfp4(77, rows, cols, scale_lo=0x30, scale_hi=0x50, p7f=0)
+    gs = 1.0e-3
+    f = _load(w, rows, cols, gs)
+    x = normal_f32(0, 5, cols)
+    logits, idx = eng.lm_head_row(f, _dev(x), fused=True)
+    eng.check()
+    got = logits.cpu().numpy().reshape(-1)
+    rb = cols // 64 * 36
+    for r0 in (0, 75968 - 100, rows - 256):
+        ref = orc.gemv(w[r0 * rb:(r0 + 256) * rb], 256, cols, gs, x, threads=8)[0]
+        assert rel_err(got[r0:r0 + 256], ref) <= TOL, r0
+    assert int(idx.item()) == orc.argmax_ref(got) == int(np.argmax(got))
+    logits2, idx2 = eng.lm_head_row(f, _dev(x), fused=False)
+    assert np.array_equal(logits2.cpu().numpy().reshape(-1).view(np.uint32), got.view(np.uint32))
+    assert int(idx2.item()) == int(idx.item())
+    eng.check()
+
+
 # ---------------------------------------------------------------- batched GEMM on the matrix cores (config 4)
 
 @pytest.mark.parametrize("kernel", ["gemm_nvfp4_bf16_m16", "gemm_nvfp4_bf16_m32", "gemm_nvfp4_bf16_m64", "gemm_nvfp4_bf16"])
