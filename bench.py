@@ -240,7 +240,7 @@ def main() -> int:
         for m in (16, 128, 512):
             xm = torch.randn(m, K, device=dev).to(torch.bfloat16)
             ym = torch.empty(m, N, dtype=torch.float32, device=dev)
-            nm = gemm_kernel_for(m)
+            nm = gemm_kernel_for(m, N)
             l4 = Launch(eng, nm, N, K, m, [[s["gate"].data_ptr(), xm.data_ptr(), gs1.data_ptr(), ym.data_ptr(), p.i32(K), p.i32(N), p.i32(m)] for s in sets])
             us = l4.us(iters=50)
             e = entry(us, W_BYTES + m * K * 2 + m * N * 4)

@@ -36,6 +36,8 @@ const FnEntry g_table[] = {
     // shared-X GEMM blocks: two staged X tiles of MT rows x 528 bytes
     {"gemm_nvfp4_bf16", (const void*)&gemm_nvfp4_bf16, 7, 2u * 128u * 528u, 0u},
     {"gemm_nvfp4_bf16_m64", (const void*)&gemm_nvfp4_bf16_m64, 7, 2u * 64u * 528u, 0u},
+    {"gemm_nvfp4_bf16_m48", (const void*)&gemm_nvfp4_bf16_m48, 7, 2u * 48u * 528u, 0u},
+    {"gemm_nvfp4_bf16_m96", (const void*)&gemm_nvfp4_bf16_m96, 7, 2u * 96u * 528u, 0u},
     CROW_FN(gemm_nvfp4_bf16_m32, 7), CROW_FN(gemm_nvfp4_bf16_m16, 7), CROW_FN(gemv_bf16_w, 5),
 };
 const int g_table_n = (int)(sizeof(g_table) / sizeof(g_table[0]));
@@ -219,6 +221,30 @@ int crow_hip_launch(crow_fn_t f, uint32_t gx, uint32_t gy, uint32_t gz, uint32_t
 // through the workspace).  Aim: about `target` waves in total, so that every CU holds enough
 // 16-byte loads in flight to cover HBM latency, and far more units than CUs so that the
 // hardware dispatcher balances them.  The result depends on (rows, k_dim) only.
+// Which GEMM entry point for m token rows on a [rows, *] tensor.  Up to 16 rows: the K-split body over blocks; up to 96:
+// the K-split body with 32-token blocks.  Beyond that the shared-X body, whose blocks are 4 row tiles x MT tokens: the
+// dispatcher deals ceil(rows / 256) * ceil(m / MT) blocks over the CUs, so the launch lasts as long as the fullest CU.
+// Measured per-block times at K = 5120 (us; they scale with K alike, so only their ratios matter): alone on a CU / sharing it.
+const char* crow_hip_gemm_kernel(uint32_t rows, uint32_t m) {
+    if (m <= 16) return "gemm_nvfp4_bf16_m16";
+    if (m <= 96) return "gemm_nvfp4_bf16_m32";
+    static const struct { const char* name; uint32_t mt; double alone, shared; } cand[] = {
+        {"gemm_nvfp4_bf16_m48", 48, 58.0, 45.0}, {"gemm_nvfp4_bf16_m64", 64, 63.0, 48.5}, {"gemm_nvfp4_bf16_m96", 96, 78.0, 78.0}};
+    const unsigned long long quads = (rows + 4 * CROW_TILE_ROWS - 1) / (4 * CROW_TILE_ROWS);
+    const unsigned long long cus = g.cus > 0 ? (unsigned long long)g.cus : 256ull;
+    const char* best = cand[1].name;
+    double best_t = 0.0;
+    for (const auto& c : cand) {
+        const unsigned long long blocks = quads * ((m + c.mt - 1) / c.mt), per_cu = (blocks + cus - 1) / cus;
+        const double t = per_cu <= 1 ? c.alone : (double)per_cu * c.shared;
+        if (best_t == 0.0 || t < best_t) {
+            best_t = t;
+            best = c.name;
+        }
+    }
+    return best;
+}
+
 int crow_hip_launch_dims(const char* name, uint32_t rows, uint32_t k_dim, uint32_t z, crow_dims* out) {
     if (!out || !name || rows == 0 || z == 0) return CROW_ERR_BAD_ARGUMENT;
     const FnEntry* e = find(name);
@@ -280,7 +306,7 @@ int crow_hip_launch_dims(const char* name, uint32_t rows, uint32_t k_dim, uint32
             *out = crow_dims{rt, 1, s, 256};
             return CROW_OK;
         }
-        const uint32_t mt = strcmp(name, "gemm_nvfp4_bf16_m32") == 0 ? 32 : (strcmp(name, "gemm_nvfp4_bf16_m64") == 0 ? 64 : 128);
+        const uint32_t mt = name[15] == '_' ? (uint32_t)atoi(name + 17) : 128;  // gemm_nvfp4_bf16_m<tokens per block>
         if (mt == 32) {
             *out = crow_dims{rt, (z + 31) / 32, 1, 256};
         } else {

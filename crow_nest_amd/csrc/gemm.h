@@ -312,5 +312,7 @@ extern "C" __global__ void __launch_bounds__(256) gemm_nvfp4_bf16_m16(const unsi
         }                                                                                                                      \
         crow::gemm_pipe_body<TBK>(w, x, gs_ptr, y, *k_dim_p, *rows_p, *m_p, (__bf16*)crow_dyn_lds);                            \
     }
+CROW_GEMM_PIPE_ENTRY(gemm_nvfp4_bf16_m48, 3, 2)
 CROW_GEMM_PIPE_ENTRY(gemm_nvfp4_bf16_m64, 4, 2)
+CROW_GEMM_PIPE_ENTRY(gemm_nvfp4_bf16_m96, 6, 1)
 CROW_GEMM_PIPE_ENTRY(gemm_nvfp4_bf16, 8, 1)

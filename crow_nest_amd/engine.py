@@ -204,23 +204,20 @@ class Engine:
     # ------------------------------------------------------------------ prefill GEMM (M >= 16)
     def gemm(self, w: Fp4, m: int, x: torch.Tensor, y: torch.Tensor | None = None, kernel: str | None = None) -> torch.Tensor:
         """Y[m][rows] = X[m][cols] W^T on the matrix cores (bf16 X, exact bf16 weight tiles, f32 accumulate).
-        `kernel` forces one entry point (gemm_nvfp4_bf16_m16 takes m <= 16, the other three any m); default: gemm_kernel_for(m)."""
+        `kernel` forces one entry point (gemm_nvfp4_bf16_m16 takes m <= 16, the others any m); default: gemm_kernel_for(m, rows)."""
         rows, k = w.rows, w.cols
         assert x.is_cuda and x.is_contiguous() and x.dtype == torch.bfloat16 and x.numel() == m * k
         if y is None:
             y = torch.empty((m, rows), dtype=torch.float32, device=self.dev)
-        name = kernel or gemm_kernel_for(m)
+        name = kernel or gemm_kernel_for(m, rows)
         gx, gy, gz, bx = launch_dims(name, rows, k, m)
         p = self.p
         launch_v(self.k.f(name), gx, gy, gz, bx, [w.w_ptr, x.data_ptr(), w.gs_ptr, y.data_ptr(), p.i32(k), p.i32(rows), p.i32(m)])
         return y
 
 
-def gemm_kernel_for(m: int) -> str:
-    """Which GEMM entry point serves m token rows.  Up to 128 rows the K-split body (one row tile per block, its panels
-    dealt to the block's four waves, 32-token blocks on grid.y) keeps every SIMD busy; up to 16 rows the same body also
-    deals the panels over grid.z blocks (one panel per wave, partial tiles handed over through the workspace); beyond
-    128 the body that shares one staged X tile between four row tiles (64 tokens per wave) decodes the weights fewer times."""
-    if m <= 16:
-        return "gemm_nvfp4_bf16_m16"
-    return "gemm_nvfp4_bf16_m32" if m <= 128 else "gemm_nvfp4_bf16_m64"
+def gemm_kernel_for(m: int, rows: int = 17408) -> str:
+    """Which GEMM entry point serves m token rows of a [rows, *] tensor: the library's choice (crow_hip_gemm_kernel), which
+    weighs how the blocks of each tiling fall on the device's compute units."""
+    from . import lib as _l
+    return _l.lib().crow_hip_gemm_kernel(rows, m).decode()

@@ -78,10 +78,12 @@ CROW_KERNEL(moe_down_combine, 7)
 
 /* ---- batched GEMM on the matrix cores (bf16 x, f32 y) ------------------------------------------------------------- */
 /* w, x, gs, y, k_dim_p, rows_p, m_p.  The dense NVFP4 GEMM of kernels_glm5_moe.cu:310-543 (gemm_fp4_dense's list minus
- * the quantised-activation buffer: x is bf16).  gemm_nvfp4_bf16_m16 serves *m_p <= 16 only; the other three take any m
- * and differ in tiling (32, 64, 128 tokens per block). */
+ * the quantised-activation buffer: x is bf16).  gemm_nvfp4_bf16_m16 serves *m_p <= 16 only; the others take any m
+ * and differ in tiling (32, 48, 64, 96, 128 tokens per block); crow_hip_gemm_kernel names the one to use. */
 CROW_KERNEL(gemm_nvfp4_bf16, 7)
+CROW_KERNEL(gemm_nvfp4_bf16_m96, 7)
 CROW_KERNEL(gemm_nvfp4_bf16_m64, 7)
+CROW_KERNEL(gemm_nvfp4_bf16_m48, 7)
 CROW_KERNEL(gemm_nvfp4_bf16_m32, 7)
 CROW_KERNEL(gemm_nvfp4_bf16_m16, 7)
 

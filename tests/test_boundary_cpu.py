@@ -61,6 +61,16 @@ def test_kernel_header_is_the_library_table():
     assert listed == table
 
 
+def test_gemm_kernel_choice_names_table_entries():
+    lib = L.lib()
+    n = lib.crow_hip_function_count()
+    names = {lib.crow_hip_function_name(i).decode() for i in range(n)}
+    picks = {m: lib.crow_hip_gemm_kernel(17408, m).decode() for m in (1, 16, 17, 96, 97, 128, 256, 512, 1024, 4096)}
+    assert set(picks.values()) <= names
+    assert picks[16] == "gemm_nvfp4_bf16_m16" and picks[17] == picks[96] == "gemm_nvfp4_bf16_m32"
+    assert all(v != "gemm_nvfp4_bf16_m16" for m, v in picks.items() if m > 16)  # that entry point refuses m > 16
+
+
 def test_launch_dims_depend_on_the_matrix_only():
     import ctypes as C
     lib = L.lib()

@@ -383,7 +383,8 @@ def test_config3_full_size_head(eng):
 
 # ---------------------------------------------------------------- batched GEMM on the matrix cores (config 4)
 
-@pytest.mark.parametrize("kernel", ["gemm_nvfp4_bf16_m16", "gemm_nvfp4_bf16_m32", "gemm_nvfp4_bf16_m64", "gemm_nvfp4_bf16"])
+@pytest.mark.parametrize("kernel", ["gemm_nvfp4_bf16_m16", "gemm_nvfp4_bf16_m32", "gemm_nvfp4_bf16_m48", "gemm_nvfp4_bf16_m64", "gemm_nvfp4_bf16_m96",
+                                    "gemm_nvfp4_bf16"])
 @pytest.mark.parametrize("m,rows,cols", [(16, 320, 1024), (5, 100, 320), (16, 17408, 5120), (17, 100, 320), (33, 256, 512), (128, 512, 2048), (200, 192, 5120)])
 def test_gemm_bf16_against_the_cpu_path(eng, m, rows, cols, kernel):
     """Weights decode to exact bf16, X is bf16, products are exact in f32: only the summation order
