@@ -61,14 +61,6 @@ const unsigned COUNTER_WORDS = COUNTER_SLOTS + 1 + 1 + AM_SLOTS / 64;
 
 int hip_rc(hipError_t e) { return e == hipSuccess ? CROW_OK : (int)e; }
 
-long env_long(const char* key, long dflt) {
-    const char* v = getenv(key);
-    if (!v || !*v) return dflt;
-    char* end = nullptr;
-    long r = strtol(v, &end, 10);
-    return end && *end == 0 ? r : dflt;
-}
-
 const FnEntry* find(const char* name) {
     if (!name) return nullptr;
     for (int i = 0; i < g_table_n; i++)
@@ -245,7 +237,7 @@ const char* crow_hip_gemm_kernel(uint32_t rows, uint32_t m) {
     return best;
 }
 
-int crow_hip_launch_dims(const char* name, uint32_t rows, uint32_t k_dim, uint32_t z, crow_dims* out) {
+int crow_hip_launch_dims_split(const char* name, uint32_t rows, uint32_t k_dim, uint32_t z, uint32_t force_s, uint32_t force_w, crow_dims* out) {
     if (!out || !name || rows == 0 || z == 0) return CROW_ERR_BAD_ARGUMENT;
     const FnEntry* e = find(name);
     if (!e) return CROW_ERR_KERNEL_MISSING;
@@ -276,7 +268,6 @@ int crow_hip_launch_dims(const char* name, uint32_t rows, uint32_t k_dim, uint32
         if (units > (long)panels) units = panels;
         long w = units <= 8 ? units : (panels > 32 ? 8 : 4);
         long s = (units + w - 1) / w;
-        const long force_s = env_long("CROW_GEMV_S", 0), force_w = env_long("CROW_GEMV_W", 0);
         if (force_s > 0) s = force_s;
         if (force_w > 0) w = force_w;
         // gate/up kernels for one activation row run one tile per wave: 2 W waves per block (W per tensor), at most 1024 threads
@@ -332,6 +323,10 @@ int crow_hip_launch_dims(const char* name, uint32_t rows, uint32_t k_dim, uint32
         return CROW_OK;
     }
     return CROW_ERR_KERNEL_MISSING;
+}
+
+int crow_hip_launch_dims(const char* name, uint32_t rows, uint32_t k_dim, uint32_t z, crow_dims* out) {
+    return crow_hip_launch_dims_split(name, rows, k_dim, z, 0, 0, out);
 }
 
 int crow_hip_status(void) {

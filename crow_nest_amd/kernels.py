@@ -106,9 +106,10 @@ def status() -> None:
     _l.check(_l.lib().crow_hip_status(), "kernel status")
 
 
-def launch_dims(name: str, rows: int, k_dim: int, z: int = 1) -> tuple[int, int, int, int]:
+def launch_dims(name: str, rows: int, k_dim: int, z: int = 1, split: tuple[int, int] = (0, 0)) -> tuple[int, int, int, int]:
+    """Grid and block the library chooses; `split` = (column slices per row tile, waves per block) forces a GEMV split."""
     d = _l.Dims()
-    rc = _l.lib().crow_hip_launch_dims(name.encode(), rows, k_dim, z, C.byref(d))
+    rc = _l.lib().crow_hip_launch_dims_split(name.encode(), rows, k_dim, z, split[0], split[1], C.byref(d))
     if rc == -2:
         raise KernelMissing(f"kernel missing: {name}")
     _l.check(rc, f"launch_dims({name}, {rows}, {k_dim}, {z})")

@@ -74,6 +74,10 @@ int crow_hip_launch(crow_fn_t f, uint32_t gx, uint32_t gy, uint32_t gz, uint32_t
 /* grid/block for `name` on a [rows, k_dim] tensor with `z` token rows (batched kernels) or combos
  * (routed kernels); 1 otherwise.  The choice depends on (rows, k_dim) only, never on z. */
 int crow_hip_launch_dims(const char* name, uint32_t rows, uint32_t k_dim, uint32_t z, crow_dims* out);
+/* the same with the GEMV split forced: `s` column slices per row tile (blocks that hand their partial sums over through the
+ * workspace) and `w` waves per block and tensor; 0 = the library's choice.  Every GEMV kernel is correct for every split:
+ * this is for tuning and for tests.  Other kernels ignore s and w. */
+int crow_hip_launch_dims_split(const char* name, uint32_t rows, uint32_t k_dim, uint32_t z, uint32_t s, uint32_t w, crow_dims* out);
 /* the GEMM entry point (a name of the kernel table) that serves `m` token rows fastest on a tensor of `rows` rows: the
  * choice depends on how the blocks of each tiling fall on this device's compute units */
 const char* crow_hip_gemm_kernel(uint32_t rows, uint32_t m);

@@ -1,8 +1,6 @@
-"""Shared helpers of the GPU parity tests: input builders, the parity metrics, env overrides."""
+"""Shared helpers of the GPU parity tests: input builders and the parity metrics."""
 from __future__ import annotations
 
-import contextlib
-import os
 
 import numpy as np
 
@@ -45,19 +43,3 @@ def quantized_normal(seed: int, stream: int, rows: int, cols: int, sigma: float 
     return orc.quantize_ceil(v)
 
 
-@contextlib.contextmanager
-def env(**kv):
-    old = {k: os.environ.get(k) for k in kv}
-    try:
-        for k, v in kv.items():
-            if v is None:
-                os.environ.pop(k, None)
-            else:
-                os.environ[k] = str(v)
-        yield
-    finally:
-        for k, v in old.items():
-            if v is None:
-                os.environ.pop(k, None)
-            else:
-                os.environ[k] = v

@@ -9,7 +9,7 @@ import numpy as np
 import pytest
 import torch
 
-from gpu_common import TOL, env, gamma_ratio, quantized_normal, rel_err
+from gpu_common import TOL, gamma_ratio, quantized_normal, rel_err
 from oracle import oracle as orc
 from refgen import SplitMix64, normal_f32, random_nvfp4, scale_mix, synth_nvfp4
 
@@ -118,10 +118,17 @@ def test_gemv_is_correct_for_every_split(eng, s, wv):
     gs = 4.0e-4
     x = normal_f32(1, 5, cols)
     ref = orc.gemv(w, rows, cols, gs, x)[0]
+    from crow_nest_amd.kernels import launch_dims, launch_v
     f = _load(w, rows, cols, gs)
-    with env(CROW_GEMV_S=s, CROW_GEMV_W=wv):
-        y1 = eng.dense_proj(f, 1, _dev(x)).cpu().numpy()[0]
-        y2 = eng.dense_proj(f, 1, _dev(x)).cpu().numpy()[0]
+    xd, p = _dev(x), eng.p
+    dims = launch_dims("gemv_nvfp4_w", rows, cols, 1, split=(s, wv))
+    assert dims[0] == s and dims[3] == 64 * wv
+    ys = []
+    for _ in range(2):
+        y = torch.empty((1, rows), dtype=torch.float32, device="cuda")
+        launch_v(eng.k.f("gemv_nvfp4_w"), *dims, [f.w_ptr, xd.data_ptr(), f.gs_ptr, y.data_ptr(), p.i32(cols), p.i32(rows)])
+        ys.append(y.cpu().numpy()[0])
+    y1, y2 = ys
     eng.check()
     assert np.array_equal(y1.view(np.uint32), y2.view(np.uint32))
     assert rel_err(y1, ref) <= TOL and gamma_ratio(y1, w, rows, cols, gs, x) <= 1.0
