@@ -68,11 +68,20 @@ const FnEntry* find(const char* name) {
     return nullptr;
 }
 
+// a handle is the address of a table entry, nothing else
+const FnEntry* entry_of(crow_fn_t f) {
+    const FnEntry* e = (const FnEntry*)(void*)f;
+    if (e < g_table || e >= g_table + g_table_n) return nullptr;
+    if (((const char*)e - (const char*)g_table) % (ptrdiff_t)sizeof(FnEntry) != 0) return nullptr;
+    return e;
+}
+
 int launch_entry(const FnEntry* e, dim3 grid, dim3 block, const uint64_t* vals, uint32_t n, hipStream_t s) {
     if (!g.ready) return CROW_ERR_NOT_INITIALIZED;
     if (!e || !vals) return CROW_ERR_BAD_ARGUMENT;
     if ((int)n != e->nargs) return CROW_ERR_ARG_COUNT;
-    if (grid.x == 0 || grid.y == 0 || grid.z == 0 || block.x == 0 || block.x > 1024) return CROW_ERR_BAD_ARGUMENT;
+    // whole wavefronts only: every kernel derives its wave count (and its LDS layout) from block.x / 64
+    if (grid.x == 0 || grid.y == 0 || grid.z == 0 || block.x == 0 || block.x > 1024 || block.x % 64 != 0) return CROW_ERR_BAD_ARGUMENT;
     void* args[16];
     for (uint32_t i = 0; i < n; i++) args[i] = (void*)&vals[i];
     const size_t lds = e->lds_fixed + (size_t)e->lds_per_wave * (block.x / 64);
@@ -99,25 +108,36 @@ int crow_hip_init(int device) {
     ws.partial_floats = PARTIAL_FLOATS;
     ws.counter_slots = COUNTER_SLOTS;
     ws.am_slots = AM_SLOTS;
-    if ((e = hipMalloc((void**)&ws.partials, PARTIAL_FLOATS * sizeof(float))) != hipSuccess) return (int)e;
-    if ((e = hipMalloc((void**)&ws.counters, COUNTER_WORDS * sizeof(unsigned))) != hipSuccess) return (int)e;
-    if ((e = hipMalloc((void**)&ws.am_val, AM_SLOTS * sizeof(float))) != hipSuccess) return (int)e;
-    if ((e = hipMalloc((void**)&ws.am_idx, AM_SLOTS * sizeof(int))) != hipSuccess) return (int)e;
-    if ((e = hipMalloc((void**)&g.scalars, 16 * sizeof(int))) != hipSuccess) return (int)e;
-    if ((e = hipMemset(ws.counters, 0, COUNTER_WORDS * sizeof(unsigned))) != hipSuccess) return (int)e;
+    int* scalars = nullptr;
+    // one failure path: everything allocated so far is released again
+    auto fail = [&](hipError_t why) {
+        (void)hipFree(ws.partials);
+        (void)hipFree(ws.counters);
+        (void)hipFree(ws.am_val);
+        (void)hipFree(ws.am_idx);
+        (void)hipFree(scalars);
+        return (int)why;
+    };
+    if ((e = hipMalloc((void**)&ws.partials, PARTIAL_FLOATS * sizeof(float))) != hipSuccess) return fail(e);
+    if ((e = hipMalloc((void**)&ws.counters, COUNTER_WORDS * sizeof(unsigned))) != hipSuccess) return fail(e);
+    if ((e = hipMalloc((void**)&ws.am_val, AM_SLOTS * sizeof(float))) != hipSuccess) return fail(e);
+    if ((e = hipMalloc((void**)&ws.am_idx, AM_SLOTS * sizeof(int))) != hipSuccess) return fail(e);
+    if ((e = hipMalloc((void**)&scalars, 16 * sizeof(int))) != hipSuccess) return fail(e);
+    if ((e = hipMemset(ws.counters, 0, COUNTER_WORDS * sizeof(unsigned))) != hipSuccess) return fail(e);
     ws.status = ws.counters + COUNTER_SLOTS;
     ws.am_counter = ws.counters + COUNTER_SLOTS + 1;
-    if ((e = hipMemcpyToSymbol(HIP_SYMBOL(crow::g_ws), &ws, sizeof ws)) != hipSuccess) return (int)e;
+    if ((e = hipMemcpyToSymbol(HIP_SYMBOL(crow::g_ws), &ws, sizeof ws)) != hipSuccess) return fail(e);
     crow::Geo geo{0, 0, 0, 0};
-    if ((e = hipMemcpyToSymbol(HIP_SYMBOL(crow::g_geo), &geo, sizeof geo)) != hipSuccess) return (int)e;
-    // a GEMV block of 16 waves may need more dynamic LDS than the default per-block limit
+    if ((e = hipMemcpyToSymbol(HIP_SYMBOL(crow::g_geo), &geo, sizeof geo)) != hipSuccess) return fail(e);
+    // a GEMV block of 16 waves, and the GEMM's two staged X tiles, need more dynamic LDS than the default per-block limit
     for (int i = 0; i < g_table_n; i++) {
         const size_t most = g_table[i].lds_fixed + 16 * (size_t)g_table[i].lds_per_wave;
         if (most > 48 * 1024 &&
             (e = hipFuncSetAttribute(g_table[i].stub, hipFuncAttributeMaxDynamicSharedMemorySize, (int)most)) != hipSuccess)
-            return (int)e;
+            return fail(e);
     }
-    if ((e = hipDeviceSynchronize()) != hipSuccess) return (int)e;
+    if ((e = hipDeviceSynchronize()) != hipSuccess) return fail(e);
+    g.scalars = scalars;
     g.ws = ws;
     g.device = device;
     g.stream = nullptr;
@@ -185,9 +205,8 @@ int crow_hip_get_function(const char* name, crow_fn_t* out) {
 int crow_hip_function_count(void) { return g_table_n; }
 const char* crow_hip_function_name(int index) { return index >= 0 && index < g_table_n ? g_table[index].name : nullptr; }
 int crow_hip_function_arg_count(crow_fn_t f) {
-    const FnEntry* e = (const FnEntry*)(void*)f;
-    if (e < g_table || e >= g_table + g_table_n) return CROW_ERR_BAD_ARGUMENT;
-    return e->nargs;
+    const FnEntry* e = entry_of(f);
+    return e ? e->nargs : CROW_ERR_BAD_ARGUMENT;
 }
 
 int crow_hip_set_geo(int experts, int topk, int hidden, int inter) {
@@ -203,16 +222,11 @@ int crow_hip_set_geo(int experts, int topk, int hidden, int inter) {
 
 int crow_hip_launch(crow_fn_t f, uint32_t gx, uint32_t gy, uint32_t gz, uint32_t bx, const uint64_t* vals, uint32_t n_vals,
                     void* stream) {
-    const FnEntry* e = (const FnEntry*)(void*)f;
-    if (e < g_table || e >= g_table + g_table_n) return CROW_ERR_KERNEL_MISSING;
+    const FnEntry* e = entry_of(f);
+    if (!e) return CROW_ERR_KERNEL_MISSING;
     return launch_entry(e, dim3(gx, gy, gz), dim3(bx, 1, 1), vals, n_vals, stream ? (hipStream_t)stream : g.stream);
 }
 
-// Split of a [rows, k_dim] product over the chip.  Every wave owns one 64-row tile; a tile's
-// 256-column panels are dealt to W waves of a block (combined in LDS) and S blocks (combined
-// through the workspace).  Aim: about `target` waves in total, so that every CU holds enough
-// 16-byte loads in flight to cover HBM latency, and far more units than CUs so that the
-// hardware dispatcher balances them.  The result depends on (rows, k_dim) only.
 // Which GEMM entry point for m token rows on a [rows, *] tensor.  Up to 16 rows: the K-split body over blocks; up to 96:
 // the K-split body with 32-token blocks.  Beyond that the shared-X body, whose blocks are 4 row tiles x MT tokens: the
 // dispatcher deals ceil(rows / 256) * ceil(m / MT) blocks over the CUs, so the launch lasts as long as the fullest CU.
@@ -237,6 +251,11 @@ const char* crow_hip_gemm_kernel(uint32_t rows, uint32_t m) {
     return best;
 }
 
+// Split of a [rows, k_dim] product over the chip.  Every wave owns one 64-row tile; a tile's
+// 256-column panels are dealt to W waves of a block (combined in LDS) and S blocks (combined
+// through the workspace): enough waves that every CU holds enough 16-byte loads in flight to
+// cover HBM latency, and far more blocks than CUs so that the hardware dispatcher balances them.
+// The result depends on (rows, k_dim) only.
 int crow_hip_launch_dims_split(const char* name, uint32_t rows, uint32_t k_dim, uint32_t z, uint32_t force_s, uint32_t force_w, crow_dims* out) {
     if (!out || !name || rows == 0 || z == 0) return CROW_ERR_BAD_ARGUMENT;
     const FnEntry* e = find(name);
@@ -253,7 +272,7 @@ int crow_hip_launch_dims_split(const char* name, uint32_t rows, uint32_t k_dim, 
         const bool moe = strcmp(name, "gemv_fp4_ptrb") == 0 || strncmp(name, "moe_", 4) == 0;
         const bool tokens = strcmp(name, "gemv_fp4_b") == 0 || strcmp(name, "gemv_fp4_b1k") == 0 || strcmp(name, "gemv_fp4_bs") == 0;
         const bool two = strstr(name, "_gu") != nullptr || strncmp(name, "moe_gate_up", 11) == 0;
-        uint32_t tiles = two && !strncmp(name, "moe_", 4) ? rt : rt;  // rows = output rows for every kernel
+        const uint32_t tiles = rt;  // rows = output rows for every kernel
         const uint32_t gz = moe ? z : (tokens ? (z + 3) / 4 : 1);
         // A tile's panels are dealt to S blocks of W waves.  Measured on MI355X (17408 x 5120,
         // 5120 x 17408, 151936 x 5120): a wave that owns ONE panel, with every wave of the launch
@@ -401,8 +420,8 @@ int crow_hip_event_destroy(void* ev) { return ev ? hip_rc(hipEventDestroy((hipEv
 int crow_hip_time_launches(crow_fn_t f, uint32_t gx, uint32_t gy, uint32_t gz, uint32_t bx, const uint64_t* vals, uint32_t n_vals,
                            uint32_t n_sets, uint32_t iters, float* us_per_launch) {
     if (!g.ready) return CROW_ERR_NOT_INITIALIZED;
-    const FnEntry* e = (const FnEntry*)(void*)f;
-    if (e < g_table || e >= g_table + g_table_n) return CROW_ERR_KERNEL_MISSING;
+    const FnEntry* e = entry_of(f);
+    if (!e) return CROW_ERR_KERNEL_MISSING;
     if (!vals || !us_per_launch || n_sets == 0 || iters == 0) return CROW_ERR_BAD_ARGUMENT;
     hipEvent_t a, b;
     hipError_t rc;
@@ -428,8 +447,7 @@ int crow_hip_time_sequence(uint32_t n_kernels, const crow_fn_t* fns, const crow_
         return CROW_ERR_BAD_ARGUMENT;
     size_t per_set = 0;
     for (uint32_t k = 0; k < n_kernels; k++) {
-        const FnEntry* e = (const FnEntry*)(void*)fns[k];
-        if (e < g_table || e >= g_table + g_table_n) return CROW_ERR_KERNEL_MISSING;
+        if (!entry_of(fns[k])) return CROW_ERR_KERNEL_MISSING;
         per_set += n_vals[k];
     }
     hipEvent_t a, b;

@@ -361,6 +361,12 @@ __device__ __forceinline__ void gemv_body(const GemvArgs& a, unsigned z, lds_p l
     const int m_rows = a.m < M ? a.m : M;
     const unsigned tile_id = z * (unsigned)row_tiles + (unsigned)rt;
 
+    if constexpr (THIN && NR == 2) {
+        if (waves & 1) {  // the two tensors take half of the block's waves each (uniform over the block: nobody waits at a barrier)
+            if (threadIdx.x == 0) atomicOr(ws.status, STATUS_BAD_SHAPE);
+            return;
+        }
+    }
     lds_p zero = lds;
     lds_p xw = lds + CROW_GEMV_ZERO_BYTES + wave * (XR_ALLOC * CROW_GEMV_XROW_BYTES);
     __attribute__((address_space(3))) float* red =

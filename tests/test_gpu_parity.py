@@ -524,6 +524,27 @@ def test_captured_sequence_replays_match_eager_launches(eng):
     eng.check()
 
 
+def test_launches_with_a_wrong_block_shape_are_refused(eng):
+    """Blocks must be whole wavefronts (refused on the host); the one-row gate/up kernels need an even number of waves
+    (refused by the kernel through the status word, nothing written)."""
+    from crow_nest_amd.kernels import launch_dims, launch_v
+    from crow_nest_amd.lib import CrowHipError
+    rows, cols = 128, 512
+    w = random_nvfp4(3, rows, cols)
+    f = _load(w, rows, cols, 1.0e-3)
+    x = _dev(normal_f32(1, 9, cols))
+    y = torch.full((1, rows), 7.0, dtype=torch.float32, device="cuda")
+    p = eng.p
+    gx, gy, gz, bx = launch_dims("gemv_nvfp4_w", rows, cols)
+    with pytest.raises(CrowHipError):
+        launch_v(eng.k.f("gemv_nvfp4_w"), gx, gy, gz, 100, [f.w_ptr, x.data_ptr(), f.gs_ptr, y.data_ptr(), p.i32(cols), p.i32(rows)])
+    launch_v(eng.k.f("gemv_nvfp4_gu"), 1, 2, 1, 192, [f.w_ptr, f.w_ptr, x.data_ptr(), f.gs_ptr, f.gs_ptr, y.data_ptr(), p.i32(cols), p.i32(rows)])
+    with pytest.raises(CrowHipError):
+        eng.check()
+    assert float(y.min()) == 7.0 == float(y.max())
+    eng.check()
+
+
 def test_verify_kernels_refuse_more_than_four_rows(eng):
     """The reference's verify kernels take at most NVFP4_MMAX = 4 rows (kernels_p2.rs:397-400); a launch with m = 5 writes
     nothing and reports a shape error through the status word instead of computing four rows silently."""
