@@ -118,6 +118,7 @@ __device__ __forceinline__ void gemm_small_body(const unsigned char* __restrict_
     const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
     const int rt = (int)blockIdx.x, m0 = 32 * (int)blockIdx.y;
     const int panels = (k_dim + CROW_PANEL_COLS - 1) / CROW_PANEL_COLS;
+    if (rt * CROW_TILE_ROWS >= rows || m0 >= m_total) return;  // a grid larger than the problem: the whole block leaves
     const int waves = block_threads() >> 6;  // 16 TBK staged rows per wave
     const int slice = (int)blockIdx.z, slices = (int)gridDim.z;  // the panels may also be dealt over blocks (workspace hand-over)
     __bf16* xs = xs_all + wave * (16 * TBK * CROW_GEMM_XS_STRIDE);

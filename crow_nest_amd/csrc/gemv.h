@@ -361,6 +361,7 @@ __device__ __forceinline__ void gemv_body(const GemvArgs& a, unsigned z, lds_p l
     const int m_rows = a.m < M ? a.m : M;
     const unsigned tile_id = z * (unsigned)row_tiles + (unsigned)rt;
 
+    if (rt * CROW_TILE_ROWS >= a.rows) return;  // a grid taller than the tensor: the whole block (and every slice of the tile) leaves
     if constexpr (THIN && NR == 2) {
         if (waves & 1) {  // the two tensors take half of the block's waves each (uniform over the block: nobody waits at a barrier)
             if (threadIdx.x == 0) atomicOr(ws.status, STATUS_BAD_SHAPE);
