@@ -293,6 +293,42 @@ def main() -> int:
             others[f"config2_moe_layer_T{t}"] = entry(us, nbytes)
             others[f"config2_moe_layer_T{t}"]["launches"] = 3
             others[f"config2_moe_layer_T{t}"]["distinct_experts_mean"] = round(distinct, 2)
+        # the same layer for a batch in which experts repeat (64 tokens): per combo against grouped by expert
+        t = 64
+        combos = t * K8
+        max_tiles = min(combos, E) + combos // 4
+        xt = torch.randn(t, H, device=dev) * 0.1
+        yt = torch.zeros(t, H, device=dev)
+        lgs = [torch.randn(t, E, device=dev) for _ in range(12)]
+        distinct = sum(len(torch.unique(torch.topk(l_, K8, dim=1).indices)) for l_ in lgs) / len(lgs)
+        ids = torch.empty((t, K8), dtype=torch.int32, device=dev)
+        wts = torch.empty((t, K8), dtype=torch.float32, device=dev)
+        gup = torch.zeros((t, K8), dtype=torch.int64, device=dev)
+        dnp = torch.zeros((t, K8), dtype=torch.int64, device=dev)
+        h2 = torch.empty((combos, I), dtype=torch.float32, device=dev)
+        eo = torch.empty((combos, H), dtype=torch.float32, device=dev)
+        perm = torch.empty((combos,), dtype=torch.int32, device=dev)
+        tiles = torch.empty((max_tiles, 4), dtype=torch.int32, device=dev)
+        ntl = torch.zeros((1,), dtype=torch.int32, device=dev)
+        lr = Launch(eng, "router_top10", 1, 64, t, [[l_.data_ptr(), 0, ids.data_ptr(), wts.data_ptr(), gup.data_ptr(), dnp.data_ptr(),
+                                                      moes[i_ % 3].table.data_ptr(), 0, 0, 0] for i_, l_ in enumerate(lgs)])
+        lgu = Launch(eng, "moe_gate_up_silu", I, H, combos, [[gup.data_ptr(), xt.data_ptr(), gs1.data_ptr(), h2.data_ptr(), p.i32(H), p.i32(K8), p.i32(H), p.i32(I)]])
+        ldn = Launch(eng, "moe_down_combine", H, I, t, [[dnp.data_ptr(), h2.data_ptr(), gs1.data_ptr(), wts.data_ptr(), yt.data_ptr(), p.i32(I), p.i32(H)]])
+        lgr = Launch(eng, "moe_group", 1, 64, combos, [[ids.data_ptr(), p.i32(combos), perm.data_ptr(), tiles.data_ptr(), ntl.data_ptr(), p.i32(max_tiles)]])
+        lgg = Launch(eng, "moe_gate_up_silu_grouped", I, H, max_tiles,
+                     [[tiles.data_ptr(), ntl.data_ptr(), perm.data_ptr(), moes[i_ % 3].table.data_ptr(), xt.data_ptr(), gs1.data_ptr(), h2.data_ptr(),
+                       p.i32(H), p.i32(K8), p.i32(H), p.i32(I)] for i_ in range(len(lgs))])
+        ldg = Launch(eng, "moe_down_grouped", H, I, max_tiles,
+                     [[tiles.data_ptr(), ntl.data_ptr(), perm.data_ptr(), moes[i_ % 3].table.data_ptr(), h2.data_ptr(), gs1.data_ptr(), eo.data_ptr(),
+                       p.i32(I), p.i32(H)] for i_ in range(len(lgs))])
+        lac = Launch(eng, "acc_combo", H, 1, t, [[eo.data_ptr(), wts.data_ptr(), yt.data_ptr()]])
+        nbytes = int(distinct * (2 * I * H // 64 * 36 + H * I // 64 * 36)) + t * H * 8 + t * E * 4
+        for tag, seq in (("per_combo", [lr, lgu, ldn]), ("grouped", [lr, lgr, lgg, ldg, lac])):
+            sq = [(l_.f, l_.dims, l_.raw) for l_ in seq]
+            time_sequence(sq, len(lgs), 12)
+            us = min(time_sequence(sq, len(lgs), 120) for _ in range(3))
+            others[f"moe_layer_T64_{tag}"] = entry(us, nbytes)
+            others[f"moe_layer_T64_{tag}"]["launches"] = len(seq)
         status()
         out["others"] = others
 

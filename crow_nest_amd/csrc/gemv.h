@@ -72,6 +72,10 @@ struct GemvArgs {
     size_t y_stride;
     int k_dim, rows, m;  // m <= MMAX of the instantiation
     int* argmax_out;     // not null: also write the greedy argmax of y row 0 (fused lm_head head)
+    // grouped launches: not null = row m of this launch is routed combo c = row_map[m]: it reads activation row
+    // c / x_div and writes output row c (strides as above); null = rows 0 .. m - 1 in place
+    const int* row_map;
+    int x_div;
 };
 
 // staging rows per wave: one bf16 row per token, or three (hi, mid, lo) per f32 token, rounded up to whole sets of four
@@ -120,13 +124,15 @@ struct XStage;
 template <int M>
 struct XStage<M, true> {
     uint4 v[(M + 1) / 2];
-    __device__ __forceinline__ void fetch(const void* x, size_t x_stride, int col0, int k_dim, int m_rows, int lane) {
+    __device__ __forceinline__ void fetch(const void* x, const size_t (&xoff)[M], int col0, int k_dim, int m_rows, int lane) {
         const int c = lane & 31, col = col0 + 8 * c;
 #pragma unroll
         for (int t0 = 0; t0 < M; t0 += 2) {
             const int tok = t0 + (lane >> 5);
             v[t0 / 2] = make_uint4(0, 0, 0, 0);
-            if (tok < m_rows && col < k_dim) v[t0 / 2] = *(const uint4*)((const unsigned short*)x + (size_t)tok * x_stride + col);
+            // rows in place: offset = row * stride (xoff[1] is the stride then); gathered rows: one of two uniform offsets
+            const size_t o0 = xoff[t0], o1 = xoff[t0 + 1 < M ? t0 + 1 : t0];
+            if (tok < m_rows && col < k_dim) v[t0 / 2] = *(const uint4*)((const unsigned short*)x + ((lane >> 5) ? o1 : o0) + col);
         }
     }
     __device__ __forceinline__ void store(lds_p xw, int lane) const {
@@ -140,12 +146,12 @@ struct XStage<M, true> {
 template <int M>
 struct XStage<M, false> {
     float4 v[M];
-    __device__ __forceinline__ void fetch(const void* x, size_t x_stride, int col0, int k_dim, int m_rows, int lane) {
+    __device__ __forceinline__ void fetch(const void* x, const size_t (&xoff)[M], int col0, int k_dim, int m_rows, int lane) {
         const int col = col0 + 4 * lane;
 #pragma unroll
         for (int t = 0; t < M; t++) {
             v[t] = make_float4(0.f, 0.f, 0.f, 0.f);
-            if (t < m_rows && col < k_dim) v[t] = *(const float4*)((const float*)x + (size_t)t * x_stride + col);
+            if (t < m_rows && col < k_dim) v[t] = *(const float4*)((const float*)x + xoff[t] + col);
         }
     }
     // x = hi + mid + lo exactly: each term keeps the next 8 significant bits (truncation; the subtractions are exact)
@@ -280,7 +286,7 @@ __device__ __forceinline__ bool slice_hand_over(float (&v)[NV], unsigned tile_id
 // over panels p = p0, p0 + stride, ...  `xw` is the wave's own staging area, `zero` the block's zeroed 512 bytes.
 template <int NR, int M, bool XBF16>
 __device__ __forceinline__ void tile_accumulate(const unsigned char* const (&w)[2], int rt, int panels, int p0, int stride, int k_dim,
-                                                const void* x, size_t x_stride, int m_rows, lds_p xw, lds_p zero, float (&out)[NR][M]) {
+                                                const void* x, const size_t (&xoff)[M], int m_rows, lds_p xw, lds_p zero, float (&out)[NR][M]) {
     constexpr int NSET = XBF16 ? 1 : (3 * M + 3) / 4;
     constexpr int SET_ROWS = XBF16 ? M : 4;  // live operand rows of a set (f32: padding rows are staged as zeros)
     // register-hungry instantiations keep the segments apart: the next segment's operands are not fetched early
@@ -302,7 +308,7 @@ __device__ __forceinline__ void tile_accumulate(const unsigned char* const (&w)[
             for (int m = 0; m < M; m++) acc[r][jp][m] = 0.0f;
     for (int p = p0; p < panels; p += stride) {
         XStage<M, XBF16> xs;
-        xs.fetch(x, x_stride, p * CROW_PANEL_COLS, k_dim, m_rows, lane);
+        xs.fetch(x, xoff, p * CROW_PANEL_COLS, k_dim, m_rows, lane);
         uint4 sc[NR], cd[NR][CROW_STEPS];
         load_tile<NR>(w, rt, panels, p, lane, sc, cd);
         xs.store(xw, lane);
@@ -360,6 +366,19 @@ __device__ __forceinline__ void gemv_body(const GemvArgs& a, unsigned z, lds_p l
     const int panels = (a.k_dim + CROW_PANEL_COLS - 1) / CROW_PANEL_COLS;
     const int m_rows = a.m < M ? a.m : M;
     const unsigned tile_id = z * (unsigned)row_tiles + (unsigned)rt;
+    // element offsets of this launch's activation and output rows
+    size_t xoff[M], yoff[M];
+#pragma unroll
+    for (int m = 0; m < M; m++) {
+        if (a.row_map != nullptr) {
+            const int c = a.row_map[m < m_rows ? m : 0];
+            xoff[m] = (size_t)(c / a.x_div) * a.x_stride;
+            yoff[m] = (size_t)c * a.y_stride;
+        } else {
+            xoff[m] = (size_t)m * a.x_stride;
+            yoff[m] = (size_t)m * a.y_stride;
+        }
+    }
 
     if (rt * CROW_TILE_ROWS >= a.rows) return;  // a grid taller than the tensor: the whole block (and every slice of the tile) leaves
     if constexpr (THIN && NR == 2) {
@@ -386,7 +405,7 @@ __device__ __forceinline__ void gemv_body(const GemvArgs& a, unsigned z, lds_p l
         const int pw = wave - r_own * wpt;
         float part[1][M];
         const unsigned char* const w_own[2] = {r_own != 0 ? a.w[1] : a.w[0], nullptr};  // a select, never an indexed read
-        tile_accumulate<1, M, XBF16>(w_own, rt, panels, slice * wpt + pw, slices * wpt, a.k_dim, a.x, a.x_stride, m_rows, xw, zero, part);
+        tile_accumulate<1, M, XBF16>(w_own, rt, panels, slice * wpt + pw, slices * wpt, a.k_dim, a.x, xoff, m_rows, xw, zero, part);
         // waves of the block -> wave 0, per tensor in wave order
 #pragma unroll
         for (int m = 0; m < M; m++) acc[0][m] = part[0][m];
@@ -410,7 +429,7 @@ __device__ __forceinline__ void gemv_body(const GemvArgs& a, unsigned z, lds_p l
                 if (m < m_rows) acc[1][m] += red[((w - 1) * M + m) * 64 + lane];
         }
     } else {
-        tile_accumulate<NR, M, XBF16>(a.w, rt, panels, slice * waves + wave, slices * waves, a.k_dim, a.x, a.x_stride, m_rows, xw, zero, acc);
+        tile_accumulate<NR, M, XBF16>(a.w, rt, panels, slice * waves + wave, slices * waves, a.k_dim, a.x, xoff, m_rows, xw, zero, acc);
         // waves of the block -> wave 0, in wave order
         if (waves > 1) {
             if (wave > 0) {
@@ -504,12 +523,12 @@ __device__ __forceinline__ void gemv_body(const GemvArgs& a, unsigned z, lds_p l
         const float gs = a.gs[0][0];
 #pragma unroll
         for (int m = 0; m < M; m++)
-            if (m < m_rows) a.y[(size_t)m * a.y_stride + row] = acc[0][m] * gs;
+            if (m < m_rows) a.y[yoff[m] + row] = acc[0][m] * gs;
     } else {
         const float gg = a.gs[0][0], gu = a.gs[NR - 1][0];
 #pragma unroll
         for (int m = 0; m < M; m++)
-            if (m < m_rows) a.y[(size_t)m * a.y_stride + row] = silu_mul(acc[0][m] * gg, acc[NR - 1][m] * gu);
+            if (m < m_rows) a.y[yoff[m] + row] = silu_mul(acc[0][m] * gg, acc[NR - 1][m] * gu);
     }
 }
 

@@ -223,7 +223,8 @@ extern "C" __global__ void __launch_bounds__(1024) moe_down_combine(const unsign
     __syncthreads();
     const unsigned char* const w[2] = {(const unsigned char*)ptrs[combo], nullptr};
     float acc[1][1];
-    tile_accumulate<1, 1, false>(w, rt, (k + CROW_PANEL_COLS - 1) / CROW_PANEL_COLS, 0, 1, k, h + (size_t)combo * k, 0, 1, xw, zero, acc);
+    const size_t xoff[1] = {0};
+    tile_accumulate<1, 1, false>(w, rt, (k + CROW_PANEL_COLS - 1) / CROW_PANEL_COLS, 0, 1, k, h + (size_t)combo * k, xoff, 1, xw, zero, acc);
     red[j * 64 + lane] = rw[combo] * (acc[0][0] * gs_ptr[0]);
     __syncthreads();
     const int row = rt * CROW_TILE_ROWS + lane;
@@ -231,4 +232,43 @@ extern "C" __global__ void __launch_bounds__(1024) moe_down_combine(const unsign
     float sum = 0.0f;
     for (int q = 0; q < topk; q++) sum = __fadd_rn(sum, red[q * 64 + lane]);
     y[(size_t)t * rows + row] += sum;
+}
+
+// ------------------------------------------------------------------ routed experts, grouped by expert (batches of many tokens)
+// The per-combo kernels above read a routed expert's slab once per token that picked it.  For batches in which experts
+// repeat, moe_group (misc_kernels.h) sorts the combos by expert and cuts them into tiles of at most four combos of one
+// expert (the idea of moe_count / moe_plan / moe_scatter, engine/src/kernels.rs:3322-3384, in one launch); the two kernels
+// below multiply a tile's slab once by its (up to) four rows, gathered through `perm`.  grid (S, row tiles, max tiles):
+// blocks of tiles >= *n_tiles_p leave at once.  tiles[z] = (expert, first position in perm, combos, 0); table[2 e] /
+// table[2 e + 1] = gate|up / down slab of expert e (the router's table).  Row m of a tile is combo c = perm[first + m]:
+// it reads activation row c / *x_div_p and writes output row c.
+extern "C" __global__ void __launch_bounds__(512) moe_gate_up_silu_grouped(const int4* __restrict__ tiles, const int* __restrict__ n_tiles_p,
+                                                                            const int* __restrict__ perm, const unsigned long long* __restrict__ table,
+                                                                            const float* __restrict__ x, const float* __restrict__ gs_ptr,
+                                                                            float* __restrict__ h, const int* __restrict__ k_dim_p,
+                                                                            const int* __restrict__ x_div_p, const int* __restrict__ x_stride_p,
+                                                                            const int* __restrict__ inter_p) {
+    ENTER(tiles, n_tiles_p, perm, table, x, gs_ptr, h, k_dim_p, x_div_p, x_stride_p, inter_p);
+    const int z = (int)blockIdx.z;
+    if (z >= *n_tiles_p) return;
+    const int4 tl = tiles[z];
+    const int inter = *inter_p, k = *k_dim_p;
+    const unsigned char* w = (const unsigned char*)table[2 * tl.x];
+    const size_t up_off = (size_t)(inter / CROW_TILE_ROWS) * ((k + CROW_PANEL_COLS - 1) / CROW_PANEL_COLS) * CROW_TILE_BYTES;
+    GemvArgs a{{w, w + up_off}, {gs_ptr, gs_ptr}, x, (size_t)*x_stride_p, h, (size_t)inter, k, inter, tl.z, nullptr, perm + tl.y, *x_div_p};
+    gemv_m_dispatch<2, false, EPI_SILU_GU>(a, blockIdx.z, LDS, ws);
+}
+// down slabs: x = h [combos][k_dim], y = eo [combos][rows]; acc_combo then adds the weighted rows per token
+extern "C" __global__ void __launch_bounds__(1024) moe_down_grouped(const int4* __restrict__ tiles, const int* __restrict__ n_tiles_p,
+                                                                    const int* __restrict__ perm, const unsigned long long* __restrict__ table,
+                                                                    const float* __restrict__ h, const float* __restrict__ gs_ptr,
+                                                                    float* __restrict__ eo, const int* __restrict__ k_dim_p,
+                                                                    const int* __restrict__ rows_p) {
+    ENTER(tiles, n_tiles_p, perm, table, h, gs_ptr, eo, k_dim_p, rows_p);
+    const int z = (int)blockIdx.z;
+    if (z >= *n_tiles_p) return;
+    const int4 tl = tiles[z];
+    const int k = *k_dim_p, rows = *rows_p;
+    GemvArgs a{{(const unsigned char*)table[2 * tl.x + 1], nullptr}, {gs_ptr, nullptr}, h, (size_t)k, eo, (size_t)rows, k, rows, tl.z, nullptr, perm + tl.y, 1};
+    gemv_m_dispatch<1, false, EPI_SCALE>(a, blockIdx.z, LDS, ws);
 }

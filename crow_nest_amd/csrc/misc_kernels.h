@@ -242,6 +242,101 @@ extern "C" __global__ void __launch_bounds__(64) router_top10(const float* __res
     }
 }
 
+// Sort the n routed combos of a batch by expert and cut them into tiles of at most four combos of one expert: the work of
+// moe_count + moe_plan + moe_scatter (engine/src/kernels.rs:3334-3384) in ONE launch of one block (the reference needs
+// three because its plan also schedules host-to-device staging of cold experts, which does not exist here; its tiles hold
+// up to 8 combos, the width of its MMA; four is the row count of this library's GEMV).  ids[n] = expert of combo c;
+// perm[n] = the combos in expert order, ascending combo inside an expert (stable, so the result does not depend on timing);
+// tiles[t] = (expert, first position in perm, combos, 0), experts ascending; *n_tiles.
+// A counting sort over chunks of 64 combos (one wavefront pass each): per-chunk histograms, a running sum per expert
+// over the chunks, a block scan over the experts, then every chunk ranks its combos among equal experts with ballots.
+// n <= 4096, E = g_geo.experts <= 1024, E * ceil(n / 64) <= 16384.  grid 1, block 1024.
+#define CROW_MOE_GROUP_MAX_COMBOS 4096
+#define CROW_MOE_GROUP_HIST 16384
+extern "C" __global__ void __launch_bounds__(1024) moe_group(const int* __restrict__ ids, const int* __restrict__ n_p, int* __restrict__ perm,
+                                                             int4* __restrict__ tiles, int* __restrict__ n_tiles, const int* __restrict__ max_tiles_p) {
+    __shared__ unsigned short s_hist[CROW_MOE_GROUP_HIST];  // [chunk][expert]: count, then the count in earlier chunks
+    __shared__ int s_off[1024], s_tile[1024];
+    __shared__ int s_bad;
+    const int n = *n_p, E = g_geo.experts, max_tiles = *max_tiles_p, t = (int)threadIdx.x;
+    const int chunks = (n + 63) >> 6;
+    if (block_threads() != 1024 || n < 0 || n > CROW_MOE_GROUP_MAX_COMBOS || E < 1 || E > 1024 || E * chunks > CROW_MOE_GROUP_HIST) {
+        if (t == 0) {
+            atomicOr(g_ws.status, STATUS_BAD_GEO);
+            *n_tiles = 0;
+        }
+        return;
+    }
+    for (int i = t; i < E * chunks; i += 1024) s_hist[i] = 0;
+    if (t == 0) s_bad = 0;
+    __syncthreads();
+    // per-chunk histograms (16-bit counters, two to a word: add 1 or 1 << 16)
+    for (int i = t; i < n; i += 1024) {
+        const int e = ids[i];
+        if (e < 0 || e >= E) s_bad = 1;
+        else {
+            const int slot = (i >> 6) * E + e;
+            atomicAdd((unsigned*)s_hist + (slot >> 1), (slot & 1) ? 0x10000u : 1u);
+        }
+    }
+    __syncthreads();
+    if (s_bad) {  // an expert id outside the geometry: nothing is planned
+        if (t == 0) {
+            atomicOr(g_ws.status, STATUS_BAD_GEO);
+            *n_tiles = 0;
+        }
+        return;
+    }
+    // thread = expert: counts of earlier chunks, and the expert's total
+    int cnt = 0;
+    if (t < E) {
+        for (int c = 0; c < chunks; c++) {
+            const int v = s_hist[c * E + t];
+            s_hist[c * E + t] = (unsigned short)cnt;
+            cnt += v;
+        }
+    }
+    const int tc = (cnt + 3) >> 2;
+    s_off[t] = cnt;
+    s_tile[t] = tc;
+    __syncthreads();
+    for (int d = 1; d < 1024; d <<= 1) {  // inclusive scans over the experts: combos, and tiles of four
+        const int a = t >= d ? s_off[t - d] : 0, b = t >= d ? s_tile[t - d] : 0;
+        __syncthreads();
+        s_off[t] += a;
+        s_tile[t] += b;
+        __syncthreads();
+    }
+    const int first = s_off[t] - cnt, first_tile = s_tile[t] - tc, total_tiles = s_tile[1023];
+    if (total_tiles > max_tiles) {  // uniform: every thread reads the same total
+        if (t == 0) {
+            atomicOr(g_ws.status, STATUS_WORKSPACE_TOO_SMALL);
+            *n_tiles = 0;
+        }
+        return;
+    }
+    if (t == 0) *n_tiles = total_tiles;
+    for (int q = 0; q < tc; q++) tiles[first_tile + q] = make_int4(t, first + 4 * q, cnt - 4 * q < 4 ? cnt - 4 * q : 4, 0);
+    s_off[t] = first;  // now: the expert's first position in perm
+    __syncthreads();
+    // every chunk (one wavefront pass) ranks its combos among equal experts: position = expert's first + earlier chunks + rank
+    const int lane = lane_id(), wave = t >> 6;
+    for (int c = wave; c < chunks; c += 16) {
+        const int i = c * 64 + lane;
+        const bool live = i < n;
+        const int e = live ? ids[i] : -1;
+        int rank = 0;
+        unsigned long long todo = __ballot(live);
+        while (todo) {  // one round per distinct expert of the chunk
+            const int lead = __builtin_amdgcn_readlane(e, (int)__builtin_ctzll(todo));
+            const unsigned long long same = __ballot(e == lead);
+            if (e == lead) rank = __popcll(same & ((1ull << lane) - 1ull));
+            todo &= ~same;
+        }
+        if (live) perm[s_off[e] + s_hist[c * E + e] + rank] = i;
+    }
+}
+
 // reference: silu_mul_combo, engine/src/kernels.rs:1562-1570: [C][2 I] -> [C][I], I = g_geo.inter
 extern "C" __global__ void silu_mul_combo(const float* __restrict__ h1, float* __restrict__ h2, const int* __restrict__ n_p) {
     const int i = (int)(blockIdx.x * blockDim.x + threadIdx.x);

@@ -76,6 +76,18 @@ CROW_KERNEL(moe_gate_up_silu, 8)
  * token's combos j, in j order, of rw[t][j] * (down_j h_j). */
 CROW_KERNEL(moe_down_combine, 7)
 
+/* routed experts grouped by expert, for batches in which experts repeat (the idea of moe_count / moe_plan / moe_scatter,
+ * kernels.rs:3322-3384, without the staging of cold experts):
+ * moe_group: ids, n_p, perm, tiles, n_tiles, max_tiles_p.  One block sorts the n <= 4096 combos by expert (stable) and cuts
+ *   them into tiles (expert, first position in perm, combos <= 4, 0); sets the bad-geometry bit for an id outside
+ *   0 .. experts - 1 and the workspace bit when more than *max_tiles_p tiles would be needed (then *n_tiles = 0).
+ * moe_gate_up_silu_grouped: tiles, n_tiles_p, perm, table, x, gs, h, k_dim_p, x_div_p, x_stride_p, inter_p.
+ * moe_down_grouped: tiles, n_tiles_p, perm, table, h, gs, eo, k_dim_p, rows_p (acc_combo then combines eo per token).
+ *   grid.z = an upper bound of the tile count (crow_hip_launch_dims with z = that bound); blocks beyond *n_tiles_p leave. */
+CROW_KERNEL(moe_group, 6)
+CROW_KERNEL(moe_gate_up_silu_grouped, 11)
+CROW_KERNEL(moe_down_grouped, 9)
+
 /* ---- batched GEMM on the matrix cores (bf16 x, f32 y) ------------------------------------------------------------- */
 /* w, x, gs, y, k_dim_p, rows_p, m_p.  The dense NVFP4 GEMM of kernels_glm5_moe.cu:310-543 (gemm_fp4_dense's list minus
  * the quantised-activation buffer: x is bf16).  gemm_nvfp4_bf16_m16 serves *m_p <= 16 only; the others take any m

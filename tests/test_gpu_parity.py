@@ -310,6 +310,46 @@ def test_moe_layer_both_launch_sequences(eng, t):
     eng.check()
 
 
+@pytest.mark.parametrize("t", [3, 24, 64])
+def test_moe_layer_grouped_by_expert(eng, t):
+    """Batches in which experts repeat: the plan is a stable sort of the combos by expert cut into tiles of at most four,
+    and the layer's output matches the CPU path (which walks token by token)."""
+    from crow_nest_amd.engine import MoeW, expert_table
+    from crow_nest_amd.weights import load_expert_slabs
+    E, H, I, K = 256, 2048, 512, 8
+    print(f"case grouped moe t={t}", flush=True)
+    gu = random_nvfp4(41, E * 2 * I, H, scale_lo=0x30, scale_hi=0x48, p7f=0)
+    dn = random_nvfp4(42, E * H, I, scale_lo=0x30, scale_hi=0x48, p7f=0)
+    gs_gu, gs_dn = 2.0e-3, 3.0e-3
+    s_gu, s_dn = load_expert_slabs(gu, E, 2 * I, H, gs_gu), load_expert_slabs(dn, E, H, I, gs_dn)
+    moe = MoeW(s_gu, s_dn, expert_table(s_gu, s_dn))
+    x = (normal_f32(5, 100 + t, t * H) * np.float32(0.1)).reshape(t, H)
+    logits = normal_f32(6, 100 + t, t * E).reshape(t, E)
+    logits[:, :16] += np.float32(2.5)  # a few popular experts: long groups
+    ids_ref, w_ref, y_ref = orc.moe_layer(gu, gs_gu, dn, gs_dn, E, H, I, x, logits, K, threads=8)
+    ids, wts, y, (perm, tiles, n_tiles) = eng.moe_run_grouped(moe, _dev(x), _dev(logits))
+    eng.check()
+    assert np.array_equal(ids.cpu().numpy(), ids_ref)
+    # the plan: perm = stable argsort of the expert ids; tiles cover every group in runs of at most four
+    flat = ids_ref.reshape(-1)
+    assert np.array_equal(perm.cpu().numpy(), np.argsort(flat, kind="stable").astype(np.int32))
+    nt = int(n_tiles.item())
+    tl = tiles.cpu().numpy()[:nt]
+    want = []
+    start = 0
+    for e in range(E):
+        c = int((flat == e).sum())
+        for q in range(0, c, 4):
+            want.append((e, start + q, min(4, c - q), 0))
+        start += c
+    assert tl.tolist() == [list(w_) for w_ in want]
+    assert rel_err(y.cpu().numpy(), y_ref) <= TOL
+    # the ungrouped sequence gives the same layer
+    _, _, y2 = eng.moe_run(moe, _dev(x), _dev(logits), fused=True)
+    assert rel_err(y2.cpu().numpy(), y_ref) <= TOL
+    eng.check()
+
+
 # ---------------------------------------------------------------- BASELINE config 0 at full size
 
 def test_config0_full_size(eng):
