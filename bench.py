@@ -344,7 +344,7 @@ def main() -> int:
         for u in units:  # warm-up pass
             orc.ffn(u[0], gsv[0], u[1], gsv[1], u[2], gsv[2], K, N, xs, threads=threads, path=1)
         ts = []
-        for rep in range(24):
+        for rep in range(160):
             u = units[rep % 8]
             c0 = time.perf_counter()
             orc.ffn(u[0], gsv[0], u[1], gsv[1], u[2], gsv[2], K, N, xs, threads=threads, path=1)
@@ -352,11 +352,11 @@ def main() -> int:
         ts.sort()
         med = ts[len(ts) // 2]
         by_threads = {}
-        for th in (1, 4, 8):  # the reference reports 1 / 4 / 8 / all threads (cpu_nvfp4.rs:729-777); 8 calls each here
+        for th in (1, 4, 8):  # the reference reports 1 / 4 / 8 / all threads (cpu_nvfp4.rs:729-777); 64 calls each here
             if th >= threads:
                 continue
             tt = []
-            for rep in range(8):
+            for rep in range(64):
                 u = units[rep % 8]
                 c0 = time.perf_counter()
                 orc.ffn(u[0], gsv[0], u[1], gsv[1], u[2], gsv[2], K, N, xs, threads=th, path=1)
@@ -366,8 +366,8 @@ def main() -> int:
         by_threads[str(threads)] = round(3 * W_BYTES / med / 1e9, 2)
         out["cpu_baseline"] = {"value": round(3 * W_BYTES / med / 1e9, 2), "unit": "GB/s", "cores": threads, "kind": "port",
                                "ms_per_step": round(med * 1e3, 3), "GB/s_by_threads": by_threads,
-                               "sample": "same step (gate/up + SiLU + down, one token, f32 x) on 8 rotating 150 MB weight units, median of 24 calls "
-                                         "after a warm-up pass; AVX2 path of the C restatement of engine/src/cpu_nvfp4.rs (OpenMP row split)"}
+                               "sample": "same step (gate/up + SiLU + down, one token, f32 x) on 8 rotating 150 MB weight units, median of 160 calls "
+                                         "after a warm-up pass (64 calls for each smaller thread count: about 15 core-seconds in all); AVX2 path of the C restatement of engine/src/cpu_nvfp4.rs (OpenMP row split)"}
     print(json.dumps(out))
     return 0
 
