@@ -228,14 +228,26 @@ __device__ __forceinline__ void gemm_pipe_body(const unsigned char* __restrict__
 #pragma unroll
         for (int s = 0; s < CROW_STEPS; s++) cd[s] = stream_load(t + 64 * (s + 1));
     };
-    // chunk c = i * 256 + thread: token row c / 32, 8 columns from 8 (c % 32)
-    auto load_x = [&](int p, uint4 (&xv)[XCH]) {
+    // chunk c = i * 256 + thread: token row c / 32, 8 columns from 8 (c % 32).  The element offset of the chunk in panel 0 is
+    // worked out once; rows beyond M read row M - 1 (their results are never stored), so whole panels load without masks.
+    const int xq = ((int)threadIdx.x & 31) * 8;
+    unsigned xoff[XCH];
 #pragma unroll
-        for (int i = 0; i < XCH; i++) {
-            const int c = i * 256 + (int)threadIdx.x, r = c >> 5, q = c & 31;
-            const int m = m0 + r, k = p * CROW_PANEL_COLS + q * 8;
-            xv[i] = make_uint4(0, 0, 0, 0);
-            if (m < m_total && k < k_dim) xv[i] = *(const uint4*)(x + (size_t)m * k_dim + k);
+    for (int i = 0; i < XCH; i++) {
+        const int m = m0 + ((i * 256 + (int)threadIdx.x) >> 5);
+        xoff[i] = (unsigned)(m < m_total ? m : m_total - 1) * (unsigned)k_dim + (unsigned)xq;
+    }
+    auto load_x = [&](int p, uint4 (&xv)[XCH]) {
+        const int k0 = p * CROW_PANEL_COLS;
+        if (k0 + CROW_PANEL_COLS <= k_dim) {  // uniform
+#pragma unroll
+            for (int i = 0; i < XCH; i++) xv[i] = *(const uint4*)(x + (size_t)(xoff[i] + (unsigned)k0));
+        } else {  // the last, partial panel: columns beyond K are zeros (they meet zero weights, but must not be NaN)
+#pragma unroll
+            for (int i = 0; i < XCH; i++) {
+                xv[i] = make_uint4(0, 0, 0, 0);
+                if (k0 + xq < k_dim) xv[i] = *(const uint4*)(x + (size_t)(xoff[i] + (unsigned)k0));
+            }
         }
     };
     auto store_x = [&](__bf16* xs, const uint4 (&xv)[XCH]) {
@@ -307,7 +319,8 @@ extern "C" __global__ void __launch_bounds__(256) gemm_nvfp4_bf16_m16(const unsi
                                                            const float* __restrict__ gs_ptr, float* __restrict__ y,            \
                                                            const int* __restrict__ k_dim_p, const int* __restrict__ rows_p,    \
                                                            const int* __restrict__ m_p) {                                      \
-        if (block_threads() != 256 || *m_p < 1) {                                                                              \
+        /* 256 threads; X is addressed with 32-bit element offsets */                                                         \
+        if (block_threads() != 256 || *m_p < 1 || (unsigned long long)*m_p * (unsigned long long)*k_dim_p > 0xffffffffull) {   \
             if (threadIdx.x == 0) atomicOr(crow::g_ws.status, crow::STATUS_BAD_SHAPE);                                         \
             return;                                                                                                            \
         }                                                                                                                      \
