@@ -131,16 +131,29 @@ __device__ __forceinline__ void gemm_small_body(const unsigned char* __restrict_
         for (int j = 0; j < 4; j++) acc[tb][j] = f32x4{0.f, 0.f, 0.f, 0.f};
 
     const uint4* wt = (const uint4*)(w + (size_t)rt * panels * CROW_TILE_BYTES) + lane;
-    for (int p = slice * waves + wave; p < panels; p += slices * waves) {
-        // 16 TBK tokens x 256 columns = 512 TBK chunks of 16 bytes, 8 TBK per lane; wave-private.  Fetched before the weight
-        // loads are issued so that they do not queue behind them.
-        uint4 xv[8 * TBK];
+    // 16 TBK tokens x 256 columns = 512 TBK chunks of 16 bytes, 8 TBK per lane; wave-private.  Chunk i of this lane: token row
+    // 2 i + lane / 32, 8 columns from 8 (lane % 32); its element offset in panel 0 is worked out once (32 bits: checked by
+    // the entry points); rows beyond M read row M - 1, whose results are never stored.
+    const int xq = (lane & 31) * 8;
+    unsigned xoff[8 * TBK];
 #pragma unroll
-        for (int i = 0; i < 8 * TBK; i++) {
-            const int c = i * 64 + lane, r = c >> 5, q = c & 31;
-            const int k = p * CROW_PANEL_COLS + q * 8;
-            xv[i] = make_uint4(0, 0, 0, 0);
-            if (m0 + r < m_total && k < k_dim) xv[i] = *(const uint4*)(x + (size_t)(m0 + r) * k_dim + k);
+    for (int i = 0; i < 8 * TBK; i++) {
+        const int m = m0 + 2 * i + (lane >> 5);
+        xoff[i] = (unsigned)(m < m_total ? m : m_total - 1) * (unsigned)k_dim + (unsigned)xq;
+    }
+    for (int p = slice * waves + wave; p < panels; p += slices * waves) {
+        // fetched before the weight loads are issued so that they do not queue behind them
+        uint4 xv[8 * TBK];
+        const int k0 = p * CROW_PANEL_COLS;
+        if (k0 + CROW_PANEL_COLS <= k_dim) {  // uniform
+#pragma unroll
+            for (int i = 0; i < 8 * TBK; i++) xv[i] = *(const uint4*)(x + (size_t)(xoff[i] + (unsigned)k0));
+        } else {  // the last, partial panel: columns beyond K are zeros
+#pragma unroll
+            for (int i = 0; i < 8 * TBK; i++) {
+                xv[i] = make_uint4(0, 0, 0, 0);
+                if (k0 + xq < k_dim) xv[i] = *(const uint4*)(x + (size_t)(xoff[i] + (unsigned)k0));
+            }
         }
         uint4 sc, cd[CROW_STEPS];
         const uint4* t = wt + (size_t)p * (CROW_TILE_BYTES / 16);
@@ -297,6 +310,10 @@ extern "C" __global__ void __launch_bounds__(512) gemm_nvfp4_bf16_m32(const unsi
                                                                          const int* __restrict__ m_p) {
     __shared__ __attribute__((aligned(16))) __bf16 xs[4 * 32 * CROW_GEMM_XS_STRIDE];
     const int m = *m_p;
+    if (m < 1 || (unsigned long long)m * (unsigned long long)*k_dim_p > 0xffffffffull) {  // X is addressed with 32-bit element offsets
+        if (threadIdx.x == 0) atomicOr(crow::g_ws.status, crow::STATUS_BAD_SHAPE);
+        return;
+    }
     if (m <= 16) crow::gemm_small_body<1>(w, x, gs_ptr, y, *k_dim_p, *rows_p, m, xs);  // one 16-token block: half the matrix work and staging
     else crow::gemm_small_body<2>(w, x, gs_ptr, y, *k_dim_p, *rows_p, m, xs);
 }
@@ -307,7 +324,7 @@ extern "C" __global__ void __launch_bounds__(256) gemm_nvfp4_bf16_m16(const unsi
                                                                        const int* __restrict__ m_p) {
     __shared__ __attribute__((aligned(16))) __bf16 xs[4 * 16 * CROW_GEMM_XS_STRIDE];
     const int m = *m_p;
-    if (m > 16 || block_threads() > 256) {  // uniform over the launch
+    if (m < 1 || m > 16 || block_threads() > 256 || (unsigned long long)m * (unsigned long long)*k_dim_p > 0xffffffffull) {  // uniform over the launch
         if (threadIdx.x == 0) atomicOr(crow::g_ws.status, crow::STATUS_BAD_SHAPE);
         return;
     }
