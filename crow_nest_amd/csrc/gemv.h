@@ -54,8 +54,9 @@
 //
 // Dynamic LDS of a block (bytes; the launcher sizes it from the block size):
 //   [0, 512)                                   zeros
-//   [512 + (wave * XR + r) * 576, + 512)       activation staging, XR rows per wave (row stride 576)
-//   then (waves - 1) * NR * M * 64 floats      wave hand-over (one-tile-per-wave two-tensor kernels: waves = 2 W, NR -> 1)
+//   [512 + (wave * XR + r) * 560, + 512)       activation staging, XR rows per wave (row stride 560); when a wave has
+//                                              finished its panels, the first NR * M * 256 bytes of its area carry its
+//                                              partial sums to wave 0 (no separate hand-over area)
 #pragma once
 #include "device_common.h"
 
@@ -85,9 +86,10 @@ struct XRows {
     static constexpr int value = XBF16 ? M : 4 * ((3 * M + 3) / 4);
 };
 #define CROW_GEMV_ZERO_BYTES 512
-// 512 bytes of data per staged row; the 64 bytes of padding put four consecutive rows on four different groups of
-// 16 LDS banks, so that the operand reads of a set's rows do not collide
-#define CROW_GEMV_XROW_BYTES 576
+// 512 bytes of data per staged row; the 48 bytes of padding start four consecutive rows 48 bytes apart modulo the 256-byte
+// bank cycle, so that the operand reads of a set's rows mostly miss each other (64 bytes would separate them fully:
+// measured equal), and twelve rows for each of twelve waves still fit twice into a compute unit's 160 KB
+#define CROW_GEMV_XROW_BYTES 560
 
 typedef __attribute__((address_space(3))) unsigned char* lds_p;
 __device__ __forceinline__ void lds_store16(lds_p p, unsigned a, unsigned b, unsigned c, unsigned d) {
@@ -389,8 +391,10 @@ __device__ __forceinline__ void gemv_body(const GemvArgs& a, unsigned z, lds_p l
     }
     lds_p zero = lds;
     lds_p xw = lds + CROW_GEMV_ZERO_BYTES + wave * (XR_ALLOC * CROW_GEMV_XROW_BYTES);
-    __attribute__((address_space(3))) float* red =
-        (__attribute__((address_space(3))) float*)(lds + CROW_GEMV_ZERO_BYTES + waves * (XR_ALLOC * CROW_GEMV_XROW_BYTES));
+    // a wave's partial sums for wave 0 go where its staged activations were (dead by then): area w, NR * M rows of 256 bytes
+    typedef __attribute__((address_space(3))) float* lds_f;
+    static_assert(NR * M * 256 <= XR_ALLOC * CROW_GEMV_XROW_BYTES, "hand-over rows fit the staging area");
+    auto red_of = [&](int w) -> lds_f { return (lds_f)(lds + CROW_GEMV_ZERO_BYTES + w * (XR_ALLOC * CROW_GEMV_XROW_BYTES)); };
     if (threadIdx.x < CROW_GEMV_ZERO_BYTES / 16) lds_store16(zero + 16 * threadIdx.x, 0, 0, 0, 0);
     if (waves > 1) __syncthreads();
     else __builtin_amdgcn_wave_barrier();
@@ -410,34 +414,36 @@ __device__ __forceinline__ void gemv_body(const GemvArgs& a, unsigned z, lds_p l
 #pragma unroll
         for (int m = 0; m < M; m++) acc[0][m] = part[0][m];
         if (wave > 0) {
+            lds_f mine = red_of(wave);
 #pragma unroll
             for (int m = 0; m < M; m++)
-                if (m < m_rows) red[((wave - 1) * M + m) * 64 + lane] = part[0][m];
+                if (m < m_rows) mine[m * 64 + lane] = part[0][m];
         }
         __syncthreads();
         if (wave > 0) return;
         for (int w = 1; w < wpt; w++) {
 #pragma unroll
             for (int m = 0; m < M; m++)
-                if (m < m_rows) acc[0][m] += red[((w - 1) * M + m) * 64 + lane];
+                if (m < m_rows) acc[0][m] += red_of(w)[m * 64 + lane];
         }
 #pragma unroll
-        for (int m = 0; m < M; m++) acc[1][m] = m < m_rows ? red[((wpt - 1) * M + m) * 64 + lane] : 0.0f;
+        for (int m = 0; m < M; m++) acc[1][m] = m < m_rows ? red_of(wpt)[m * 64 + lane] : 0.0f;
         for (int w = wpt + 1; w < waves; w++) {
 #pragma unroll
             for (int m = 0; m < M; m++)
-                if (m < m_rows) acc[1][m] += red[((w - 1) * M + m) * 64 + lane];
+                if (m < m_rows) acc[1][m] += red_of(w)[m * 64 + lane];
         }
     } else {
         tile_accumulate<NR, M, XBF16>(a.w, rt, panels, slice * waves + wave, slices * waves, a.k_dim, a.x, xoff, m_rows, xw, zero, acc);
         // waves of the block -> wave 0, in wave order
         if (waves > 1) {
             if (wave > 0) {
+                lds_f mine = red_of(wave);
 #pragma unroll
                 for (int r = 0; r < NR; r++)
 #pragma unroll
                     for (int m = 0; m < M; m++)
-                        if (m < m_rows) red[((wave - 1) * NR * M + r * M + m) * 64 + lane] = acc[r][m];
+                        if (m < m_rows) mine[(r * M + m) * 64 + lane] = acc[r][m];
             }
             __syncthreads();
             if (wave > 0) return;
@@ -446,7 +452,7 @@ __device__ __forceinline__ void gemv_body(const GemvArgs& a, unsigned z, lds_p l
                 for (int r = 0; r < NR; r++)
 #pragma unroll
                     for (int m = 0; m < M; m++)
-                        if (m < m_rows) acc[r][m] += red[((w - 1) * NR * M + r * M + m) * 64 + lane];
+                        if (m < m_rows) acc[r][m] += red_of(w)[(r * M + m) * 64 + lane];
             }
         }
     }

@@ -215,22 +215,22 @@ extern "C" __global__ void __launch_bounds__(1024) moe_down_combine(const unsign
     }
     const int t = (int)blockIdx.z, rt = (int)blockIdx.y, j = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6)), lane = lane_id();
     const int combo = t * topk + j;
-    // dynamic LDS: zeros, 4 staging rows per wave (f32 activations, one token: hi, mid, lo, zero), then one float per (wave, lane)
+    // dynamic LDS: zeros, 4 staging rows per wave (f32 activations, one token: hi, mid, lo, zero); a wave's weighted result
+    // for wave 0 goes where its staged activations were
+    typedef __attribute__((address_space(3))) float* lds_f;
     lds_p zero = LDS, xw = LDS + CROW_GEMV_ZERO_BYTES + j * (4 * CROW_GEMV_XROW_BYTES);
-    __attribute__((address_space(3))) float* red =
-        (__attribute__((address_space(3))) float*)(LDS + CROW_GEMV_ZERO_BYTES + topk * (4 * CROW_GEMV_XROW_BYTES));
     if (threadIdx.x < CROW_GEMV_ZERO_BYTES / 16) lds_store16(zero + 16 * threadIdx.x, 0, 0, 0, 0);
     __syncthreads();
     const unsigned char* const w[2] = {(const unsigned char*)ptrs[combo], nullptr};
     float acc[1][1];
     const size_t xoff[1] = {0};
     tile_accumulate<1, 1, false>(w, rt, (k + CROW_PANEL_COLS - 1) / CROW_PANEL_COLS, 0, 1, k, h + (size_t)combo * k, xoff, 1, xw, zero, acc);
-    red[j * 64 + lane] = rw[combo] * (acc[0][0] * gs_ptr[0]);
+    ((lds_f)xw)[lane] = rw[combo] * (acc[0][0] * gs_ptr[0]);
     __syncthreads();
     const int row = rt * CROW_TILE_ROWS + lane;
     if (j != 0 || row >= rows) return;
     float sum = 0.0f;
-    for (int q = 0; q < topk; q++) sum = __fadd_rn(sum, red[q * 64 + lane]);
+    for (int q = 0; q < topk; q++) sum = __fadd_rn(sum, ((lds_f)(LDS + CROW_GEMV_ZERO_BYTES + q * (4 * CROW_GEMV_XROW_BYTES)))[lane]);
     y[(size_t)t * rows + row] += sum;
 }
 
