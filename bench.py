@@ -29,8 +29,8 @@ for p in (ROOT, os.path.join(ROOT, "tests")):
 
 PEAK_HBM_GBS = 8000.0
 # HBM bytes per launch of the dominant kernel, measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE and scaled by
-# a 256 MiB copy kernel in the same run (profiles/gemv_nvfp4_gu_bf16__config1_m1.md): 101,142,440 read + 818,176 written
-TRAFFIC_GATE_UP_M1 = 101960616
+# a 256 MiB copy kernel in the same run (profiles/gemv_nvfp4_gu_bf16__config1_m1.md): 101,142,923 read + 818,176 written
+TRAFFIC_GATE_UP_M1 = 101961099
 N, K = 17408, 5120
 W_BYTES = N * K // 64 * 36  # 50,135,040: container encoding, 4.5 bits per weight
 
