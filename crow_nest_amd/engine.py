@@ -157,9 +157,9 @@ class Engine:
 
     def moe_layer(self, moe: MoeW, x: torch.Tensor, logits: torch.Tensor, y: torch.Tensor | None = None):
         """The routed part of one MoE layer with the launch sequence that is faster for this batch: per combo (three
-        launches) up to 47 tokens, grouped by expert (five launches, every expert slab read once per four combos) from 48
-        (measured crossover on MI355X at 256 experts, top-8: 16 tokens 48 / 57 us, 64 tokens 134 / 112 us)."""
-        if x.shape[0] >= 48:
+        launches) up to 23 tokens, grouped by expert (five launches, every expert slab read once per four combos) from 24
+        (measured on MI355X at 256 experts, top-8: 16 tokens 47 / 53 us, 24 tokens 65 / 63 us, 64 tokens 134 / 92 us)."""
+        if x.shape[0] >= 24:
             return self.moe_run_grouped(moe, x, logits, y)[:3]
         return self.moe_run(moe, x, logits, True, y)
 
