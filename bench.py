@@ -286,13 +286,18 @@ def main() -> int:
             ldn = Launch(eng, "moe_down_combine", H, I, t, [[dnp.data_ptr(), h2.data_ptr(), gs1.data_ptr(), wts.data_ptr(), yt.data_ptr(), p.i32(I), p.i32(H)]])
             ldn.dims = (1, (H + 63) // 64, t, 64 * K8)
 
-            seq2 = [(lr.f, lr.dims, lr.raw), (lgu.f, lgu.dims, lgu.raw), (ldn.f, ldn.dims, ldn.raw)]
-            time_sequence(seq2, len(lgs), 24)
-            us = min(time_sequence(seq2, len(lgs), 240) for _ in range(3))
+            # the layer as Engine.moe_layer runs it at these widths: the router inside the gate|up launch, then down + combine
+            lrg = Launch(eng, "moe_route_gate_up_silu", I, H, t * K8,
+                         [[l_.data_ptr(), moes[i_ % 3].table.data_ptr(), xt.data_ptr(), gs1.data_ptr(), h2.data_ptr(), ids.data_ptr(), wts.data_ptr(),
+                           dnp.data_ptr(), p.i32(H), p.i32(H), p.i32(I)] for i_, l_ in enumerate(lgs)])
             nbytes = int(distinct * (2 * I * H // 64 * 36 + H * I // 64 * 36)) + t * H * 8 + t * E * 4  # every distinct expert once
-            others[f"config2_moe_layer_T{t}"] = entry(us, nbytes)
-            others[f"config2_moe_layer_T{t}"]["launches"] = 3
-            others[f"config2_moe_layer_T{t}"]["distinct_experts_mean"] = round(distinct, 2)
+            for tag, seq in (("", [lrg, ldn]), ("_router_apart", [lr, lgu, ldn])):
+                seq2 = [(l_.f, l_.dims, l_.raw) for l_ in seq]
+                time_sequence(seq2, len(lgs), 24)
+                us = min(time_sequence(seq2, len(lgs), 240) for _ in range(3))
+                others[f"config2_moe_layer_T{t}{tag}"] = entry(us, nbytes)
+                others[f"config2_moe_layer_T{t}{tag}"]["launches"] = len(seq)
+                others[f"config2_moe_layer_T{t}{tag}"]["distinct_experts_mean"] = round(distinct, 2)
         # the same layer for a batch in which experts repeat (64 tokens): per combo against grouped by expert
         t = 64
         combos = t * K8

@@ -30,7 +30,7 @@ const FnEntry g_table[] = {
     CROW_GEMV(gemv_nvfp4_wm_bf16, 7, 1, 4, 4), CROW_GEMV(gemv_nvfp4_gum_bf16, 9, 2, 4, 4), CROW_GEMV(gemv_fp4, 6, 1, 1, 4),
     CROW_GEMV(gemv_fp4_b, 7, 1, 4, 12),        CROW_GEMV(gemv_fp4_b1k, 7, 1, 4, 12),      CROW_GEMV(gemv_fp4_bs, 8, 1, 4, 12),
     CROW_GEMV(gemv_fp4_ptrb, 8, 1, 1, 4),      CROW_GEMV(moe_gate_up_silu, 8, 1, 1, 4),   CROW_GEMV(moe_down_combine, 7, 1, 1, 4),
-    CROW_GEMV(moe_gate_up_silu_grouped, 11, 2, 4, 12), CROW_GEMV(moe_down_grouped, 9, 1, 4, 12), CROW_FN(moe_group, 6),
+    CROW_GEMV(moe_route_gate_up_silu, 11, 1, 1, 4), CROW_GEMV(moe_gate_up_silu_grouped, 11, 2, 4, 12), CROW_GEMV(moe_down_grouped, 9, 1, 4, 12), CROW_FN(moe_group, 6),
     CROW_FN(router_top10, 10),     CROW_FN(silu_mul_combo, 3),      CROW_FN(acc_combo, 3),
     CROW_FN(argmax_k, 3),          CROW_FN(argmax_tiles, 2),        CROW_FN(dequant_fp4_flat, 4),    CROW_FN(repack_nvfp4, 4),
     CROW_FN(unpack_nvfp4, 4),      CROW_FN(dequant_nvfp4_tiled, 5),
@@ -268,11 +268,12 @@ int crow_hip_launch_dims_split(const char* name, uint32_t rows, uint32_t k_dim, 
         *out = crow_dims{(rows + 3) / 4, z, 1, 256};
         return CROW_OK;
     }
-    if (strncmp(name, "gemv_", 5) == 0 || strncmp(name, "moe_gate_up", 11) == 0 || strcmp(name, "moe_down_grouped") == 0) {
+    if (strncmp(name, "gemv_", 5) == 0 || strncmp(name, "moe_gate_up", 11) == 0 || strcmp(name, "moe_down_grouped") == 0 ||
+        strcmp(name, "moe_route_gate_up_silu") == 0) {
         if (k_dim == 0 || k_dim % CROW_BLOCK_VALUES != 0) return CROW_ERR_SHAPE;
         const bool moe = strcmp(name, "gemv_fp4_ptrb") == 0 || strncmp(name, "moe_", 4) == 0;
         const bool tokens = strcmp(name, "gemv_fp4_b") == 0 || strcmp(name, "gemv_fp4_b1k") == 0 || strcmp(name, "gemv_fp4_bs") == 0;
-        const bool two = strstr(name, "_gu") != nullptr || strncmp(name, "moe_gate_up", 11) == 0;
+        const bool two = strstr(name, "_gu") != nullptr || strncmp(name, "moe_gate_up", 11) == 0 || strcmp(name, "moe_route_gate_up_silu") == 0;
         const uint32_t tiles = rt;  // rows = output rows for every kernel
         const uint32_t gz = moe ? z : (tokens ? (z + 3) / 4 : 1);
         // A tile's panels are dealt to S blocks of W waves.  Measured on MI355X (17408 x 5120,
@@ -298,7 +299,8 @@ int crow_hip_launch_dims_split(const char* name, uint32_t rows, uint32_t k_dim, 
         if (force_s > 0) s = force_s;
         if (force_w > 0) w = force_w;
         // gate/up kernels for one activation row run one tile per wave: 2 W waves per block (W per tensor), at most 1024 threads
-        const bool thin = strcmp(name, "gemv_nvfp4_gu") == 0 || strcmp(name, "gemv_nvfp4_gu_bf16") == 0 || strcmp(name, "moe_gate_up_silu") == 0;
+        const bool thin = strcmp(name, "gemv_nvfp4_gu") == 0 || strcmp(name, "gemv_nvfp4_gu_bf16") == 0 || strcmp(name, "moe_gate_up_silu") == 0 ||
+                          strcmp(name, "moe_route_gate_up_silu") == 0;
         // (the two-tensor kernels on four f32 rows are built for blocks of at most 512 threads)
         const bool half = thin || strcmp(name, "gemv_nvfp4_gum") == 0 || strcmp(name, "moe_gate_up_silu_grouped") == 0;
         if (w > (half ? 8 : 16)) w = half ? 8 : 16;

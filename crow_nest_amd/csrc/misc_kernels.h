@@ -132,15 +132,51 @@ __device__ __forceinline__ unsigned wave_umax(unsigned v) {
     return (unsigned)__builtin_amdgcn_readlane((int)v, 63);
 }
 
+// Wave-wide float maximum, the same lane moves as wave_umax (identity -inf); and the halving-tree sum in which lane t takes
+// lane t + 32, then + 16 (the two half / quarter swaps), then + 8, 4, 2, 1 (row shifts): lane 0 ends with exactly the sum a
+// shuffle-down tree gives, each step the same single f32 addition.  Both return the result in every lane.
+template <int CTRL, int ROW_MASK>
+__device__ __forceinline__ float dpp_fmax_step(float v) {
+    const float o = __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(__builtin_bit_cast(int, -INFINITY), __builtin_bit_cast(int, v), CTRL, ROW_MASK, 0xf, false));
+    return fmaxf(o, v);
+}
+__device__ __forceinline__ float wave_fmax(float v) {
+    v = dpp_fmax_step<0x111, 0xf>(v);
+    v = dpp_fmax_step<0x112, 0xf>(v);
+    v = dpp_fmax_step<0x114, 0xf>(v);
+    v = dpp_fmax_step<0x118, 0xf>(v);
+    v = dpp_fmax_step<0x142, 0xa>(v);
+    v = dpp_fmax_step<0x143, 0xc>(v);
+    return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), 63));
+}
+template <int CTRL>
+__device__ __forceinline__ float dpp_shl_add(float v) {  // lane t: v[t] + v[t + n] inside its row of 16 (row_shl:n); lanes without a source add 0
+    const float o = __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xf, 0xf, false));
+    return __fadd_rn(v, o);
+}
+__device__ __forceinline__ float wave_tree_sum(float v) {
+    const unsigned b = __float_as_uint(v);
+    const u32x2 h = __builtin_amdgcn_permlane32_swap(b, b, false, false);  // .x = lanes 0..31's value, .y = lanes 32..63's
+    v = __fadd_rn(__uint_as_float(h.x), __uint_as_float(h.y));
+    const unsigned c = __float_as_uint(v);
+    const u32x2 q = __builtin_amdgcn_permlane16_swap(c, c, false, false);  // .x = the even 16-lane group's value, .y = the odd one's
+    v = __fadd_rn(__uint_as_float(q.x), __uint_as_float(q.y));
+    v = dpp_shl_add<0x108>(v);
+    v = dpp_shl_add<0x104>(v);
+    v = dpp_shl_add<0x102>(v);
+    v = dpp_shl_add<0x101>(v);
+    return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), 0));
+}
+
 // One token's routing on one wavefront, SLOTS = E / 64 experts per lane: expert e lives in lane e % 64, slot e / 64.
 template <int SLOTS>
 __device__ __forceinline__ void router_body(const float* __restrict__ logits, const unsigned int* __restrict__ bitmap, int* __restrict__ ids,
                                             float* __restrict__ wts, unsigned long long* __restrict__ gu_ptrs,
                                             unsigned long long* __restrict__ dn_ptrs, const unsigned long long* __restrict__ table,
                                             unsigned int* __restrict__ cold_mask, unsigned long long* __restrict__ counters,
-                                            unsigned long long* __restrict__ sel_counts, int K) {
+                                            unsigned long long* __restrict__ sel_counts, int K, int t, bool write, int& picked) {
     constexpr int E = SLOTS * 64;
-    const int t = (int)blockIdx.x, lane = lane_id();
+    const int lane = lane_id();
     float l[SLOTS], red[SLOTS];
     float mx = -INFINITY;
 #pragma unroll
@@ -148,7 +184,7 @@ __device__ __forceinline__ void router_body(const float* __restrict__ logits, co
         l[j] = logits[(size_t)t * E + j * 64 + lane];
         mx = fmaxf(mx, l[j]);
     }
-    for (int o = 32; o > 0; o >>= 1) mx = fmaxf(mx, __shfl_xor(mx, o));
+    mx = wave_fmax(mx);
 #pragma unroll
     for (int j = 0; j < SLOTS; j++) red[j] = l[j] = expf(l[j] - mx);
     // tree over E slots: strides E/2 .. 64 pair slots inside a lane, strides 32 .. 1 pair lanes
@@ -156,9 +192,7 @@ __device__ __forceinline__ void router_body(const float* __restrict__ logits, co
     for (int st = SLOTS / 2; st > 0; st >>= 1)
 #pragma unroll
         for (int j = 0; j < st; j++) red[j] += red[j + st];
-    float den = red[0];
-    for (int o = 32; o > 0; o >>= 1) den += __shfl_down(den, o);
-    den = __shfl(den, 0);
+    const float den = wave_tree_sum(red[0]);
     // keys: probabilities are >= 0, so their bit patterns order like the values; + 1 keeps 0 for "already picked"
     unsigned key[SLOTS];
 #pragma unroll
@@ -195,6 +229,8 @@ __device__ __forceinline__ void router_body(const float* __restrict__ logits, co
                 if (j == (pick >> 6)) key[j] = 0u;
         }
     }
+    picked = my_id;  // lane k: the k-th pick
+    if (!write) return;
     unsigned cold = 0;
     if (lane < K) {
         wts[(size_t)t * K + lane] = my_w / sum;
@@ -218,6 +254,20 @@ __device__ __forceinline__ void router_body(const float* __restrict__ logits, co
     }
 }
 
+__device__ __forceinline__ void router_dispatch(int E, const float* __restrict__ logits, const unsigned int* __restrict__ bitmap, int* __restrict__ ids,
+                                                float* __restrict__ wts, unsigned long long* __restrict__ gu_ptrs, unsigned long long* __restrict__ dn_ptrs,
+                                                const unsigned long long* __restrict__ table, unsigned int* __restrict__ cold_mask,
+                                                unsigned long long* __restrict__ counters, unsigned long long* __restrict__ sel_counts, int K, int t,
+                                                bool write, int& picked) {
+    switch (E >> 6) {
+        case 1: router_body<1>(logits, bitmap, ids, wts, gu_ptrs, dn_ptrs, table, cold_mask, counters, sel_counts, K, t, write, picked); break;
+        case 2: router_body<2>(logits, bitmap, ids, wts, gu_ptrs, dn_ptrs, table, cold_mask, counters, sel_counts, K, t, write, picked); break;
+        case 4: router_body<4>(logits, bitmap, ids, wts, gu_ptrs, dn_ptrs, table, cold_mask, counters, sel_counts, K, t, write, picked); break;
+        case 8: router_body<8>(logits, bitmap, ids, wts, gu_ptrs, dn_ptrs, table, cold_mask, counters, sel_counts, K, t, write, picked); break;
+        default: router_body<16>(logits, bitmap, ids, wts, gu_ptrs, dn_ptrs, table, cold_mask, counters, sel_counts, K, t, write, picked); break;
+    }
+}
+
 // reference: router_top10, engine/src/kernels.rs:3109-3184.  grid (T), block 64: one wavefront per
 // token.  The softmax denominator is added in the reference's halving-tree order (slots first, then
 // lanes), so weights match an E-thread tree.  Ties go to the lowest expert id.
@@ -233,13 +283,39 @@ extern "C" __global__ void __launch_bounds__(64) router_top10(const float* __res
         if (threadIdx.x == 0) atomicOr(g_ws.status, STATUS_BAD_GEO);
         return;
     }
-    switch (E >> 6) {
-        case 1: router_body<1>(logits, bitmap, ids, wts, gu_ptrs, dn_ptrs, table, cold_mask, counters, sel_counts, K); break;
-        case 2: router_body<2>(logits, bitmap, ids, wts, gu_ptrs, dn_ptrs, table, cold_mask, counters, sel_counts, K); break;
-        case 4: router_body<4>(logits, bitmap, ids, wts, gu_ptrs, dn_ptrs, table, cold_mask, counters, sel_counts, K); break;
-        case 8: router_body<8>(logits, bitmap, ids, wts, gu_ptrs, dn_ptrs, table, cold_mask, counters, sel_counts, K); break;
-        default: router_body<16>(logits, bitmap, ids, wts, gu_ptrs, dn_ptrs, table, cold_mask, counters, sel_counts, K); break;
+    int picked;
+    router_dispatch(E, logits, bitmap, ids, wts, gu_ptrs, dn_ptrs, table, cold_mask, counters, sel_counts, K, (int)blockIdx.x, true, picked);
+}
+
+// Router and routed gate|up + SwiGLU in ONE launch: every block works out its token's routing itself (wave 0; the
+// logits row is 1 KB) instead of reading pointers a router launch left behind, which takes a launch (4 us back to back) off
+// the layer.  grid (1, inter / 64, T K), block 1024 as moe_gate_up_silu.  Block (row tile 0, pick 0) of each token writes
+// ids, wts and dn_ptrs for moe_down_combine.  table[2 e] / table[2 e + 1] = gate|up / down slab of expert e.
+extern "C" __global__ void __launch_bounds__(1024) moe_route_gate_up_silu(const float* __restrict__ logits, const unsigned long long* __restrict__ table,
+                                                                          const float* __restrict__ x, const float* __restrict__ gs_ptr,
+                                                                          float* __restrict__ h, int* __restrict__ ids, float* __restrict__ wts,
+                                                                          unsigned long long* __restrict__ dn_ptrs, const int* __restrict__ k_dim_p,
+                                                                          const int* __restrict__ x_stride_p, const int* __restrict__ inter_p) {
+    ENTER(logits, table, x, gs_ptr, h, ids, wts, dn_ptrs, k_dim_p, x_stride_p, inter_p);
+    __shared__ unsigned long long s_slab;
+    const int E = g_geo.experts, K = g_geo.topk;
+    if (E < 64 || E > 1024 || (E & (E - 1)) != 0 || K < 1 || K > 16 || K > E || table == nullptr) {
+        if (threadIdx.x == 0) atomicOr(ws.status, STATUS_BAD_GEO);
+        return;
     }
+    const int combo = (int)blockIdx.z, t = combo / K, j = combo % K;
+    if (threadIdx.x < 64) {  // wave 0
+        int picked;
+        router_dispatch(E, logits, nullptr, ids, wts, nullptr, dn_ptrs, table, nullptr, nullptr, nullptr, K, t, blockIdx.y == 0 && j == 0, picked);
+        const int e = __builtin_amdgcn_readlane(picked, j);
+        if (threadIdx.x == 0) s_slab = table[2 * e];
+    }
+    __syncthreads();
+    const int inter = *inter_p, k = *k_dim_p;
+    const unsigned char* w = (const unsigned char*)s_slab;
+    const size_t up_off = (size_t)(inter / CROW_TILE_ROWS) * ((k + CROW_PANEL_COLS - 1) / CROW_PANEL_COLS) * CROW_TILE_BYTES;
+    GemvArgs a{{w, w + up_off}, {gs_ptr, gs_ptr}, x + (size_t)t * *x_stride_p, 0, h + (size_t)combo * inter, 0, k, inter, 1, nullptr};
+    gemv_body<2, 1, false, EPI_SILU_GU, XRows<1, false>::value, true>(a, blockIdx.z, LDS, ws);
 }
 
 // Sort the n routed combos of a batch by expert and cut them into tiles of at most four combos of one expert: the work of

@@ -156,12 +156,14 @@ class Engine:
         return ids, wts, gu, dn
 
     def moe_layer(self, moe: MoeW, x: torch.Tensor, logits: torch.Tensor, y: torch.Tensor | None = None):
-        """The routed part of one MoE layer with the launch sequence that is faster for this batch: per combo (three
-        launches) up to 23 tokens, grouped by expert (five launches, every expert slab read once per four combos) from 24
-        (measured on MI355X at 256 experts, top-8: 16 tokens 47 / 53 us, 24 tokens 65 / 63 us, 64 tokens 134 / 92 us)."""
+        """The routed part of one MoE layer with the launch sequence that is faster for this batch, as measured on MI355X at
+        256 experts, top-8: up to 4 tokens the router rides inside the gate|up launch (two launches: 1 token 16.0 us against
+        17.5 us for three, 4 tokens 18.8 / 20.4; at 8 tokens 29.4 / 29.0, every block repeating its token's routing no longer
+        pays); 5 to 23 tokens per combo in three launches; from 24 grouped by expert (five launches, every expert slab read
+        once per four combos: 16 tokens 47 / 53 us per combo / grouped, 24 tokens 65 / 63, 64 tokens 134 / 92)."""
         if x.shape[0] >= 24:
             return self.moe_run_grouped(moe, x, logits, y)[:3]
-        return self.moe_run(moe, x, logits, True, y)
+        return self.moe_run(moe, x, logits, "route" if x.shape[0] <= 4 else True, y)
 
     def moe_run_grouped(self, moe: MoeW, x: torch.Tensor, logits: torch.Tensor, y: torch.Tensor | None = None):
         """The routed part of one MoE layer for a batch in which experts repeat: router_top10, moe_group (combos sorted by
@@ -195,17 +197,29 @@ class Engine:
     def moe_run(self, moe: MoeW, x: torch.Tensor, logits: torch.Tensor, fused: bool = True, y: torch.Tensor | None = None):
         """Routed part of one MoE layer: y[t][H] (+)= sum_j w_j * down_e(silu(gate_e x) * up_e x).
         fused=False walks the reference's five launches (router_top10, gemv_fp4_ptrb, silu_mul_combo,
-        gemv_fp4_ptrb, acc_combo); fused=True uses moe_gate_up_silu + moe_down_combine."""
+        gemv_fp4_ptrb, acc_combo); fused=True uses router_top10 + moe_gate_up_silu + moe_down_combine; fused="route"
+        takes the router into the gate|up launch (moe_route_gate_up_silu + moe_down_combine: two launches)."""
         t, hdim = x.shape
         inter, topk = self.geo.inter, self.geo.topk
         assert hdim == self.geo.hidden and moe.gate_up.rows == 2 * inter and moe.down.rows == hdim
         p = self.p
-        ids, wts, gu, dn = self.router(logits, moe)
         combos = t * topk
         if y is None:
             y = torch.zeros((t, hdim), dtype=torch.float32, device=self.dev)
         gs_gu, gs_dn = moe.gate_up.gs.data_ptr(), moe.down.gs.data_ptr()
         h2 = torch.empty((combos, inter), dtype=torch.float32, device=self.dev)
+        if fused == "route":
+            assert logits.shape == (t, self.geo.experts) and logits.dtype == torch.float32 and logits.is_contiguous()
+            ids = torch.empty((t, topk), dtype=torch.int32, device=self.dev)
+            wts = torch.empty((t, topk), dtype=torch.float32, device=self.dev)
+            dn = torch.zeros((t, topk), dtype=torch.int64, device=self.dev)
+            launch_v(self.k.f("moe_route_gate_up_silu"), *launch_dims("moe_route_gate_up_silu", inter, hdim, combos),
+                     [logits.data_ptr(), moe.table.data_ptr(), x.data_ptr(), gs_gu, h2.data_ptr(), ids.data_ptr(), wts.data_ptr(), dn.data_ptr(),
+                      p.i32(hdim), p.i32(hdim), p.i32(inter)])
+            launch_v(self.k.f("moe_down_combine"), *launch_dims("moe_down_combine", hdim, inter, t),
+                     [dn.data_ptr(), h2.data_ptr(), gs_dn, wts.data_ptr(), y.data_ptr(), p.i32(inter), p.i32(hdim)])
+            return ids, wts, y
+        ids, wts, gu, dn = self.router(logits, moe)
         if fused:
             gx, gy, gz, bx = launch_dims("moe_gate_up_silu", inter, hdim, combos)
             launch_v(self.k.f("moe_gate_up_silu"), gx, gy, gz, bx,

@@ -72,6 +72,10 @@ CROW_KERNEL(acc_combo, 3)      /* x, rw, y.     kernels.rs:1583-1592 */
 /* ptrs, x, gs, h, k_dim_p, x_div_p, x_stride_p, inter_p.  gemv_fp4_ptrb on a fused gate_up slab + silu_mul_combo in one
  * launch: h[c][i] = silu(gate_c x)[i] * (up_c x)[i]. */
 CROW_KERNEL(moe_gate_up_silu, 8)
+/* logits, table, x, gs, h, ids, wts, dn_ptrs, k_dim_p, x_stride_p, inter_p.  router_top10 + moe_gate_up_silu in one launch:
+ * every block works out its token's routing itself and takes its slab from table[2 e]; one block per token writes ids, wts
+ * and dn_ptrs (table[2 e + 1]) for moe_down_combine.  Same routing, same h as the two launches it replaces. */
+CROW_KERNEL(moe_route_gate_up_silu, 11)
 /* ptrs, h, gs, rw, y, k_dim_p, rows_p.  gemv_fp4_ptrb on the down slabs + acc_combo in one launch: y[t] = sum over the
  * token's combos j, in j order, of rw[t][j] * (down_j h_j). */
 CROW_KERNEL(moe_down_combine, 7)

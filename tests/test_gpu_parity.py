@@ -300,7 +300,7 @@ def test_moe_layer_both_launch_sequences(eng, t):
     x = (normal_f32(5, t, t * H) * np.float32(0.1)).reshape(t, H)
     logits = normal_f32(6, t, t * E).reshape(t, E)
     ids_ref, w_ref, y_ref = orc.moe_layer(gu, gs_gu, dn, gs_dn, E, H, I, x, logits, K, threads=8)
-    for fused in (False, True):
+    for fused in (False, True, "route"):
         print(f"case moe t={t} fused={fused}", flush=True)
         ids, wts, y = eng.moe_run(moe, _dev(x), _dev(logits), fused=fused)
         eng.check()
