@@ -134,6 +134,30 @@ def test_gemv_is_correct_for_every_split(eng, s, wv):
     assert rel_err(y1, ref) <= TOL and gamma_ratio(y1, w, rows, cols, gs, x) <= 1.0
 
 
+def test_split_launches_back_to_back_with_changing_inputs(eng):
+    """A small cross-block split launched 24 times in a row without a host wait, every launch on another x: the partial
+    sums a block reads are the ones this launch's blocks wrote, never an earlier launch's (the launches are small enough
+    for all of their lines to stay in the caches between them)."""
+    rows, cols, n = 128, 4096, 24
+    w = random_nvfp4(91, rows, cols)
+    gs = 6.0e-4
+    f = _load(w, rows, cols, gs)
+    from crow_nest_amd.kernels import launch_dims, launch_v
+    xs = normal_f32(6, 1, n * cols).reshape(n, cols) * np.linspace(0.25, 4.0, n, dtype=np.float32)[:, None]
+    xd = _dev(xs)
+    p = eng.p
+    for s, wv in ((4, 4), (16, 1), (2, 8)):
+        dims = launch_dims("gemv_nvfp4_w", rows, cols, 1, split=(s, wv))
+        y = torch.empty((n, rows), dtype=torch.float32, device="cuda")
+        for i in range(n):
+            launch_v(eng.k.f("gemv_nvfp4_w"), *dims, [f.w_ptr, xd[i].data_ptr(), f.gs_ptr, y[i].data_ptr(), p.i32(cols), p.i32(rows)])
+        eng.check()
+        got = y.cpu().numpy()
+        ref = orc.gemv(w, rows, cols, gs, xs)
+        for i in range(n):
+            assert rel_err(got[i], ref[i]) <= TOL, (s, wv, i)
+
+
 def test_verify_rows_are_bit_identical_to_one_row_decode(eng):
     """kernels_p2.rs:391-396: row m of an M-row launch == a one-row launch on x row m."""
     rows, cols = 700, 5120
