@@ -57,8 +57,8 @@ struct State {
 const unsigned long long PARTIAL_FLOATS = 16ull << 20;  // 64 MiB of split-K partial sums
 const unsigned COUNTER_SLOTS = 1u << 16;
 const unsigned AM_SLOTS = 1u << 16;
-// tile counters, then the status word, then 1 + AM_SLOTS / 64 argmax counters (top, groups)
-const unsigned COUNTER_WORDS = COUNTER_SLOTS + 1 + 1 + AM_SLOTS / 64;
+// tile counters, then the status word
+const unsigned COUNTER_WORDS = COUNTER_SLOTS + 1;
 
 int hip_rc(hipError_t e) { return e == hipSuccess ? CROW_OK : (int)e; }
 
@@ -126,7 +126,6 @@ int crow_hip_init(int device) {
     if ((e = hipMalloc((void**)&scalars, 16 * sizeof(int))) != hipSuccess) return fail(e);
     if ((e = hipMemset(ws.counters, 0, COUNTER_WORDS * sizeof(unsigned))) != hipSuccess) return fail(e);
     ws.status = ws.counters + COUNTER_SLOTS;
-    ws.am_counter = ws.counters + COUNTER_SLOTS + 1;
     if ((e = hipMemcpyToSymbol(HIP_SYMBOL(crow::g_ws), &ws, sizeof ws)) != hipSuccess) return fail(e);
     crow::Geo geo{0, 0, 0, 0};
     if ((e = hipMemcpyToSymbol(HIP_SYMBOL(crow::g_geo), &geo, sizeof geo)) != hipSuccess) return fail(e);

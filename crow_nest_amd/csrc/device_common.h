@@ -40,7 +40,6 @@ struct Workspace {
     unsigned* status;                   // device word: non-zero = a launch did not fit the workspace
     float* am_val;                      // fused lm_head argmax: one (value, index) candidate per row tile
     int* am_idx;
-    unsigned* am_counter;
     unsigned am_slots;
 };
 __device__ Workspace g_ws;
