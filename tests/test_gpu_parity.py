@@ -456,10 +456,19 @@ def test_config3_full_size_head(eng):
 
 @pytest.mark.parametrize("kernel", ["gemm_nvfp4_bf16_m16", "gemm_nvfp4_bf16_m32", "gemm_nvfp4_bf16_m48", "gemm_nvfp4_bf16_m64", "gemm_nvfp4_bf16_m96",
                                     "gemm_nvfp4_bf16"])
-@pytest.mark.parametrize("m,rows,cols", [(16, 320, 1024), (5, 100, 320), (16, 17408, 5120), (17, 100, 320), (33, 256, 512), (128, 512, 2048), (200, 192, 5120)])
+@pytest.mark.parametrize("m,rows,cols", [(16, 320, 1024), (5, 100, 320), (17, 100, 320), (33, 256, 512), (128, 512, 2048), (200, 192, 5120)])
 def test_gemm_bf16_against_the_cpu_path(eng, m, rows, cols, kernel):
     """Weights decode to exact bf16, X is bf16, products are exact in f32: only the summation order
     differs from the CPU path (which gets the exactly widened X)."""
+    _gemm_case(eng, m, rows, cols, kernel)
+
+
+def test_gemm_m16_full_size_cross_block_split(eng):
+    """[17408, 5120] at 16 tokens: the K-split kernel's five column slices meet through the workspace."""
+    _gemm_case(eng, 16, 17408, 5120, "gemm_nvfp4_bf16_m16")
+
+
+def _gemm_case(eng, m, rows, cols, kernel):
     print(f"case m={m} rows={rows} cols={cols} {kernel}", flush=True)
     if kernel == "gemm_nvfp4_bf16_m16" and m > 16:
         from crow_nest_amd.kernels import launch_dims
@@ -467,8 +476,6 @@ def test_gemm_bf16_against_the_cpu_path(eng, m, rows, cols, kernel):
         with pytest.raises(CrowHipError):  # refused on the host, nothing launched
             launch_dims(kernel, rows, cols, m)
         return
-    if rows > 1024 and kernel != "gemm_nvfp4_bf16_m16":
-        pytest.skip("the full-size case is there for the cross-block split")
     w = random_nvfp4(m * 7 + rows, rows, cols)
     gs = 6.0e-4
     f = _load(w, rows, cols, gs)
