@@ -255,6 +255,12 @@ def main() -> int:
             lb = Launch(eng, "gemv_bf16_w", rows_b, k_b, 1, [[w_.data_ptr(), xb_.data_ptr(), ybuf.data_ptr(), p.i32(k_b), p.i32(rows_b)] for w_ in wbs])
             others[f"bf16_keep_gemv_{rows_b}x{k_b}"] = entry(lb.us(), rows_b * k_b * 2 + k_b * 4 + rows_b * 4)
             del wbs
+        # the f32 router projection [256, 2560] (gemv_b: its result is the router's logits)
+        wr = [torch.randn(256, 2560, device=dev) for _ in range(16)]
+        xr = torch.randn(2560, device=dev)
+        lrp = Launch(eng, "gemv_b", 256, 2560, 1, [[w_.data_ptr(), xr.data_ptr(), ybuf.data_ptr(), p.i32(2560), p.i32(256)] for w_ in wr])
+        others["f32_router_gemv_256x2560"] = entry(lrp.us(), 256 * 2560 * 4 + 2560 * 4 + 256 * 4)
+        del wr
         # config 2: one MoE layer, 256 experts top-8, H 2048, I 512 (router + fused gate|up+SiLU + fused down+combine)
         from crow_nest_amd.engine import MoeW, expert_table
         from crow_nest_amd.weights import ExpertSlabs

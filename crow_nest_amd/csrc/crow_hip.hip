@@ -40,6 +40,7 @@ const FnEntry g_table[] = {
     {"gemm_nvfp4_bf16_m48", (const void*)&gemm_nvfp4_bf16_m48, 7, 2u * 48u * 528u, 0u},
     {"gemm_nvfp4_bf16_m96", (const void*)&gemm_nvfp4_bf16_m96, 7, 2u * 96u * 528u, 0u},
     CROW_FN(gemm_nvfp4_bf16_m32, 7), CROW_FN(gemm_nvfp4_bf16_m16, 7), CROW_FN(gemv_bf16_w, 5),
+    CROW_FN(gemv_bf16, 5), CROW_FN(gemv_bf16_b, 5), CROW_FN(gemv_b, 5),
 };
 const int g_table_n = (int)(sizeof(g_table) / sizeof(g_table[0]));
 
@@ -262,8 +263,15 @@ int crow_hip_launch_dims_split(const char* name, uint32_t rows, uint32_t k_dim, 
     if (!e) return CROW_ERR_KERNEL_MISSING;
     const uint32_t rt = (rows + CROW_TILE_ROWS - 1) / CROW_TILE_ROWS;
     const uint32_t panels = (k_dim + CROW_PANEL_COLS - 1) / CROW_PANEL_COLS;
-    if (strcmp(name, "gemv_bf16_w") == 0) {  // z = T activation rows
-        if (k_dim == 0 || k_dim % 8 != 0) return CROW_ERR_SHAPE;
+    if (strcmp(name, "gemv_bf16_w") == 0 || strcmp(name, "gemv_bf16") == 0 || strcmp(name, "gemv_bf16_b") == 0 || strcmp(name, "gemv_b") == 0) {
+        // z = T activation rows; whole 16-byte loads: 8 bf16 or 4 f32 weights
+        if (k_dim == 0 || k_dim % (strcmp(name, "gemv_b") == 0 ? 4 : 8) != 0) return CROW_ERR_SHAPE;
+        if (strcmp(name, "gemv_bf16") == 0 && z != 1) return CROW_ERR_SHAPE;  // the one-token form
+        // short tensors: a block of four waves per (row, token); force_w = 4 / 1 asks for one shape or the other
+        if (force_w == 4 || (force_w == 0 && (unsigned long long)rows * z <= 2048)) {
+            *out = crow_dims{rows, z, 1, 256};
+            return CROW_OK;
+        }
         *out = crow_dims{(rows + 3) / 4, z, 1, 256};
         return CROW_OK;
     }

@@ -501,47 +501,87 @@ extern "C" __global__ void __launch_bounds__(256) argmax_tiles(int* __restrict__
     }
 }
 
-// ------------------------------------------------------------------ BF16 keeps
-// reference: gemv_bf16_w, engine/src/kernels.rs:1130-1157 - y[t][row] = sum_k bf16(w[row][k]) * x[t][k] for the tensors the
-// container keeps in bf16 (router, q/k, MTP head), f32 activations, f32 accumulation; k_dim % 8 == 0.
-// One wavefront per (row, t): grid (ceil(rows / 4), T), block 256 = 4 rows; 16-byte non-temporal weight loads (8 bf16 per
-// lane per step, 1024 contiguous bytes per instruction), x through the vector cache (it is re-read by every row).
-// Order: a lane adds its products in column order with one FMA each (columns 8 lane + 512 j + 0..7), then the 64 lane sums
-// are added by halving (lane l += lane l + 32, + 16, ... + 1).
-extern "C" __global__ void __launch_bounds__(256) gemv_bf16_w(const unsigned short* __restrict__ w, const float* __restrict__ x,
-                                                              float* __restrict__ y, const int* __restrict__ k_dim_p,
-                                                              const int* __restrict__ rows_p) {
-    const int k = *k_dim_p, rows = *rows_p;
+// ------------------------------------------------------------------ BF16 and F32 keeps
+// The tensors the container keeps unquantised (router, q/k, MTP head): y[t][row] = sum_k w[row][k] * x[t][k], f32
+// activations, f32 accumulation.  16-byte non-temporal weight loads (8 bf16 or 4 f32 per lane per step: 1024 contiguous
+// bytes per wave instruction), x through the vector cache (it is re-read by every row).  Two launch shapes, told apart by
+// grid.x, block 256 in both:
+//   grid (ceil(rows / 4), T)   one wavefront per (row, t): the shape for tall tensors (crow_hip_launch_dims picks it
+//                              when rows * T > 2048)
+//   grid (rows, T)             one block per (row, t), its four waves take every fourth 1024-byte run of the row and add
+//                              their sums in wave order through LDS: a short tensor (the router: 256 rows) still puts a
+//                              thousand waves on the chip, and a row's loads are all in flight at once.  This is also
+//                              the grid of the reference's block-per-row kernels, whose call sites keep their dims.
+// Order: a lane adds its products in column order with one FMA each, four steps of loads in flight at a time, then the
+// 64 lane sums are added by halving (lane l += lane l + 32, + 16, ... + 1), then (second shape) the wave sums in wave order.
+//   gemv_bf16_w   engine/src/kernels.rs:1130-1157 (warp per row; k_dim % 8 == 0)
+//   gemv_bf16     engine/src/kernels.rs:1061-1077 (block per row, one token; + rows_p: the reference's grid.x is the row count)
+//   gemv_bf16_b   engine/src/kernels.rs:1080-1098 (block per row, grid.y tokens; + rows_p)
+//   gemv_b        engine/src/kernels.rs:97-115   (f32 weights, the router projection of gen.rs:4182; + rows_p; k_dim % 4 == 0)
+template <bool WBF16>
+__device__ __forceinline__ void keep_gemv_body(const void* __restrict__ w, const float* __restrict__ x, float* __restrict__ y, int k, int rows) {
+    constexpr int PER = WBF16 ? 8 : 4;  // weights per 16-byte load
+    __shared__ float wave_sum[4];
     const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6)), lane = lane_id();
-    const int row = (int)blockIdx.x * 4 + wave, t = (int)blockIdx.y;
-    if (row >= rows) return;
-    const unsigned short* wp = w + (size_t)row * k;
+    const bool block_per_row = gridDim.x == (unsigned)rows;  // uniform over the launch
+    const int row = block_per_row ? (int)blockIdx.x : (int)blockIdx.x * 4 + wave, t = (int)blockIdx.y;
+    if (row >= rows) return;  // (first shape only: a whole wave leaves, nobody waits for it)
+    const int parts = block_per_row ? 4 : 1, part = block_per_row ? wave : 0;
+    const char* wp = (const char*)w + (size_t)row * k * (WBF16 ? 2 : 4);
     const float* xp = x + (size_t)t * k;
+    const int run = parts * 64 * PER;  // columns between two loads of a lane
     float acc = 0.0f;
-    for (int i0 = lane * 8; i0 < k; i0 += 4 * 512) {
+    for (int i0 = (part * 64 + lane) * PER; i0 < k; i0 += 4 * run) {
         uint4 v[4];
 #pragma unroll
         for (int j = 0; j < 4; j++) {
-            const int i = i0 + j * 512;
+            const int i = i0 + j * run;
             v[j] = make_uint4(0, 0, 0, 0);
-            if (i < k) v[j] = stream_load((const uint4*)(wp + i));
+            if (i < k) v[j] = stream_load((const uint4*)(wp + (size_t)i * (WBF16 ? 2 : 4)));
         }
 #pragma unroll
         for (int j = 0; j < 4; j++) {
-            const int i = i0 + j * 512;
+            const int i = i0 + j * run;
             if (i < k) {
-                const float4 a = *(const float4*)(xp + i), b = *(const float4*)(xp + i + 4);
-                acc = __builtin_fmaf(__uint_as_float(v[j].x << 16), a.x, acc);
-                acc = __builtin_fmaf(__uint_as_float(v[j].x & 0xffff0000u), a.y, acc);
-                acc = __builtin_fmaf(__uint_as_float(v[j].y << 16), a.z, acc);
-                acc = __builtin_fmaf(__uint_as_float(v[j].y & 0xffff0000u), a.w, acc);
-                acc = __builtin_fmaf(__uint_as_float(v[j].z << 16), b.x, acc);
-                acc = __builtin_fmaf(__uint_as_float(v[j].z & 0xffff0000u), b.y, acc);
-                acc = __builtin_fmaf(__uint_as_float(v[j].w << 16), b.z, acc);
-                acc = __builtin_fmaf(__uint_as_float(v[j].w & 0xffff0000u), b.w, acc);
+                const float4 a = *(const float4*)(xp + i);
+                if (WBF16) {
+                    const float4 b = *(const float4*)(xp + i + 4);
+                    acc = __builtin_fmaf(__uint_as_float(v[j].x << 16), a.x, acc);
+                    acc = __builtin_fmaf(__uint_as_float(v[j].x & 0xffff0000u), a.y, acc);
+                    acc = __builtin_fmaf(__uint_as_float(v[j].y << 16), a.z, acc);
+                    acc = __builtin_fmaf(__uint_as_float(v[j].y & 0xffff0000u), a.w, acc);
+                    acc = __builtin_fmaf(__uint_as_float(v[j].z << 16), b.x, acc);
+                    acc = __builtin_fmaf(__uint_as_float(v[j].z & 0xffff0000u), b.y, acc);
+                    acc = __builtin_fmaf(__uint_as_float(v[j].w << 16), b.z, acc);
+                    acc = __builtin_fmaf(__uint_as_float(v[j].w & 0xffff0000u), b.w, acc);
+                } else {
+                    acc = __builtin_fmaf(__uint_as_float(v[j].x), a.x, acc);
+                    acc = __builtin_fmaf(__uint_as_float(v[j].y), a.y, acc);
+                    acc = __builtin_fmaf(__uint_as_float(v[j].z), a.z, acc);
+                    acc = __builtin_fmaf(__uint_as_float(v[j].w), a.w, acc);
+                }
             }
         }
     }
     for (int o = 32; o > 0; o >>= 1) acc += __shfl_down(acc, o);
-    if (lane == 0) y[(size_t)t * rows + row] = acc;
+    if (!block_per_row) {
+        if (lane == 0) y[(size_t)t * rows + row] = acc;
+        return;
+    }
+    if (lane == 0) wave_sum[wave] = acc;
+    __syncthreads();
+    if (threadIdx.x == 0) y[(size_t)t * rows + row] = ((wave_sum[0] + wave_sum[1]) + wave_sum[2]) + wave_sum[3];
 }
+#define CROW_KEEP_GEMV(NAME, WT, WBF16)                                                                                              \
+    extern "C" __global__ void __launch_bounds__(256) NAME(const WT* __restrict__ w, const float* __restrict__ x, float* __restrict__ y, \
+                                                           const int* __restrict__ k_dim_p, const int* __restrict__ rows_p) {        \
+        if (block_threads() != 256) {                                                                                                \
+            if (threadIdx.x == 0) atomicOr(g_ws.status, STATUS_BAD_SHAPE);                                                           \
+            return;                                                                                                                  \
+        }                                                                                                                            \
+        keep_gemv_body<WBF16>(w, x, y, *k_dim_p, *rows_p);                                                                           \
+    }
+CROW_KEEP_GEMV(gemv_bf16_w, unsigned short, true)
+CROW_KEEP_GEMV(gemv_bf16, unsigned short, true)
+CROW_KEEP_GEMV(gemv_bf16_b, unsigned short, true)
+CROW_KEEP_GEMV(gemv_b, float, false)

@@ -241,15 +241,27 @@ class Engine:
         return ids, wts, y
 
     # ------------------------------------------------------------------ BF16 keeps (router, q/k, MTP head)
-    def bf16_proj(self, w: torch.Tensor, t: int, x: torch.Tensor, y: torch.Tensor | None = None) -> torch.Tensor:
-        """y[t][rows] = bf16 W [rows][k] times f32 x [t][k]: ``gemv_bf16_w`` (engine/src/kernels.rs:1130-1157)."""
+    def bf16_proj(self, w: torch.Tensor, t: int, x: torch.Tensor, y: torch.Tensor | None = None, kernel: str = "gemv_bf16_w") -> torch.Tensor:
+        """y[t][rows] = bf16 W [rows][k] times f32 x [t][k]: ``gemv_bf16_w`` (engine/src/kernels.rs:1130-1157), or under the
+        names of the reference's block-per-row forms ``gemv_bf16`` (one token) / ``gemv_bf16_b`` (kernels.rs:1061-1098)."""
         assert w.is_cuda and w.dtype == torch.bfloat16 and w.dim() == 2 and w.is_contiguous()
+        assert kernel in ("gemv_bf16_w", "gemv_bf16", "gemv_bf16_b")
+        return self._keep_proj(kernel, w, t, x, y)
+
+    def f32_proj(self, w: torch.Tensor, t: int, x: torch.Tensor, y: torch.Tensor | None = None) -> torch.Tensor:
+        """y[t][rows] = f32 W [rows][k] times f32 x [t][k]: ``gemv_b``, the router projection (engine/src/gen.rs:4182,
+        kernels.rs:97-115); its result is router_top10's logits."""
+        assert w.is_cuda and w.dtype == torch.float32 and w.dim() == 2 and w.is_contiguous()
+        return self._keep_proj("gemv_b", w, t, x, y)
+
+    def _keep_proj(self, name: str, w: torch.Tensor, t: int, x: torch.Tensor, y: torch.Tensor | None, waves_per_row: int = 0) -> torch.Tensor:
+        """waves_per_row: 0 = the library's choice (a block of four waves per row for short tensors), 1 or 4 to force."""
         rows, k = w.shape
         assert x.is_cuda and x.dtype == torch.float32 and x.is_contiguous() and x.numel() == t * k
         if y is None:
             y = torch.empty((t, rows), dtype=torch.float32, device=self.dev)
         p = self.p
-        launch_v(self.k.f("gemv_bf16_w"), *launch_dims("gemv_bf16_w", rows, k, t), [w.data_ptr(), x.data_ptr(), y.data_ptr(), p.i32(k), p.i32(rows)])
+        launch_v(self.k.f(name), *launch_dims(name, rows, k, t, split=(0, waves_per_row)), [w.data_ptr(), x.data_ptr(), y.data_ptr(), p.i32(k), p.i32(rows)])
         return y
 
     # ------------------------------------------------------------------ prefill GEMM (M >= 16)

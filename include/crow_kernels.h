@@ -106,6 +106,14 @@ CROW_KERNEL(gemm_nvfp4_bf16_m16, 7)
 /* ---- BF16 weights the container keeps unquantised (router, MTP head) ---------------------------------------------- */
 /* w(bf16 [rows][k_dim]), x, y, k_dim_p, rows_p.  gemv_bf16_w of kernels.rs:1130-1157; tokens on grid.y. */
 CROW_KERNEL(gemv_bf16_w, 5)
+/* the block-per-row forms of the same product, gemv_bf16 (one token, kernels.rs:1061-1077: the bf16 lm_head of gen.rs:4780)
+ * and gemv_bf16_b (grid.y tokens, kernels.rs:1080-1098: the GLM5 router of glm5_moe.rs:731), + rows_p: the reference's
+ * grid.x is the row count.  Launched with the dims of gemv_bf16_w. */
+CROW_KERNEL(gemv_bf16, 5)
+CROW_KERNEL(gemv_bf16_b, 5)
+/* w(f32 [rows][k_dim]), x, y, k_dim_p, rows_p.  gemv_b of kernels.rs:97-115 (the router projection of gen.rs:4182), + rows_p;
+ * k_dim a multiple of 4; tokens on grid.y. */
+CROW_KERNEL(gemv_b, 5)
 
 /* ---- layout and decode ---------------------------------------------------------------------------------------------- */
 CROW_KERNEL(repack_nvfp4, 4)        /* src(container bytes), dst(tiled), rows_p, k_dim_p: what crow_hip_repack_nvfp4 launches */

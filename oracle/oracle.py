@@ -215,3 +215,35 @@ def gemv_bf16(w_bits, rows: int, cols: int, x) -> np.ndarray:
     xv = _f32(x).reshape(-1, cols).astype(np.float64)
     return (xv @ w.T).astype(np.float32)
 
+
+def gemv_f32w(w, rows: int, cols: int, x) -> np.ndarray:
+    """F32-weight GEMV of the reference (gemv_b, engine/src/kernels.rs:97-115: the router projection): y[t][r] =
+    sum_k w[r][k] * x[t][k].  As for gemv_bf16 the result is defined by the real-number sum: every f32 * f32 product is
+    exact in f64 (48 significant bits), the f64 sum of K <= 2^20 of them is rounded once to f32.  The reference's own
+    order (256 strided partial sums, then a halving tree) is one of the f32 orders the bound gamma(K) * sum |w x| covers."""
+    wv = _f32(w).reshape(rows, cols).astype(np.float64)
+    xv = _f32(x).reshape(-1, cols).astype(np.float64)
+    return (xv @ wv.T).astype(np.float32)
+
+
+def gemv_f32w_reference_order(w, rows: int, cols: int, x) -> np.ndarray:
+    """The same product in the order the reference's kernel uses (engine/src/kernels.rs:104-114): thread t of 256 adds
+    w[i] * x[i] for i = t, t + 256, ... in f32, each product and each add rounded on its own; then red[t] += red[t + st]
+    for st = 128, 64, ..., 1."""
+    wv = _f32(w).reshape(rows, cols)
+    xv = _f32(x).reshape(-1, cols)
+    out = np.zeros((xv.shape[0], rows), np.float32)
+    pad = (-cols) % 256
+    for t in range(xv.shape[0]):
+        prod = (wv * xv[t][None, :]).astype(np.float32)                      # one rounding per product
+        prod = np.pad(prod, ((0, 0), (0, pad))).reshape(rows, -1, 256)       # step j, thread t: column 256 j + t
+        red = np.zeros((rows, 256), np.float32)
+        for j in range(prod.shape[1]):
+            live = min(256, cols - 256 * j)                                  # threads beyond K add nothing on the last step
+            red[:, :live] = (red[:, :live] + prod[:, j, :live]).astype(np.float32)
+        st = 128
+        while st > 0:
+            red[:, :st] = (red[:, :st] + red[:, st:2 * st]).astype(np.float32)
+            st >>= 1
+        out[t] = red[:, 0]
+    return out

@@ -643,14 +643,53 @@ def test_bf16_keep_gemv(eng, rows, cols, t):
     w_bits = orc.f32_to_bf16_bits(w32).reshape(rows, cols)
     x = normal_f32(71, t, t * cols).reshape(t, cols)
     wd = torch.from_numpy(w_bits.view(np.int16)).cuda().view(torch.bfloat16)
-    y = eng.bf16_proj(wd, t, _dev(x)).cpu().numpy()
     ref = orc.gemv_bf16(w_bits, rows, cols, x)
-    assert rel_err(y, ref) <= TOL
     wf = orc.bf16_bits_to_f32(w_bits).astype(np.float64)
     bound = orc.gamma(16 * (cols + 6)) * (np.abs(x.astype(np.float64)) @ np.abs(wf).T)  # gamma(n) of the oracle counts n / 16 + 10 steps
-    assert np.all(np.abs(y.astype(np.float64) - ref.astype(np.float64)) <= bound + 1e-30)
+    xd = _dev(x)
+    for waves_per_row in (0, 1, 4):  # the library's choice, one wave per row, a block of four waves per row
+        y = eng._keep_proj("gemv_bf16_w", wd, t, xd, None, waves_per_row).cpu().numpy()
+        eng.check()
+        assert rel_err(y, ref) <= TOL, waves_per_row
+        assert np.all(np.abs(y.astype(np.float64) - ref.astype(np.float64)) <= bound + 1e-30), waves_per_row
+
+
+
+def test_bf16_keep_gemv_under_the_block_per_row_names(eng):
+    """gemv_bf16 (one token) and gemv_bf16_b are the same product under the reference's other two names: same bits."""
+    rows, cols, t = 300, 2560, 3
+    w_bits = orc.f32_to_bf16_bits(normal_f32(72, 1, rows * cols) * np.float32(0.05)).reshape(rows, cols)
+    x = normal_f32(73, t, t * cols).reshape(t, cols)
+    wd = torch.from_numpy(w_bits.view(np.int16)).cuda().view(torch.bfloat16)
+    y = eng.bf16_proj(wd, t, _dev(x)).cpu().numpy()
+    yb = eng.bf16_proj(wd, t, _dev(x), kernel="gemv_bf16_b").cpu().numpy()
+    y1 = eng.bf16_proj(wd, 1, _dev(x[1]), kernel="gemv_bf16").cpu().numpy()
+    assert np.array_equal(y.view(np.uint32), yb.view(np.uint32)) and np.array_equal(y1.view(np.uint32)[0], y.view(np.uint32)[1])
+    assert rel_err(y, orc.gemv_bf16(w_bits, rows, cols, x)) <= TOL
+    from crow_nest_amd.lib import CrowHipError
+    with pytest.raises(CrowHipError):  # the one-token name takes one token
+        eng.bf16_proj(wd, 2, _dev(x[:2]), kernel="gemv_bf16")
     eng.check()
 
+
+@pytest.mark.parametrize("rows,cols,t", [(256, 2560, 1), (256, 2560, 4), (37, 20, 3), (288, 4096, 2), (5, 4, 1), (1000, 1028, 1)])
+def test_f32_keep_gemv_router_projection(eng, rows, cols, t):
+    """gemv_b: f32 weights (the router), against the exact dot product within the f32 summation bound, and against the
+    reference's own summation order within the tolerance; then the logits feed the router."""
+    print(f"case rows={rows} cols={cols} t={t}", flush=True)
+    w = normal_f32(74, rows, rows * cols).reshape(rows, cols) * np.float32(0.05)
+    x = normal_f32(75, t, t * cols).reshape(t, cols)
+    ref = orc.gemv_f32w(w, rows, cols, x)
+    ref_order = orc.gemv_f32w_reference_order(w, rows, cols, x)
+    bound = orc.gamma(16 * (cols + 6)) * (np.abs(x.astype(np.float64)) @ np.abs(w.astype(np.float64)).T)
+    wd, xd = _dev(w), _dev(x)
+    for waves_per_row in (0, 1, 4):  # the library's choice, one wave per row, a block of four waves per row
+        y = eng._keep_proj("gemv_b", wd, t, xd, None, waves_per_row).cpu().numpy()
+        eng.check()
+        assert rel_err(y, ref) <= TOL, waves_per_row
+        assert rel_err(y, ref_order) <= TOL, waves_per_row
+        assert np.all(np.abs(y.astype(np.float64) - ref.astype(np.float64)) <= bound + 1e-30), waves_per_row
+    assert np.array_equal(eng.f32_proj(wd, t, xd).cpu().numpy(), eng._keep_proj("gemv_b", wd, t, xd, None, 0).cpu().numpy())
 
 
 # ---------------------------------------------------------------- the ABI from plain C

@@ -455,3 +455,44 @@ def test_bf16_keep_gemv_is_the_exact_rational_dot_product():
             exact = sum(Fraction(float(wf[r, k])) * Fraction(float(x[ti, k])) for k in range(cols))
             assert y[ti, r] == np.float32(float(exact)), (ti, r)
 
+
+def test_f32_keep_gemv_is_the_exact_rational_dot_product_and_the_reference_order_agrees():
+    """gemv_f32w's f64 evaluation against exact rational arithmetic on small inputs; the restatement of the reference's
+    own order (256 strided partial sums, halving tree) against a plain loop written from kernels.rs:104-114, and within
+    the f32 summation bound of the exact value."""
+    from fractions import Fraction
+    rng = np.random.default_rng(6)
+    rows, cols, t = 4, 28, 2
+    w = rng.standard_normal((rows, cols)).astype(np.float32)
+    x = rng.standard_normal((t, cols)).astype(np.float32)
+    y = orc.gemv_f32w(w, rows, cols, x)
+    for ti in range(t):
+        for r in range(rows):
+            exact = sum(Fraction(float(w[r, k])) * Fraction(float(x[ti, k])) for k in range(cols))
+            assert y[ti, r] == np.float32(float(exact)), (ti, r)
+    # the reference's order, scalar loop: K = 600 leaves threads 88..255 with two terms and the rest with three
+    rows, cols = 3, 600
+    w = rng.standard_normal((rows, cols)).astype(np.float32)
+    x = rng.standard_normal((1, cols)).astype(np.float32)
+    got = orc.gemv_f32w_reference_order(w, rows, cols, x)
+    for r in range(rows):
+        red = [np.float32(0.0)] * 256
+        for th in range(256):
+            acc = np.float32(0.0)
+            for i in range(th, cols, 256):
+                acc = np.float32(acc + np.float32(w[r, i] * x[0, i]))
+            red[th] = acc
+        st = 128
+        while st > 0:
+            for th in range(st):
+                red[th] = np.float32(red[th] + red[th + st])
+            st >>= 1
+        assert got[0, r] == red[0], r
+    exact = orc.gemv_f32w(w, rows, cols, x).astype(np.float64)
+    bound = orc.gamma(16 * (cols + 6)) * (np.abs(x.astype(np.float64)) @ np.abs(w.astype(np.float64)).T)
+    assert np.all(np.abs(got.astype(np.float64) - exact) <= bound)
+    # integers: every order gives the same exact sum
+    wi = rng.integers(-8, 9, size=(5, 512)).astype(np.float32)
+    xi = rng.integers(-8, 9, size=(2, 512)).astype(np.float32)
+    assert np.array_equal(orc.gemv_f32w(wi, 5, 512, xi), orc.gemv_f32w_reference_order(wi, 5, 512, xi))
+    assert np.array_equal(orc.gemv_f32w(wi, 5, 512, xi), (xi.astype(np.int64) @ wi.astype(np.int64).T).astype(np.float32))
