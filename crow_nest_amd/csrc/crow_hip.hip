@@ -40,7 +40,7 @@ const FnEntry g_table[] = {
     {"gemm_nvfp4_bf16_m48", (const void*)&gemm_nvfp4_bf16_m48, 7, 2u * 48u * 528u, 0u},
     {"gemm_nvfp4_bf16_m96", (const void*)&gemm_nvfp4_bf16_m96, 7, 2u * 96u * 528u, 0u},
     CROW_FN(gemm_nvfp4_bf16_m32, 7), CROW_FN(gemm_nvfp4_bf16_m16, 7), CROW_FN(gemv_bf16_w, 5),
-    CROW_FN(gemv_bf16, 5), CROW_FN(gemv_bf16_b, 5), CROW_FN(gemv_b, 5),
+    CROW_FN(gemv_bf16, 5), CROW_FN(gemv_bf16_b, 5), CROW_FN(gemv_b, 5), CROW_FN(gemv_bf16_ws, 5), CROW_FN(gemv_bf16_bs, 6),
 };
 const int g_table_n = (int)(sizeof(g_table) / sizeof(g_table[0]));
 
@@ -263,7 +263,8 @@ int crow_hip_launch_dims_split(const char* name, uint32_t rows, uint32_t k_dim, 
     if (!e) return CROW_ERR_KERNEL_MISSING;
     const uint32_t rt = (rows + CROW_TILE_ROWS - 1) / CROW_TILE_ROWS;
     const uint32_t panels = (k_dim + CROW_PANEL_COLS - 1) / CROW_PANEL_COLS;
-    if (strcmp(name, "gemv_bf16_w") == 0 || strcmp(name, "gemv_bf16") == 0 || strcmp(name, "gemv_bf16_b") == 0 || strcmp(name, "gemv_b") == 0) {
+    if (strcmp(name, "gemv_bf16_w") == 0 || strcmp(name, "gemv_bf16") == 0 || strcmp(name, "gemv_bf16_b") == 0 || strcmp(name, "gemv_b") == 0 ||
+        strcmp(name, "gemv_bf16_ws") == 0 || strcmp(name, "gemv_bf16_bs") == 0) {
         // z = T activation rows; whole 16-byte loads: 8 bf16 or 4 f32 weights
         if (k_dim == 0 || k_dim % (strcmp(name, "gemv_b") == 0 ? 4 : 8) != 0) return CROW_ERR_SHAPE;
         if (strcmp(name, "gemv_bf16") == 0 && z != 1) return CROW_ERR_SHAPE;  // the one-token form

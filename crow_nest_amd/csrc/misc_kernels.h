@@ -518,8 +518,11 @@ extern "C" __global__ void __launch_bounds__(256) argmax_tiles(int* __restrict__
 //   gemv_bf16     engine/src/kernels.rs:1061-1077 (block per row, one token; + rows_p: the reference's grid.x is the row count)
 //   gemv_bf16_b   engine/src/kernels.rs:1080-1098 (block per row, grid.y tokens; + rows_p)
 //   gemv_b        engine/src/kernels.rs:97-115   (f32 weights, the router projection of gen.rs:4182; + rows_p; k_dim % 4 == 0)
-template <bool WBF16>
-__device__ __forceinline__ void keep_gemv_body(const void* __restrict__ w, const float* __restrict__ x, float* __restrict__ y, int k, int rows) {
+//   gemv_bf16_ws  engine/src/kernels.rs:1430-1458 (gemv_bf16_w with y = 1 / (1 + expf(-sum)) at the store)
+//   gemv_bf16_bs  engine/src/kernels.rs:1100-1124 (gemv_bf16_b with an explicit y row stride; + rows_p)
+template <bool WBF16, bool SIGMOID = false>
+__device__ __forceinline__ void keep_gemv_body(const void* __restrict__ w, const float* __restrict__ x, float* __restrict__ y, int k, int rows,
+                                               size_t y_stride) {
     constexpr int PER = WBF16 ? 8 : 4;  // weights per 16-byte load
     __shared__ float wave_sum[4];
     const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6)), lane = lane_id();
@@ -564,13 +567,14 @@ __device__ __forceinline__ void keep_gemv_body(const void* __restrict__ w, const
         }
     }
     for (int o = 32; o > 0; o >>= 1) acc += __shfl_down(acc, o);
+    auto finish = [](float v) { return SIGMOID ? 1.0f / (1.0f + expf(-v)) : v; };
     if (!block_per_row) {
-        if (lane == 0) y[(size_t)t * rows + row] = acc;
+        if (lane == 0) y[(size_t)t * y_stride + row] = finish(acc);
         return;
     }
     if (lane == 0) wave_sum[wave] = acc;
     __syncthreads();
-    if (threadIdx.x == 0) y[(size_t)t * rows + row] = ((wave_sum[0] + wave_sum[1]) + wave_sum[2]) + wave_sum[3];
+    if (threadIdx.x == 0) y[(size_t)t * y_stride + row] = finish(((wave_sum[0] + wave_sum[1]) + wave_sum[2]) + wave_sum[3]);
 }
 #define CROW_KEEP_GEMV(NAME, WT, WBF16)                                                                                              \
     extern "C" __global__ void __launch_bounds__(256) NAME(const WT* __restrict__ w, const float* __restrict__ x, float* __restrict__ y, \
@@ -579,9 +583,27 @@ __device__ __forceinline__ void keep_gemv_body(const void* __restrict__ w, const
             if (threadIdx.x == 0) atomicOr(g_ws.status, STATUS_BAD_SHAPE);                                                           \
             return;                                                                                                                  \
         }                                                                                                                            \
-        keep_gemv_body<WBF16>(w, x, y, *k_dim_p, *rows_p);                                                                           \
+        keep_gemv_body<WBF16>(w, x, y, *k_dim_p, *rows_p, (size_t)*rows_p);                                                          \
     }
 CROW_KEEP_GEMV(gemv_bf16_w, unsigned short, true)
 CROW_KEEP_GEMV(gemv_bf16, unsigned short, true)
 CROW_KEEP_GEMV(gemv_bf16_b, unsigned short, true)
 CROW_KEEP_GEMV(gemv_b, float, false)
+
+extern "C" __global__ void __launch_bounds__(256) gemv_bf16_ws(const unsigned short* __restrict__ w, const float* __restrict__ x, float* __restrict__ y,
+                                                               const int* __restrict__ k_dim_p, const int* __restrict__ rows_p) {
+    if (block_threads() != 256) {
+        if (threadIdx.x == 0) atomicOr(g_ws.status, STATUS_BAD_SHAPE);
+        return;
+    }
+    keep_gemv_body<true, true>(w, x, y, *k_dim_p, *rows_p, (size_t)*rows_p);
+}
+extern "C" __global__ void __launch_bounds__(256) gemv_bf16_bs(const unsigned short* __restrict__ w, const float* __restrict__ x, float* __restrict__ y,
+                                                               const int* __restrict__ k_dim_p, const int* __restrict__ y_stride_p,
+                                                               const int* __restrict__ rows_p) {
+    if (block_threads() != 256 || *y_stride_p < *rows_p) {
+        if (threadIdx.x == 0) atomicOr(g_ws.status, STATUS_BAD_SHAPE);
+        return;
+    }
+    keep_gemv_body<true>(w, x, y, *k_dim_p, *rows_p, (size_t)*y_stride_p);
+}

@@ -245,8 +245,19 @@ class Engine:
         """y[t][rows] = bf16 W [rows][k] times f32 x [t][k]: ``gemv_bf16_w`` (engine/src/kernels.rs:1130-1157), or under the
         names of the reference's block-per-row forms ``gemv_bf16`` (one token) / ``gemv_bf16_b`` (kernels.rs:1061-1098)."""
         assert w.is_cuda and w.dtype == torch.bfloat16 and w.dim() == 2 and w.is_contiguous()
-        assert kernel in ("gemv_bf16_w", "gemv_bf16", "gemv_bf16_b")
+        assert kernel in ("gemv_bf16_w", "gemv_bf16", "gemv_bf16_b", "gemv_bf16_ws")  # _ws: sigmoid at the store (kernels.rs:1430-1458)
         return self._keep_proj(kernel, w, t, x, y)
+
+    def bf16_proj_strided(self, w: torch.Tensor, t: int, x: torch.Tensor, y: torch.Tensor, y_stride: int) -> torch.Tensor:
+        """``gemv_bf16_bs`` (kernels.rs:1100-1124): row r of token i lands in y.flatten()[i * y_stride + r] - y may be a view
+        that starts inside a wider [t][y_stride] buffer (the shared expert's gate | up pair)."""
+        assert w.is_cuda and w.dtype == torch.bfloat16 and w.dim() == 2 and w.is_contiguous()
+        rows, k = w.shape
+        assert x.is_cuda and x.dtype == torch.float32 and x.is_contiguous() and x.numel() == t * k and y.is_cuda and y.dtype == torch.float32
+        p = self.p
+        launch_v(self.k.f("gemv_bf16_bs"), *launch_dims("gemv_bf16_bs", rows, k, t),
+                 [w.data_ptr(), x.data_ptr(), y.data_ptr(), p.i32(k), p.i32(y_stride), p.i32(rows)])
+        return y
 
     def f32_proj(self, w: torch.Tensor, t: int, x: torch.Tensor, y: torch.Tensor | None = None) -> torch.Tensor:
         """y[t][rows] = f32 W [rows][k] times f32 x [t][k]: ``gemv_b``, the router projection (engine/src/gen.rs:4182,

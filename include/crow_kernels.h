@@ -114,6 +114,11 @@ CROW_KERNEL(gemv_bf16_b, 5)
 /* w(f32 [rows][k_dim]), x, y, k_dim_p, rows_p.  gemv_b of kernels.rs:97-115 (the router projection of gen.rs:4182), + rows_p;
  * k_dim a multiple of 4; tokens on grid.y. */
 CROW_KERNEL(gemv_b, 5)
+/* w(bf16), x, y, k_dim_p, rows_p.  gemv_bf16_ws of kernels.rs:1430-1458: gemv_bf16_w with the sigmoid applied at the store. */
+CROW_KERNEL(gemv_bf16_ws, 5)
+/* w(bf16), x, y, k_dim_p, y_stride_p, rows_p.  gemv_bf16_bs of kernels.rs:1100-1124: gemv_bf16_b writing y[t * *y_stride_p + row]
+ * (two tensors into one [t][stride] buffer), + rows_p. */
+CROW_KERNEL(gemv_bf16_bs, 6)
 
 /* ---- layout and decode ---------------------------------------------------------------------------------------------- */
 CROW_KERNEL(repack_nvfp4, 4)        /* src(container bytes), dst(tiled), rows_p, k_dim_p: what crow_hip_repack_nvfp4 launches */

@@ -669,6 +669,16 @@ def test_bf16_keep_gemv_under_the_block_per_row_names(eng):
     from crow_nest_amd.lib import CrowHipError
     with pytest.raises(CrowHipError):  # the one-token name takes one token
         eng.bf16_proj(wd, 2, _dev(x[:2]), kernel="gemv_bf16")
+    # gemv_bf16_ws: the sigmoid at the store; gemv_bf16_bs: two tensors into one [t][2 rows] buffer
+    ys = eng.bf16_proj(wd, t, _dev(x), kernel="gemv_bf16_ws").cpu().numpy()
+    want = (np.float32(1.0) / (np.float32(1.0) + np.exp(-y, dtype=np.float32))).astype(np.float32)
+    assert np.max(np.abs(ys - want)) <= 2e-7  # expf in the last place; the sums are the plain kernel's
+    both = torch.full((t, 2 * rows + 8), 7.0, dtype=torch.float32, device="cuda")
+    eng.bf16_proj_strided(wd, t, _dev(x), both, 2 * rows + 8)
+    eng.bf16_proj_strided(wd, t, _dev(x), both.view(-1)[rows:], 2 * rows + 8)
+    got = both.cpu().numpy()
+    assert np.array_equal(got[:, :rows].view(np.uint32), y.view(np.uint32)) and np.array_equal(got[:, rows:2 * rows].view(np.uint32), y.view(np.uint32))
+    assert bool((got[:, 2 * rows:] == 7.0).all())
     eng.check()
 
 
