@@ -213,6 +213,8 @@ int crow_hip_function_arg_count(crow_fn_t f) {
 int crow_hip_set_geo(int experts, int topk, int hidden, int inter) {
     if (!g.ready) return CROW_ERR_NOT_INITIALIZED;
     if (experts < 0 || topk < 0 || hidden < 0 || inter < 0) return CROW_ERR_BAD_ARGUMENT;
+    // what the routing kernels take: no routed experts at all, or a power of two of them in 64..1024 with 1..16 picks
+    if (experts != 0 && (experts < 64 || experts > 1024 || (experts & (experts - 1)) != 0 || topk < 1 || topk > 16)) return CROW_ERR_GEO;
     crow::Geo geo{experts, topk, hidden, inter};
     hipError_t e = hipMemcpyToSymbolAsync(HIP_SYMBOL(crow::g_geo), &geo, sizeof geo, 0, hipMemcpyHostToDevice, g.stream);
     if (e != hipSuccess) return (int)e;

@@ -182,6 +182,10 @@ extern "C" __global__ void __launch_bounds__(1024) gemv_fp4_ptrb(const unsigned 
     ENTER(ptrs, x, gs_ptr, y, k_dim_p, x_div_p, x_stride_p, rows_p);
     const int combo = (int)blockIdx.z, rows = *rows_p;
     const unsigned char* w = (const unsigned char*)ptrs[combo];
+    if (w == nullptr) {  // a router launch that refused its geometry leaves the pointer table untouched (zeros): refuse too
+        if (threadIdx.x == 0) atomicOr(ws.status, STATUS_BAD_GEO);
+        return;
+    }
     GemvArgs a{{w, nullptr}, {gs_ptr, nullptr}, x + (size_t)(combo / *x_div_p) * *x_stride_p, 0, y + (size_t)combo * rows, 0, *k_dim_p, rows, 1, nullptr};
     gemv_body<1, 1, false, EPI_SCALE, XRows<1, false>::value>(a, blockIdx.z, LDS, ws);
 }
@@ -195,6 +199,10 @@ extern "C" __global__ void __launch_bounds__(1024) moe_gate_up_silu(const unsign
     ENTER(ptrs, x, gs_ptr, h, k_dim_p, x_div_p, x_stride_p, inter_p);
     const int combo = (int)blockIdx.z, inter = *inter_p, k = *k_dim_p;
     const unsigned char* w = (const unsigned char*)ptrs[combo];
+    if (w == nullptr) {  // see gemv_fp4_ptrb
+        if (threadIdx.x == 0) atomicOr(ws.status, STATUS_BAD_GEO);
+        return;
+    }
     const size_t up_off = (size_t)(inter / CROW_TILE_ROWS) * ((k + CROW_PANEL_COLS - 1) / CROW_PANEL_COLS) * CROW_TILE_BYTES;
     GemvArgs a{{w, w + up_off}, {gs_ptr, gs_ptr}, x + (size_t)(combo / *x_div_p) * *x_stride_p, 0, h + (size_t)combo * inter, 0, k, inter, 1, nullptr};
     gemv_body<2, 1, false, EPI_SILU_GU, XRows<1, false>::value, true>(a, blockIdx.z, LDS, ws);
@@ -222,9 +230,13 @@ extern "C" __global__ void __launch_bounds__(1024) moe_down_combine(const unsign
     if (threadIdx.x < CROW_GEMV_ZERO_BYTES / 16) lds_store16(zero + 16 * threadIdx.x, 0, 0, 0, 0);
     __syncthreads();
     const unsigned char* const w[2] = {(const unsigned char*)ptrs[combo], nullptr};
-    float acc[1][1];
+    float acc[1][1] = {{0.0f}};
     const size_t xoff[1] = {0};
-    tile_accumulate<1, 1, false>(w, rt, (k + CROW_PANEL_COLS - 1) / CROW_PANEL_COLS, 0, 1, k, h + (size_t)combo * k, xoff, 1, xw, zero, acc);
+    if (w[0] != nullptr) {
+        tile_accumulate<1, 1, false>(w, rt, (k + CROW_PANEL_COLS - 1) / CROW_PANEL_COLS, 0, 1, k, h + (size_t)combo * k, xoff, 1, xw, zero, acc);
+    } else if (lane == 0) {  // a routing launch that refused its geometry left zeros behind: no weights to read; the wave
+        atomicOr(g_ws.status, STATUS_BAD_GEO);  // still joins the barrier below
+    }
     ((lds_f)xw)[lane] = rw[combo] * (acc[0][0] * gs_ptr[0]);
     __syncthreads();
     const int row = rt * CROW_TILE_ROWS + lane;

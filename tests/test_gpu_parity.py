@@ -616,6 +616,43 @@ def test_launches_with_a_wrong_block_shape_are_refused(eng):
     eng.check()
 
 
+def test_an_unsupported_geometry_is_refused_and_an_empty_pointer_table_is_not_followed(eng):
+    """crow_hip_set_geo refuses an expert count the routing kernels do not take (on the host, nothing launched); and the
+    routed kernels, handed a pointer table a refused routing launch would have left as zeros, report through the status
+    word instead of reading weights at address zero."""
+    from crow_nest_amd.kernels import KernelGeo, launch_dims, launch_v, set_geo
+    from crow_nest_amd.lib import CrowHipError
+    for bad in (KernelGeo(16, 4, 512, 256), KernelGeo(96, 4, 512, 256), KernelGeo(2048, 8, 512, 256), KernelGeo(256, 17, 512, 256), KernelGeo(64, 0, 512, 256)):
+        with pytest.raises(CrowHipError) as ei:
+            set_geo(bad)
+        assert ei.value.code == -8  # CROW_ERR_GEO
+    set_geo(eng.geo)
+    H, I, K = eng.geo.hidden, eng.geo.inter, eng.geo.topk
+    p = eng.p
+    gs = torch.tensor([1e-3], dtype=torch.float32, device="cuda")
+    zeros = torch.zeros(K, dtype=torch.int64, device="cuda")
+    x = torch.zeros(H, dtype=torch.float32, device="cuda")
+    h2 = torch.full((K, I), 7.0, dtype=torch.float32, device="cuda")
+    y = torch.full((1, H), 7.0, dtype=torch.float32, device="cuda")
+    wts = torch.ones(K, dtype=torch.float32, device="cuda")
+    launch_v(eng.k.f("moe_gate_up_silu"), *launch_dims("moe_gate_up_silu", I, H, K),
+             [zeros.data_ptr(), x.data_ptr(), gs.data_ptr(), h2.data_ptr(), p.i32(H), p.i32(K), p.i32(H), p.i32(I)])
+    with pytest.raises(CrowHipError) as ei:
+        eng.check()
+    assert ei.value.code == -8 and float(h2.min()) == 7.0 == float(h2.max())
+    launch_v(eng.k.f("gemv_fp4_ptrb"), *launch_dims("gemv_fp4_ptrb", 2 * I, H, K),
+             [zeros.data_ptr(), x.data_ptr(), gs.data_ptr(), torch.empty((K, 2 * I), device="cuda").data_ptr(), p.i32(H), p.i32(K), p.i32(H), p.i32(2 * I)])
+    with pytest.raises(CrowHipError) as ei:
+        eng.check()
+    assert ei.value.code == -8
+    launch_v(eng.k.f("moe_down_combine"), *launch_dims("moe_down_combine", H, I, 1),
+             [zeros.data_ptr(), h2.data_ptr(), gs.data_ptr(), wts.data_ptr(), y.data_ptr(), p.i32(I), p.i32(H)])
+    with pytest.raises(CrowHipError) as ei:
+        eng.check()
+    assert ei.value.code == -8 and float(y.min()) == 7.0 == float(y.max())  # y += 0 from every combo
+    eng.check()
+
+
 def test_verify_kernels_refuse_more_than_four_rows(eng):
     """The reference's verify kernels take at most NVFP4_MMAX = 4 rows (kernels_p2.rs:397-400); a launch with m = 5 writes
     nothing and reports a shape error through the status word instead of computing four rows silently."""
