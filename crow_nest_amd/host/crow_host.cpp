@@ -247,9 +247,57 @@ void Engine::moe_run(const MoeW& moe, int t, uint64_t x, uint64_t logits, uint64
     launch_v(k.f("moe_down_combine"), launch_dims("moe_down_combine", (uint32_t)hdim, (uint32_t)inter, (uint32_t)t),
              {dn_ptrs, h2, moe.down.gs.ptr(), wts, y, p.i32(inter), p.i32(hdim)});
 }
+void Engine::moe_run_grouped(const MoeW& moe, int t, uint64_t x, uint64_t logits, uint64_t ids, uint64_t wts, uint64_t y, uint64_t h2, uint64_t eo,
+                             uint64_t gu_ptrs, uint64_t dn_ptrs, uint64_t perm, uint64_t tiles, uint64_t n_tiles) {
+    const int hdim = geo.hidden, inter = geo.inter, topk = geo.topk;
+    if (moe.gate_up.rows != 2 * inter || moe.gate_up.cols != hdim || moe.down.rows != hdim || moe.down.cols != inter || moe.gate_up.experts != geo.experts)
+        throw Panic("moe_run_grouped: the expert tensors do not match the geometry");
+    const int combos = t * topk, max_tiles = moe_max_tiles(combos, geo.experts);
+    launch_v(k.f("router_top10"), launch_dims("router_top10", 1, 64, (uint32_t)t), {logits, 0, ids, wts, gu_ptrs, dn_ptrs, moe.table.ptr(), 0, 0, 0});
+    launch_v(k.f("moe_group"), launch_dims("moe_group", 1, 64, (uint32_t)combos), {ids, p.i32(combos), perm, tiles, n_tiles, p.i32(max_tiles)});
+    launch_v(k.f("moe_gate_up_silu_grouped"), launch_dims("moe_gate_up_silu_grouped", (uint32_t)inter, (uint32_t)hdim, (uint32_t)max_tiles),
+             {tiles, n_tiles, perm, moe.table.ptr(), x, moe.gate_up.gs.ptr(), h2, p.i32(hdim), p.i32(topk), p.i32(hdim), p.i32(inter)});
+    launch_v(k.f("moe_down_grouped"), launch_dims("moe_down_grouped", (uint32_t)hdim, (uint32_t)inter, (uint32_t)max_tiles),
+             {tiles, n_tiles, perm, moe.table.ptr(), h2, moe.down.gs.ptr(), eo, p.i32(inter), p.i32(hdim)});
+    launch_v(k.f("acc_combo"), launch_dims("acc_combo", (uint32_t)hdim, 1, (uint32_t)t), {eo, wts, y});
+}
+void Engine::bf16_proj(uint64_t w_bf16, int rows, int kd, int t, uint64_t x, uint64_t y) {
+    launch_v(k.f("gemv_bf16_w"), launch_dims("gemv_bf16_w", (uint32_t)rows, (uint32_t)kd, (uint32_t)t), {w_bf16, x, y, p.i32(kd), p.i32(rows)});
+}
+void Engine::f32_proj(uint64_t w_f32, int rows, int kd, int t, uint64_t x, uint64_t y) {
+    launch_v(k.f("gemv_b"), launch_dims("gemv_b", (uint32_t)rows, (uint32_t)kd, (uint32_t)t), {w_f32, x, y, p.i32(kd), p.i32(rows)});
+}
 void Engine::gemm(const Fp4& w, int m, uint64_t x_bf16, uint64_t y) {
     const char* name = crow_hip_gemm_kernel((uint32_t)w.rows, (uint32_t)m);
     launch_v(k.f(name), launch_dims(name, (uint32_t)w.rows, (uint32_t)w.cols, (uint32_t)m), {w.w.ptr(), x_bf16, w.gs.ptr(), y, p.i32(w.cols), p.i32(w.rows), p.i32(m)});
+}
+
+// ---------------------------------------------------------------- graph capture
+Graph::Graph() {
+    ensure_init();
+    ck(crow_hip_stream_create(&stream_), "crow_hip_stream_create");
+}
+Graph::~Graph() {
+    if (exec_) (void)crow_hip_graph_exec_destroy(exec_);
+    if (crow_hip_cur_stream() == stream_) crow_hip_set_stream(nullptr);
+    if (stream_) (void)crow_hip_stream_destroy(stream_);
+}
+void Graph::begin() {
+    prev_ = crow_hip_cur_stream();
+    ck(crow_hip_begin_capture(stream_), "crow_hip_begin_capture");
+}
+void Graph::end() {
+    const int rc = crow_hip_end_capture_instantiate(stream_, &exec_);
+    crow_hip_set_stream(prev_);  // launches after the capture go where they went before it
+    ck(rc, "crow_hip_end_capture_instantiate");
+}
+void Graph::launch() { ck(crow_hip_launch_graph(exec_, stream_), "crow_hip_launch_graph"); }
+void Graph::sync() {  // the graph runs on its own non-blocking stream
+    void* cur = crow_hip_cur_stream();
+    crow_hip_set_stream(stream_);
+    const int rc = crow_hip_sync();
+    crow_hip_set_stream(cur);
+    ck(rc, "sync");
 }
 
 // ---------------------------------------------------------------- sha256 (FIPS 180-4), for the index checks of the container

@@ -167,8 +167,18 @@ class Engine {
     // h2 is scratch [t K][I], dn_ptrs scratch u64 [t][K].  Up to 4 tokens the router runs inside the gate|up launch.
     void moe_run(const MoeW& moe, int t, uint64_t x, uint64_t logits, uint64_t ids, uint64_t wts, uint64_t y, uint64_t h2, uint64_t gu_ptrs,
                  uint64_t dn_ptrs);
+    // the same for a batch in which experts repeat (the prefill path's idea, kernels.rs:3322-3384): router_top10, moe_group
+    // (combos sorted by expert, tiles of at most four), every tile's slab multiplied once by its rows, acc_combo.
+    // eo is scratch [t K][H], perm i32 [t K], tiles i32 [max_tiles][4], n_tiles i32 [1]; max_tiles = min(t K, E) + t K / 4
+    void moe_run_grouped(const MoeW& moe, int t, uint64_t x, uint64_t logits, uint64_t ids, uint64_t wts, uint64_t y, uint64_t h2, uint64_t eo,
+                         uint64_t gu_ptrs, uint64_t dn_ptrs, uint64_t perm, uint64_t tiles, uint64_t n_tiles);
+    static int moe_max_tiles(int combos, int experts) { return (combos < experts ? combos : experts) + combos / 4; }
     // prefill projection: Y[m][rows] = X[m][cols] W^T on the matrix cores, bf16 X
     void gemm(const Fp4& w, int m, uint64_t x_bf16, uint64_t y);
+    // the unquantised keeps: y[t][rows] = W[rows][k] x[t][k], f32 x; W bf16 (gemv_bf16_w, kernels.rs:1130-1157) or f32
+    // (gemv_b, kernels.rs:97-115: the router projection)
+    void bf16_proj(uint64_t w_bf16, int rows, int k, int t, uint64_t x, uint64_t y);
+    void f32_proj(uint64_t w_f32, int rows, int k, int t, uint64_t x, uint64_t y);
     void check() { status(); }
     Kernels k;
     Params p;
@@ -176,6 +186,25 @@ class Engine {
 
   private:
     Engine(Module m, const KernelGeo* geo);
+};
+
+// A captured launch sequence (the reference's CROW_GRAPH path, cuda.rs:113-203): begin() makes the graph's own
+// non-blocking stream the current stream and starts capture, launch_v records, end() instantiates, launch() replays.
+class Graph {
+  public:
+    Graph();
+    ~Graph();
+    Graph(const Graph&) = delete;
+    Graph& operator=(const Graph&) = delete;
+    void begin();
+    void end();
+    void launch();
+    void sync();
+
+  private:
+    void* stream_ = nullptr;
+    void* exec_ = nullptr;
+    void* prev_ = nullptr;
 };
 
 // ---------------------------------------------------------------- CNQ1 container reader

@@ -7,10 +7,13 @@
 //   cnq-list <file>             the container's table, one line per tensor (no GPU needed)
 //   cnq-refuse <file>           prints the text open_checked refuses the file with (no GPU needed)
 //   cnq-dequant <file> <dir>    every 2-D NVFP4 tensor: load_fp4(cnq, name, sec), dequantise, write <dir>/<index>.f32
-//   dense <dir>                 meta: H I R T xbf16; dense_ffn_w (T <= 4) -> h.bin, y.bin; dense_proj(gate) on f32 x -> gate_y.bin
+//   dense <dir>                 meta: H I R T xbf16; dense_ffn_w (T <= 4) -> h.bin, y.bin; dense_proj(gate) on f32 x -> gate_y.bin;
+//                               T = 1, f32 x: the step captured in a Graph and replayed -> y_graph.bin
 //   head <dir>                  meta: V K; lm_head_row -> logits.bin, prints the token
 //   moe <dir>                   meta: E topk H I T; moe_run -> ids.bin, wts.bin, y.bin
 //   gemm <dir>                  meta: rows cols M; Engine::gemm -> y.bin
+//   moe-grouped <dir>           meta as moe; moe_run_grouped -> ids.bin, wts.bin, y.bin
+//   keeps <dir>                 meta: rows k t; bf16_proj, f32_proj -> y_bf16.bin, y_f32.bin
 //   panics                      Kernels::f on an unknown name, proj_m outside 1..=4 -> prints the texts
 #include <cstdio>
 #include <cstdlib>
@@ -110,6 +113,21 @@ static int dense(const std::string& dir) {
         from_dev(h, dir + "/h.bin");
         from_dev(y, dir + "/y.bin");
     }
+    if (T == 1 && !xbf16) {  // the same step captured once and replayed (the reference's CROW_GRAPH path): same bits as the eager launches
+        DevBuf hg((size_t)I * 4), yg((size_t)R * 4);
+        eng.dense_ffn_w(mlp, x.ptr(), 1, hg.ptr(), yg.ptr());  // eager once more: every Params word exists before the capture
+        sync();
+        Graph g;
+        g.begin();
+        eng.dense_ffn_w(mlp, x.ptr(), 1, hg.ptr(), yg.ptr());
+        g.end();
+        for (int rep = 0; rep < 3; rep++) {
+            g.launch();
+            g.sync();
+        }
+        eng.check();
+        from_dev(yg, dir + "/y_graph.bin");
+    }
     if (!xbf16) {  // dense_proj alone on the same rows, through its own dispatch (t == 1, 2..4, more)
         DevBuf y2((size_t)T * I * 4);
         eng.dense_proj(mlp.gate, T, x.ptr(), y2.ptr());
@@ -150,6 +168,41 @@ static int moe(const std::string& dir) {
     from_dev(ids, dir + "/ids.bin");
     from_dev(wts, dir + "/wts.bin");
     from_dev(y, dir + "/y.bin");
+    return 0;
+}
+
+static int moe_grouped(const std::string& dir) {
+    const std::vector<long> m = meta(dir);
+    const int E = (int)m.at(0), K = (int)m.at(1), H = (int)m.at(2), I = (int)m.at(3), T = (int)m.at(4);
+    const std::vector<uint8_t> gsb = slurp(dir + "/gs.bin");
+    const float* gs = (const float*)gsb.data();
+    const KernelGeo geo{E, K, H, I};
+    Engine eng(&geo);
+    const std::vector<uint8_t> gu = slurp(dir + "/gu.bin"), dn = slurp(dir + "/dn.bin");
+    const MoeW w = make_moe(load_expert_slabs(gu.data(), gu.size(), E, 2 * I, H, gs[0]), load_expert_slabs(dn.data(), dn.size(), E, H, I, gs[1]));
+    DevBuf x = to_dev(slurp(dir + "/x.bin")), logits = to_dev(slurp(dir + "/logits.bin"));
+    const int combos = T * K, max_tiles = Engine::moe_max_tiles(combos, E);
+    DevBuf ids((size_t)combos * 4), wts((size_t)combos * 4), y((size_t)T * H * 4), h2((size_t)combos * I * 4), eo((size_t)combos * H * 4), gup((size_t)combos * 8),
+        dnp((size_t)combos * 8), perm((size_t)combos * 4), tiles((size_t)max_tiles * 16), ntl(4);
+    eng.moe_run_grouped(w, T, x.ptr(), logits.ptr(), ids.ptr(), wts.ptr(), y.ptr(), h2.ptr(), eo.ptr(), gup.ptr(), dnp.ptr(), perm.ptr(), tiles.ptr(), ntl.ptr());
+    eng.check();
+    from_dev(ids, dir + "/ids.bin");
+    from_dev(wts, dir + "/wts.bin");
+    from_dev(y, dir + "/y.bin");
+    return 0;
+}
+
+static int keeps(const std::string& dir) {  // meta: rows k t; w_bf16.bin (u16), w_f32.bin, x.bin -> y_bf16.bin, y_f32.bin
+    const std::vector<long> m = meta(dir);
+    const int rows = (int)m.at(0), k = (int)m.at(1), t = (int)m.at(2);
+    Engine eng;
+    DevBuf wb = to_dev(slurp(dir + "/w_bf16.bin")), wf = to_dev(slurp(dir + "/w_f32.bin")), x = to_dev(slurp(dir + "/x.bin"));
+    DevBuf yb((size_t)t * rows * 4), yf((size_t)t * rows * 4);
+    eng.bf16_proj(wb.ptr(), rows, k, t, x.ptr(), yb.ptr());
+    eng.f32_proj(wf.ptr(), rows, k, t, x.ptr(), yf.ptr());
+    eng.check();
+    from_dev(yb, dir + "/y_bf16.bin");
+    from_dev(yf, dir + "/y_f32.bin");
     return 0;
 }
 
@@ -220,6 +273,8 @@ int main(int argc, char** argv) {
         if (cmd == "head" && argc == 3) return head(argv[2]);
         if (cmd == "moe" && argc == 3) return moe(argv[2]);
         if (cmd == "gemm" && argc == 3) return gemm(argv[2]);
+        if (cmd == "moe-grouped" && argc == 3) return moe_grouped(argv[2]);
+        if (cmd == "keeps" && argc == 3) return keeps(argv[2]);
         if (cmd == "panics") return panics();
         fprintf(stderr, "usage: host_parity missing | matrix-checks | cnq-list F | cnq-refuse F | cnq-dequant F DIR | dense DIR | head DIR | moe DIR | gemm DIR | panics\n");
         return 2;

@@ -161,6 +161,8 @@ def test_dense_ffn_w_and_dense_proj(tmp_path, t, xbf16):
         assert rel_err(_read(d, "y.bin", np.float32, (t, R)), orc.gemv(wd, R, I, gs[2], h_ref)) <= TOL
     if not xbf16:
         assert rel_err(_read(d, "gate_y.bin", np.float32, (t, I)), orc.gemv(wg, I, H, gs[0], xw)) <= TOL
+    if t == 1 and not xbf16:  # the captured step, replayed three times: the eager launches' bits
+        assert np.array_equal(_read(d, "y_graph.bin", np.uint32, (1, R)), _read(d, "y.bin", np.uint32, (1, R)))
 
 
 @pytest.mark.gpu
@@ -198,6 +200,40 @@ def test_moe_run(tmp_path, t):
     assert np.array_equal(_read(d, "ids.bin", np.int32, (t, K)), np.asarray(ids_ref).reshape(t, K))
     assert np.allclose(_read(d, "wts.bin", np.float32, (t, K)), np.asarray(wts_ref).reshape(t, K), rtol=1e-6, atol=1e-7)
     assert rel_err(_read(d, "y.bin", np.float32, (t, H)), np.asarray(y_ref).reshape(t, H)) <= TOL
+
+
+@pytest.mark.gpu
+def test_moe_run_grouped(tmp_path):
+    from gpu_common import TOL, rel_err
+    E, K, H, I, t = 64, 4, 512, 256, 24
+    d = str(tmp_path)
+    gu, dn = random_nvfp4(63, E * 2 * I, H), random_nvfp4(64, E * H, I)
+    gs = np.array([1.3e-3, 0.9e-3], np.float32)
+    x = normal_f32(14, 1, t * H).reshape(t, H) * np.float32(0.1)
+    logits = normal_f32(15, 1, t * E).reshape(t, E)
+    for name, a in (("gu.bin", gu), ("dn.bin", dn), ("gs.bin", gs), ("x.bin", x), ("logits.bin", logits)):
+        _write(d, name, a)
+    open(os.path.join(d, "meta.txt"), "w").write(f"{E} {K} {H} {I} {t}\n")
+    run("moe-grouped", d)
+    ids_ref, wts_ref, y_ref = orc.moe_layer(gu, gs[0], dn, gs[1], E, H, I, x, logits, K, threads=4)
+    assert np.array_equal(_read(d, "ids.bin", np.int32, (t, K)), np.asarray(ids_ref).reshape(t, K))
+    assert rel_err(_read(d, "y.bin", np.float32, (t, H)), np.asarray(y_ref).reshape(t, H)) <= TOL
+
+
+@pytest.mark.gpu
+def test_keep_projections(tmp_path):
+    from gpu_common import TOL, rel_err
+    rows, k, t = 256, 2560, 2
+    d = str(tmp_path)
+    w = normal_f32(16, 1, rows * k).reshape(rows, k) * np.float32(0.05)
+    bits = orc.f32_to_bf16_bits(w).reshape(rows, k)
+    x = normal_f32(17, 1, t * k).reshape(t, k)
+    for name, a in (("w_bf16.bin", bits), ("w_f32.bin", w), ("x.bin", x)):
+        _write(d, name, a)
+    open(os.path.join(d, "meta.txt"), "w").write(f"{rows} {k} {t}\n")
+    run("keeps", d)
+    assert rel_err(_read(d, "y_bf16.bin", np.float32, (t, rows)), orc.gemv_bf16(bits, rows, k, x)) <= TOL
+    assert rel_err(_read(d, "y_f32.bin", np.float32, (t, rows)), orc.gemv_f32w(w, rows, k, x)) <= TOL
 
 
 @pytest.mark.gpu
