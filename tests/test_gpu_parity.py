@@ -134,6 +134,35 @@ def test_gemv_is_correct_for_every_split(eng, s, wv):
     assert rel_err(y1, ref) <= TOL and gamma_ratio(y1, w, rows, cols, gs, x) <= 1.0
 
 
+def test_ragged_shapes_drawn_at_random(eng):
+    """Forty shapes drawn with a fixed seed - any row count (partial last row tile), any whole number of 64-value blocks per
+    row (partial last panel), 1..4 activation rows, f32 or bf16 activations - through dense_proj / proj_m and the fused
+    gate/up kernels, each against the CPU path."""
+    from crow_nest_amd.engine import MlpW
+    g = np.random.default_rng(20240611)
+    for case in range(40):
+        rows = int(g.integers(1, 260))
+        cols = 64 * int(g.integers(1, 41))
+        m = int(g.integers(1, 5))
+        bf16 = bool(g.integers(0, 2))
+        print(f"case {case}: rows={rows} cols={cols} m={m} bf16={bf16}", flush=True)
+        w, w2 = random_nvfp4(1000 + case, rows, cols), random_nvfp4(2000 + case, rows, cols)
+        gs, gs2 = 7.0e-4, 1.1e-3
+        f, f2 = _load(w, rows, cols, gs), _load(w2, rows, cols, gs2)
+        x = normal_f32(8, case, m * cols).reshape(m, cols)
+        if bf16:
+            xb, xw = _bf16_dev(x)
+            xd, xo = xb.reshape(m, cols).contiguous(), xw.reshape(m, cols)
+        else:
+            xd, xo = _dev(x), x
+        ref = orc.gemv(w, rows, cols, gs, xo)
+        y = (eng.proj_m(f, m, xd) if (bf16 or m > 1) else eng.dense_proj(f, 1, xd)).cpu().numpy()
+        assert rel_err(y, ref) <= TOL, case
+        h = eng.gate_up(MlpW(f, f2, f), m, xd).cpu().numpy()
+        assert rel_err(h, orc.silu_mul(ref, orc.gemv(w2, rows, cols, gs2, xo))) <= TOL, case
+    eng.check()
+
+
 def test_split_launches_back_to_back_with_changing_inputs(eng):
     """A small cross-block split launched 24 times in a row without a host wait, every launch on another x: the partial
     sums a block reads are the ones this launch's blocks wrote, never an earlier launch's (the launches are small enough
