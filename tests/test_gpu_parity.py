@@ -363,6 +363,45 @@ def test_moe_layer_both_launch_sequences(eng, t):
     eng.check()
 
 
+def test_moe_layer_other_geometries_drawn_at_random(eng):
+    """Eight routed layers with other expert counts, pick counts, widths and batch sizes (fixed seed), every launch
+    sequence - five launches, three, two (router inside gate|up), grouped by expert - against the CPU path."""
+    from crow_nest_amd.engine import MoeW, expert_table
+    from crow_nest_amd.kernels import KernelGeo
+    from crow_nest_amd.weights import load_expert_slabs
+    g = np.random.default_rng(77)
+    keep = eng.geo
+    try:
+        for case in range(8):
+            E = int(g.choice([64, 128]))
+            K = int(g.choice([1, 2, 3, 6, 8, 10]))
+            H = 64 * int(g.integers(2, 13))
+            I = 64 * int(g.integers(1, 7))
+            t = int(g.integers(1, 8))
+            print(f"case {case}: E={E} K={K} H={H} I={I} t={t}", flush=True)
+            eng.set_geo(KernelGeo(experts=E, topk=K, hidden=H, inter=I))
+            gu = random_nvfp4(300 + case, E * 2 * I, H, scale_lo=0x30, scale_hi=0x48, p7f=0)
+            dn = random_nvfp4(400 + case, E * H, I, scale_lo=0x30, scale_hi=0x48, p7f=0)
+            gs_gu, gs_dn = 2.0e-3, 3.0e-3
+            s_gu, s_dn = load_expert_slabs(gu, E, 2 * I, H, gs_gu), load_expert_slabs(dn, E, H, I, gs_dn)
+            moe = MoeW(s_gu, s_dn, expert_table(s_gu, s_dn))
+            x = (normal_f32(15, case, t * H) * np.float32(0.1)).reshape(t, H)
+            logits = normal_f32(16, case, t * E).reshape(t, E)
+            ids_ref, w_ref, y_ref = orc.moe_layer(gu, gs_gu, dn, gs_dn, E, H, I, x, logits, K, threads=4)
+            for fused in (False, True, "route", "grouped"):
+                if fused == "grouped":
+                    ids, wts, y, _ = eng.moe_run_grouped(moe, _dev(x), _dev(logits))
+                else:
+                    ids, wts, y = eng.moe_run(moe, _dev(x), _dev(logits), fused=fused)
+                eng.check()
+                assert np.array_equal(ids.cpu().numpy(), ids_ref), (case, fused)
+                assert np.allclose(wts.cpu().numpy(), w_ref, rtol=2e-6, atol=0), (case, fused)
+                assert rel_err(y.cpu().numpy(), y_ref) <= TOL, (case, fused)
+    finally:
+        eng.set_geo(keep)
+    eng.check()
+
+
 @pytest.mark.parametrize("t", [3, 24, 64])
 def test_moe_layer_grouped_by_expert(eng, t):
     """Batches in which experts repeat: the plan is a stable sort of the combos by expert cut into tiles of at most four,
