@@ -531,6 +531,28 @@ def test_gemm_bf16_against_the_cpu_path(eng, m, rows, cols, kernel):
     _gemm_case(eng, m, rows, cols, kernel)
 
 
+def test_gemm_ragged_shapes_drawn_at_random(eng):
+    """Sixteen (tokens, rows, columns) triples drawn with a fixed seed - partial row tiles, partial panels, partial token
+    blocks - through the entry point the library picks and through one drawn at random."""
+    g = np.random.default_rng(4242)
+    names = ["gemm_nvfp4_bf16_m32", "gemm_nvfp4_bf16_m48", "gemm_nvfp4_bf16_m64", "gemm_nvfp4_bf16_m96", "gemm_nvfp4_bf16"]
+    for case in range(16):
+        m = int(g.integers(5, 300))
+        rows = int(g.integers(1, 700))
+        cols = 64 * int(g.integers(1, 50))
+        forced = names[int(g.integers(0, len(names)))] if m > 16 else "gemm_nvfp4_bf16_m16"
+        print(f"case {case}: m={m} rows={rows} cols={cols} forced={forced}", flush=True)
+        w = random_nvfp4(500 + case, rows, cols)
+        gs = 6.0e-4
+        f = _load(w, rows, cols, gs)
+        xb, xw = _bf16_dev(normal_f32(17, case, m * cols))
+        ref = orc.gemv(w, rows, cols, gs, xw.reshape(m, cols), threads=8)
+        for kernel in (None, forced):
+            y = eng.gemm(f, m, xb.reshape(m, cols).contiguous(), kernel=kernel).cpu().numpy()
+            eng.check()
+            assert rel_err(y, ref) <= TOL, (case, kernel)
+
+
 def test_gemm_m16_full_size_cross_block_split(eng):
     """[17408, 5120] at 16 tokens: the K-split kernel's five column slices meet through the workspace."""
     _gemm_case(eng, 16, 17408, 5120, "gemm_nvfp4_bf16_m16")
