@@ -3,7 +3,7 @@
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-others] [--no-cpu]
 
-One "step" is one pass of BASELINE config 1 at batch 1 (M = 1): the fused gate/up + SiLU GEMV
+One "step" is one pass of benchmark config 1 at batch 1 (M = 1): the fused gate/up + SiLU GEMV
 (W_gate, W_up [17408, 5120] NVFP4, X bf16) followed by the down projection (W_down [5120, 17408]
 on the f32 H) - the dense FFN of one decode token at the 27B shape.  Weights are N(0, 0.02^2),
 seed 0, through the ceil encoder; they are resident in HBM before the timed region and every step
@@ -11,7 +11,7 @@ reads a different copy (10 copies, 1.5 GB) so that the 256 MB memory-side cache 
 `value` = algorithmic bytes of the step / wall time per step.  The JSON line also carries the
 roofline of the dominant kernel (HIP events around back-to-back launches of that kernel alone on
 the launch stream), the CPU baseline (the C restatement of the reference's CPU NVFP4 path on this
-host's cores: a port, not the Rust binary), and microseconds per call for the other BASELINE shapes.
+host's cores: a port, not the Rust binary), and microseconds per call for the other benchmark shapes (configs 0, 2, 3, 4).
 """
 from __future__ import annotations
 
@@ -197,7 +197,7 @@ def main() -> int:
         "roofline": roof,
     }
 
-    # ---------------- the other BASELINE shapes: us per call (timing only: random codes, valid scale bytes)
+    # ---------------- the other benchmark shapes: us per call (timing only: random codes, valid scale bytes)
     if not a.no_others:
         others = {}
 

@@ -38,7 +38,7 @@ def gamma_ratio(y, w, rows, cols, gs, x) -> float:
 
 
 def quantized_normal(seed: int, stream: int, rows: int, cols: int, sigma: float = 0.02):
-    """BASELINE's weights: N(0, sigma^2) through the ceil encoder -> (container bytes, global scale)."""
+    """The benchmark's weights: N(0, sigma^2) through the ceil encoder -> (container bytes, global scale)."""
     v = normal_f32(seed, stream, rows * cols, sigma)
     return orc.quantize_ceil(v)
 

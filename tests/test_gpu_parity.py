@@ -219,7 +219,7 @@ def test_fused_gate_up_silu_and_down(eng, t):
     y = eng.dense_ffn_w(mlp, _dev(x), t).cpu().numpy()
     y_ref = orc.ffn(wg, gs[0], wu, gs[1], wd, gs[2], H, I, x)
     assert rel_err(y, y_ref) <= TOL
-    # bf16 activations (BASELINE config 1): the oracle gets the exactly widened values
+    # bf16 activations (benchmark config 1: bf16 X): the oracle gets the exactly widened values
     xb, xw = _bf16_dev(x)
     hb = eng.gate_up(mlp, t, xb.reshape(t, H).contiguous()).cpu().numpy()
     hb_ref = orc.silu_mul(orc.gemv(wg, I, H, gs[0], xw), orc.gemv(wu, I, H, gs[1], xw))
@@ -442,7 +442,7 @@ def test_moe_layer_grouped_by_expert(eng, t):
     eng.check()
 
 
-# ---------------------------------------------------------------- BASELINE config 0 at full size
+# ---------------------------------------------------------------- benchmark config 0 (dense GEMV [17408, 5120], f32 x) at full size
 
 def test_config0_full_size(eng):
     rows, cols = 17408, 5120
@@ -461,10 +461,10 @@ def test_config0_full_size(eng):
     assert np.array_equal(d.view(np.uint32), orc.dequant(w[:256 * cols // 64 * 36], gs).view(np.uint32))
 
 
-# ---------------------------------------------------------------- BASELINE config 1 at full size
+# ---------------------------------------------------------------- benchmark config 1 (gate | up + SiLU and down, M <= 4) at full size
 
 def test_config1_full_size_properties(eng):
-    """[17408, 5120] gate / up and [5120, 17408] down, BASELINE's weights and bf16 X, four token rows: sampled row slabs
+    """[17408, 5120] gate / up and [5120, 17408] down, the benchmark's weights and bf16 X, four token rows: sampled row slabs
     against the CPU path, every row of the four-row launch bit-identical to its own one-row launch, and the down
     projection exactly linear under power-of-two scaling."""
     from crow_nest_amd.engine import MlpW
@@ -496,7 +496,7 @@ def test_config1_full_size_properties(eng):
         assert np.array_equal(y1.view(np.uint32)[0], y.view(np.uint32)[t]), t
 
 
-# ---------------------------------------------------------------- BASELINE config 3 at full size
+# ---------------------------------------------------------------- benchmark config 3 (lm_head [151936, 5120] + greedy argmax) at full size
 
 def test_config3_full_size_head(eng):
     """[151936, 5120] head (random codes and scales: the encoder is not what is tested here): sampled row slabs against the
@@ -578,7 +578,7 @@ def _gemm_case(eng, m, rows, cols, kernel):
 
 
 def test_gemm_full_size_sampled_rows(eng):
-    """BASELINE config 4 at M = 512 on the full [17408, 5120] tensor; the CPU path checks 768 sampled rows."""
+    """Benchmark config 4 (batched GEMM) at M = 512 on the full [17408, 5120] tensor; the CPU path checks 768 sampled rows."""
     rows, cols, m = 17408, 5120, 512
     w, gs = quantized_normal(0, 0, rows, cols)
     f = _load(w, rows, cols, gs)
