@@ -635,7 +635,7 @@ uint64_t Cnq::byte_len(const TensorInfo& t) {
     return (t.n_values + 63) / 64 * 36;  // nvfp4
 }
 std::vector<uint8_t> Cnq::read_at(uint64_t off, uint64_t n) const {
-    if (off + n > file_len - 8) throw Refused("read of " + std::to_string(n) + " B at " + std::to_string(off) + " runs off the payload of a " + std::to_string(file_len) + " B container");
+    if (n > file_len - 8 || off > file_len - 8 - n) throw Refused("read of " + std::to_string(n) + " B at " + std::to_string(off) + " runs off the payload of a " + std::to_string(file_len) + " B container");
     std::ifstream f(path, std::ios::binary);
     std::vector<uint8_t> out(n);
     f.seekg((std::streamoff)off);
