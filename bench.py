@@ -290,7 +290,6 @@ def main() -> int:
             lgu = Launch(eng, "moe_gate_up_silu", I, H, t * K8, [[gup.data_ptr(), xt.data_ptr(), gs1.data_ptr(), h2.data_ptr(), p.i32(H), p.i32(K8),
                                                                   p.i32(H), p.i32(I)]])
             ldn = Launch(eng, "moe_down_combine", H, I, t, [[dnp.data_ptr(), h2.data_ptr(), gs1.data_ptr(), wts.data_ptr(), yt.data_ptr(), p.i32(I), p.i32(H)]])
-            ldn.dims = (1, (H + 63) // 64, t, 64 * K8)
 
             # the layer as Engine.moe_layer runs it at these widths: the router inside the gate|up launch, then down + combine
             lrg = Launch(eng, "moe_route_gate_up_silu", I, H, t * K8,

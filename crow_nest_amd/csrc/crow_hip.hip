@@ -16,29 +16,35 @@ struct FnEntry {
     const char* name;
     const void* stub;
     int nargs;
-    unsigned lds_fixed, lds_per_wave;  // dynamic LDS of a launch = lds_fixed + lds_per_wave * (block size / 64)
+    unsigned lds_fixed;  // dynamic LDS of a launch (kernels outside the GEMV family)
+    // GEMV family (gemv.h): tensors per block (0 = not of the family), and the dynamic LDS of a block as a function of the most
+    // groups one of its waves owns: zero area + one staging area per wave
+    int nr;
+    int (*lds_zero)(int most);
+    int (*lds_per_wave)(int most);
 };
 
-// GEMV blocks (gemv.h): 512 zero bytes, then per wave XR staging rows (which also take the wave's NR * M hand-over rows
-// of 256 bytes once the staged activations are dead)
-#define CROW_FN(name, nargs) {#name, (const void*)&name, nargs, 0u, 0u}
-#define CROW_GEMV(name, nargs, NR, M, XR) {#name, (const void*)&name, nargs, CROW_GEMV_ZERO_BYTES, (XR) * CROW_GEMV_XROW_BYTES}
+#define CROW_FN(name, nargs) {#name, (const void*)&name, nargs, 0u, 0, nullptr, nullptr}
+// NR tensors per block, bodies for 1 .. MMAX activation rows, bf16 or f32 activations
+#define CROW_GEMV(name, nargs, NR, MMAX, XBF16) \
+    {#name, (const void*)&name, nargs, 0u, NR, &crow::StagingAlloc<MMAX, XBF16>::zero_bytes, &crow::StagingAlloc<MMAX, XBF16>::per_wave}
 const FnEntry g_table[] = {
-    CROW_GEMV(gemv_nvfp4_w, 6, 1, 1, 4),       CROW_GEMV(gemv_nvfp4_w_bf16, 6, 1, 1, 1),  CROW_GEMV(gemv_nvfp4_w_argmax, 7, 1, 1, 4),
-    CROW_GEMV(gemv_nvfp4_gu, 8, 1, 1, 4),      CROW_GEMV(gemv_nvfp4_gu_bf16, 8, 1, 1, 1),
-        CROW_GEMV(gemv_nvfp4_wm, 7, 1, 4, 12),     CROW_GEMV(gemv_nvfp4_gum, 9, 2, 4, 12),
-    CROW_GEMV(gemv_nvfp4_wm_bf16, 7, 1, 4, 4), CROW_GEMV(gemv_nvfp4_gum_bf16, 9, 2, 4, 4), CROW_GEMV(gemv_fp4, 6, 1, 1, 4),
-    CROW_GEMV(gemv_fp4_b, 7, 1, 4, 12),        CROW_GEMV(gemv_fp4_b1k, 7, 1, 4, 12),      CROW_GEMV(gemv_fp4_bs, 8, 1, 4, 12),
-    CROW_GEMV(gemv_fp4_ptrb, 8, 1, 1, 4),      CROW_GEMV(moe_gate_up_silu, 8, 1, 1, 4),   CROW_GEMV(moe_down_combine, 7, 1, 1, 4),
-    CROW_GEMV(moe_route_gate_up_silu, 11, 1, 1, 4), CROW_GEMV(moe_gate_up_silu_grouped, 11, 2, 4, 12), CROW_GEMV(moe_down_grouped, 9, 1, 4, 12), CROW_FN(moe_group, 6),
+    CROW_GEMV(gemv_nvfp4_w, 6, 1, 1, false),       CROW_GEMV(gemv_nvfp4_w_bf16, 6, 1, 1, true),  CROW_GEMV(gemv_nvfp4_w_argmax, 7, 1, 1, false),
+    CROW_GEMV(gemv_nvfp4_gu, 8, 2, 1, false),      CROW_GEMV(gemv_nvfp4_gu_bf16, 8, 2, 1, true),
+    CROW_GEMV(gemv_nvfp4_wm, 7, 1, 4, false),      CROW_GEMV(gemv_nvfp4_gum, 9, 2, 4, false),
+    CROW_GEMV(gemv_nvfp4_wm_bf16, 7, 1, 4, true),  CROW_GEMV(gemv_nvfp4_gum_bf16, 9, 2, 4, true), CROW_GEMV(gemv_fp4, 6, 1, 1, false),
+    CROW_GEMV(gemv_fp4_b, 7, 1, 4, false),         CROW_GEMV(gemv_fp4_b1k, 7, 1, 4, false),      CROW_GEMV(gemv_fp4_bs, 8, 1, 4, false),
+    CROW_GEMV(gemv_fp4_ptrb, 8, 1, 1, false),      CROW_GEMV(moe_gate_up_silu, 8, 2, 1, false),  CROW_GEMV(moe_down_combine, 7, 1, 1, false),
+    CROW_GEMV(moe_route_gate_up_silu, 11, 2, 1, false), CROW_GEMV(moe_gate_up_silu_grouped, 11, 2, 4, false), CROW_GEMV(moe_down_grouped, 9, 1, 4, false),
+    CROW_FN(moe_group, 6),
     CROW_FN(router_top10, 10),     CROW_FN(silu_mul_combo, 3),      CROW_FN(acc_combo, 3),
     CROW_FN(argmax_k, 3),          CROW_FN(argmax_tiles, 2),        CROW_FN(dequant_fp4_flat, 4),    CROW_FN(repack_nvfp4, 4),
     CROW_FN(unpack_nvfp4, 4),      CROW_FN(dequant_nvfp4_tiled, 5),
     // shared-X GEMM blocks: two staged X tiles of MT rows x 528 bytes
-    {"gemm_nvfp4_bf16", (const void*)&gemm_nvfp4_bf16, 7, 2u * 128u * 528u, 0u},
-    {"gemm_nvfp4_bf16_m64", (const void*)&gemm_nvfp4_bf16_m64, 7, 2u * 64u * 528u, 0u},
-    {"gemm_nvfp4_bf16_m48", (const void*)&gemm_nvfp4_bf16_m48, 7, 2u * 48u * 528u, 0u},
-    {"gemm_nvfp4_bf16_m96", (const void*)&gemm_nvfp4_bf16_m96, 7, 2u * 96u * 528u, 0u},
+    {"gemm_nvfp4_bf16", (const void*)&gemm_nvfp4_bf16, 7, 2u * 128u * 528u, 0, nullptr, nullptr},
+    {"gemm_nvfp4_bf16_m64", (const void*)&gemm_nvfp4_bf16_m64, 7, 2u * 64u * 528u, 0, nullptr, nullptr},
+    {"gemm_nvfp4_bf16_m48", (const void*)&gemm_nvfp4_bf16_m48, 7, 2u * 48u * 528u, 0, nullptr, nullptr},
+    {"gemm_nvfp4_bf16_m96", (const void*)&gemm_nvfp4_bf16_m96, 7, 2u * 96u * 528u, 0, nullptr, nullptr},
     CROW_FN(gemm_nvfp4_bf16_m32, 7), CROW_FN(gemm_nvfp4_bf16_m16, 7), CROW_FN(gemv_bf16_w, 5),
     CROW_FN(gemv_bf16, 5), CROW_FN(gemv_bf16_b, 5), CROW_FN(gemv_b, 5), CROW_FN(gemv_bf16_ws, 5), CROW_FN(gemv_bf16_bs, 6),
 };
@@ -53,6 +59,7 @@ struct State {
     int* scalars = nullptr;  // two device words for the library's own launches (rows, k_dim)
     char name[256] = {0};
     int geo_topk = 0;  // host copy of the routed geometry (crow_hip_set_geo), for launch shapes
+    size_t lds_cap = 64u * 1024u;  // most LDS one workgroup may take on this device
 } g;
 
 const unsigned long long PARTIAL_FLOATS = 16ull << 20;  // 64 MiB of split-K partial sums
@@ -78,16 +85,38 @@ const FnEntry* entry_of(crow_fn_t f) {
     return e;
 }
 
+
+// The launch dimensions of the GEMV family carry the problem in `gy` (crow_hip_launch_dims writes it, callers pass it on
+// unchanged): bits 0..19 = K / 64, bits 20..23 = activation rows of the last token group (0 = not given), bits 24..31 = S, the
+// number of column slices per strip.  The real grid is (gx, S, gz); the low 24 bits reach the kernel by value.
 int launch_entry(const FnEntry* e, dim3 grid, dim3 block, const uint64_t* vals, uint32_t n, hipStream_t s) {
     if (!g.ready) return CROW_ERR_NOT_INITIALIZED;
     if (!e || !vals) return CROW_ERR_BAD_ARGUMENT;
     if ((int)n != e->nargs) return CROW_ERR_ARG_COUNT;
     // whole wavefronts only: every kernel derives its wave count (and its LDS layout) from block.x / 64
     if (grid.x == 0 || grid.y == 0 || grid.z == 0 || block.x == 0 || block.x > 1024 || block.x % 64 != 0) return CROW_ERR_BAD_ARGUMENT;
-    void* args[16];
+    void* args[17];
     for (uint32_t i = 0; i < n; i++) args[i] = (void*)&vals[i];
-    const size_t lds = e->lds_fixed + (size_t)e->lds_per_wave * (block.x / 64);
-    return hip_rc(hipLaunchKernel(e->stub, grid, block, args, lds, s));
+    size_t lds = e->lds_fixed;
+    int geo = 0;
+    if (e->nr != 0) {
+        const unsigned word = grid.y;
+        const int pairs = (int)(word & 0xFFFFFu), slices = (int)(word >> 24) == 0 ? 1 : (int)(word >> 24);
+        const int waves = (int)(block.x / 64), wpt = waves / e->nr;
+        if (pairs == 0 || wpt == 0) return CROW_ERR_BAD_ARGUMENT;
+        const int groups = (pairs + CROW_GROUP_PAIRS - 1) / CROW_GROUP_PAIRS;
+        // (moe_down_combine's waves are the token's picks: each owns all groups of its strip)
+        int most = e->stub == (const void*)&moe_down_combine ? groups : crow::crow_most_groups(groups, slices * wpt);
+        if (most > CROW_GEMV_GMAX) most = CROW_GEMV_GMAX;
+        lds = (size_t)e->lds_zero(most) + (size_t)waves * (size_t)e->lds_per_wave(most);
+        if (lds > g.lds_cap) return CROW_ERR_SHAPE;
+        geo = (int)(word & 0xFFFFFFu);
+        grid.y = (unsigned)slices;
+        args[n] = (void*)&geo;
+    }
+    const hipError_t rc = hipLaunchKernel(e->stub, grid, block, args, lds, s);
+    if (rc != hipSuccess) (void)hipGetLastError();  // reported here: not left behind for an unrelated later call to find
+    return hip_rc(rc);
 }
 
 }  // namespace
@@ -106,6 +135,7 @@ int crow_hip_init(int device) {
         return CROW_ERR_BAD_ARGUMENT;
     }
     g.cus = pr.multiProcessorCount;
+    g.lds_cap = pr.maxSharedMemoryPerMultiProcessor > 0 ? (size_t)pr.maxSharedMemoryPerMultiProcessor : (size_t)pr.sharedMemPerBlock;
     crow::Workspace ws{};
     ws.partial_floats = PARTIAL_FLOATS;
     ws.counter_slots = COUNTER_SLOTS;
@@ -132,7 +162,11 @@ int crow_hip_init(int device) {
     if ((e = hipMemcpyToSymbol(HIP_SYMBOL(crow::g_geo), &geo, sizeof geo)) != hipSuccess) return fail(e);
     // a GEMV block of 16 waves, and the GEMM's two staged X tiles, need more dynamic LDS than the default per-block limit
     for (int i = 0; i < g_table_n; i++) {
-        const size_t most = g_table[i].lds_fixed + 16 * (size_t)g_table[i].lds_per_wave;
+        size_t most = g_table[i].lds_fixed;
+        if (g_table[i].nr != 0) {  // the GEMV family: a block of sixteen waves at the longest staged rows, within the device's limit
+            most = (size_t)g_table[i].lds_zero(CROW_GEMV_GMAX) + 16 * (size_t)g_table[i].lds_per_wave(CROW_GEMV_GMAX);
+            if (most > g.lds_cap) most = g.lds_cap;
+        }
         if (most > 48 * 1024 &&
             (e = hipFuncSetAttribute(g_table[i].stub, hipFuncAttributeMaxDynamicSharedMemorySize, (int)most)) != hipSuccess)
             return fail(e);
@@ -254,17 +288,16 @@ const char* crow_hip_gemm_kernel(uint32_t rows, uint32_t m) {
     return best;
 }
 
-// Split of a [rows, k_dim] product over the chip.  Every wave owns one 64-row tile; a tile's
-// 256-column panels are dealt to W waves of a block (combined in LDS) and S blocks (combined
-// through the workspace): enough waves that every CU holds enough 16-byte loads in flight to
-// cover HBM latency, and far more blocks than CUs so that the hardware dispatcher balances them.
-// The result depends on (rows, k_dim) only.
+// Split of a [rows, k_dim] product over the chip.  A block owns one 16-row strip; the strip's 256-column groups are dealt
+// to W waves of the block (combined in LDS) and, only when a strip has more groups than one block's waves can hold, to S
+// blocks (combined through the workspace).  The result depends on (rows, k_dim) only.
 int crow_hip_launch_dims_split(const char* name, uint32_t rows, uint32_t k_dim, uint32_t z, uint32_t force_s, uint32_t force_w, crow_dims* out) {
     if (!out || !name || rows == 0 || z == 0) return CROW_ERR_BAD_ARGUMENT;
     const FnEntry* e = find(name);
     if (!e) return CROW_ERR_KERNEL_MISSING;
-    const uint32_t rt = (rows + CROW_TILE_ROWS - 1) / CROW_TILE_ROWS;
-    const uint32_t panels = (k_dim + CROW_PANEL_COLS - 1) / CROW_PANEL_COLS;
+    const uint32_t strips = (rows + CROW_STRIP_ROWS - 1) / CROW_STRIP_ROWS;
+    const uint32_t groups = (k_dim + CROW_GROUP_COLS - 1) / CROW_GROUP_COLS;
+    const uint32_t rt = (rows + CROW_TILE_ROWS - 1) / CROW_TILE_ROWS, panels = groups;  // the GEMM's 64-row tiles
     if (strcmp(name, "gemv_bf16_w") == 0 || strcmp(name, "gemv_bf16") == 0 || strcmp(name, "gemv_bf16_b") == 0 || strcmp(name, "gemv_b") == 0 ||
         strcmp(name, "gemv_bf16_ws") == 0 || strcmp(name, "gemv_bf16_bs") == 0) {
         // z = T activation rows; whole 16-byte loads: 8 bf16 or 4 f32 weights
@@ -278,53 +311,45 @@ int crow_hip_launch_dims_split(const char* name, uint32_t rows, uint32_t k_dim, 
         *out = crow_dims{(rows + 3) / 4, z, 1, 256};
         return CROW_OK;
     }
-    if (strncmp(name, "gemv_", 5) == 0 || strncmp(name, "moe_gate_up", 11) == 0 || strcmp(name, "moe_down_grouped") == 0 ||
-        strcmp(name, "moe_route_gate_up_silu") == 0) {
-        if (k_dim == 0 || k_dim % CROW_BLOCK_VALUES != 0) return CROW_ERR_SHAPE;
-        const bool moe = strcmp(name, "gemv_fp4_ptrb") == 0 || strncmp(name, "moe_", 4) == 0;
+    if (e->nr != 0) {  // the NVFP4 GEMV family
+        if (k_dim == 0 || k_dim % CROW_BLOCK_VALUES != 0 || k_dim / CROW_BLOCK_VALUES > 0xFFFFFu) return CROW_ERR_SHAPE;
+        const uint32_t pairs = k_dim / CROW_BLOCK_VALUES;
+        const bool down_combine = strcmp(name, "moe_down_combine") == 0;
+        const bool routed = strcmp(name, "gemv_fp4_ptrb") == 0 || strncmp(name, "moe_", 4) == 0;
         const bool tokens = strcmp(name, "gemv_fp4_b") == 0 || strcmp(name, "gemv_fp4_b1k") == 0 || strcmp(name, "gemv_fp4_bs") == 0;
-        const bool two = strstr(name, "_gu") != nullptr || strncmp(name, "moe_gate_up", 11) == 0 || strcmp(name, "moe_route_gate_up_silu") == 0;
-        const uint32_t tiles = rt;  // rows = output rows for every kernel
-        const uint32_t gz = moe ? z : (tokens ? (z + 3) / 4 : 1);
-        // A tile's panels are dealt to S blocks of W waves.  Measured on MI355X (17408 x 5120,
-        // 5120 x 17408, 151936 x 5120): a wave that owns ONE panel, with every wave of the launch
-        // resident at once, streams best (all loads are in flight from the start; a second panel in
-        // the same wave pays the memory latency again); W = 4..12 waves combine in LDS, the S
-        // blocks of a tile through the workspace (each costs a round trip, so S stays small: for
-        // the 68 panels of K = 17408, 6 x 12 measured 6 % faster than 9 x 8).
-        // When there are more (tile, panel) units than resident waves, waves take several panels.
-        const long resident = 32L * g.cus;  // wave slots at <= 64 VGPRs
-        const long all_tiles = (long)tiles * (moe ? gz : 1);
-        long units = all_tiles * (long)panels <= resident ? (long)panels : (2 * resident + all_tiles - 1) / all_tiles;
-        if (units < 1) units = 1;
-        if (units > (long)panels) units = panels;
-        long w = units <= 8 ? units : (panels > 32 ? 12 : 4);
-        long s = (units + w - 1) / w;
-        // the grouped gate|up kernel (two tensors, four f32 rows: the heaviest wave) runs best in small blocks whose waves
-        // take equal shares of the panels (measured at 8 panels: 4 waves 51 us, 6 waves 67 us, 8 waves 61 us for 64 tokens)
-        if (strcmp(name, "moe_gate_up_silu_grouped") == 0 && panels >= 4) {
-            w = 4;
+        const bool verify = strcmp(name, "gemv_nvfp4_wm") == 0 || strcmp(name, "gemv_nvfp4_gum") == 0 || strcmp(name, "gemv_nvfp4_wm_bf16") == 0 ||
+                            strcmp(name, "gemv_nvfp4_gum_bf16") == 0;
+        if (down_combine) {  // rows = hidden; one wave per picked expert, every wave all columns of its strip
+            if (g.geo_topk < 1 || g.geo_topk > 16) return CROW_ERR_GEO;
+            *out = crow_dims{strips, pairs | (1u << 24), z, 64u * (uint32_t)g.geo_topk};
+            return CROW_OK;
+        }
+        if (verify && z > 4) return CROW_ERR_SHAPE;
+        const uint32_t wmax = 16u / (uint32_t)e->nr;  // waves per tensor in a block of at most 1024 threads
+        // A wave takes at most four groups (9 KB of loads, all in flight from its first instruction).  One block holds a
+        // strip when that needs no more waves than a block has; longer strips are cut into slices of four waves.
+        const uint32_t units = (groups + CROW_GEMV_GMAX - 1) / CROW_GEMV_GMAX;
+        uint32_t w, s;
+        if (units <= wmax) {
+            w = units;
             s = 1;
+        } else {
+            w = 4;
+            s = (units + w - 1) / w;
         }
         if (force_s > 0) s = force_s;
         if (force_w > 0) w = force_w;
-        // gate/up kernels for one activation row run one tile per wave: 2 W waves per block (W per tensor), at most 1024 threads
-        const bool thin = strcmp(name, "gemv_nvfp4_gu") == 0 || strcmp(name, "gemv_nvfp4_gu_bf16") == 0 || strcmp(name, "moe_gate_up_silu") == 0 ||
-                          strcmp(name, "moe_route_gate_up_silu") == 0;
-        // (the two-tensor kernels on four f32 rows are built for blocks of at most 512 threads)
-        const bool half = thin || strcmp(name, "gemv_nvfp4_gum") == 0 || strcmp(name, "moe_gate_up_silu_grouped") == 0;
-        if (w > (half ? 8 : 16)) w = half ? 8 : 16;
-        if (w < 1) w = 1;
-        if (s < 1) s = 1;
-        if (s * w > (long)panels) s = (panels + w - 1) / w;
-        const int nrm = (two ? 2 : 1) * 4;
-        out->gx = (uint32_t)s;
-        out->gy = tiles;
-        out->gz = gz;
-        out->bx = (uint32_t)(64 * w * (thin ? 2 : 1));
-        const unsigned long long need = (unsigned long long)tiles * gz * s * nrm * 64;
-        if (s > 1 && (need > PARTIAL_FLOATS || (unsigned long long)tiles * gz > COUNTER_SLOTS)) return CROW_ERR_WORKSPACE;
-        if (strcmp(name, "gemv_nvfp4_w_argmax") == 0 && tiles > AM_SLOTS) return CROW_ERR_WORKSPACE;
+        if (w > wmax) w = wmax;
+        if (s > 255) s = 255;
+        if (s * w > groups) {  // never more units than groups
+            if (w > groups) w = groups;
+            s = groups / w;
+        }
+        const uint32_t gz = routed ? z : (tokens ? (z + 3) / 4 : 1);
+        const uint32_t hint = verify ? z : (tokens ? (z - 1) % 4 + 1 : 0);
+        *out = crow_dims{strips, pairs | (hint << 20) | (s << 24), gz, 64u * w * (uint32_t)e->nr};
+        if (s > 1 && ((unsigned long long)strips * gz * s * 2 * 64 > PARTIAL_FLOATS || (unsigned long long)strips * gz > COUNTER_SLOTS)) return CROW_ERR_WORKSPACE;
+        if (strcmp(name, "gemv_nvfp4_w_argmax") == 0 && strips > AM_SLOTS) return CROW_ERR_WORKSPACE;
         return CROW_OK;
     }
     if (strncmp(name, "gemm_nvfp4_bf16", 15) == 0) {  // z = M token rows
@@ -345,13 +370,8 @@ int crow_hip_launch_dims_split(const char* name, uint32_t rows, uint32_t k_dim, 
         }
         return CROW_OK;
     }
-    if (strcmp(name, "moe_down_combine") == 0) {  // rows = hidden; one wave per picked expert
-        if (g.geo_topk < 1 || g.geo_topk > 16) return CROW_ERR_GEO;
-        *out = crow_dims{1, rt, z, 64u * (uint32_t)g.geo_topk};
-        return CROW_OK;
-    }
     if (strcmp(name, "repack_nvfp4") == 0 || strcmp(name, "unpack_nvfp4") == 0 || strcmp(name, "dequant_nvfp4_tiled") == 0) {
-        *out = crow_dims{panels, rt, 1, 64};
+        *out = crow_dims{groups, strips, 1, 64};
         return CROW_OK;
     }
     if (strcmp(name, "router_top10") == 0) { *out = crow_dims{z, 1, 1, 64}; return CROW_OK; }
@@ -372,7 +392,9 @@ int crow_hip_launch_dims(const char* name, uint32_t rows, uint32_t k_dim, uint32
 
 int crow_hip_status(void) {
     if (!g.ready) return CROW_ERR_NOT_INITIALIZED;
-    hipError_t e = hipStreamSynchronize(g.stream);
+    // every stream idle: a launch on another stream (an explicit one, or a graph's) may be in the middle of a hand-over whose
+    // arrival counters are cleared below, or may still be about to raise a status bit
+    hipError_t e = hipDeviceSynchronize();
     if (e != hipSuccess) return (int)e;
     unsigned st = 0;
     if ((e = hipMemcpy(&st, g.ws.status, sizeof st, hipMemcpyDeviceToHost)) != hipSuccess) return (int)e;
@@ -556,8 +578,8 @@ int crow_hip_time_graph(void* graph_exec, void* stream, uint32_t iters, float* u
 
 size_t crow_hip_container_bytes(uint32_t rows, uint32_t cols) { return crow_container_bytes(rows, cols); }
 size_t crow_hip_tiled_bytes(uint32_t rows, uint32_t cols) { return crow_tiled_bytes(rows, cols); }
-uint32_t crow_hip_tile_code_offset(uint32_t row, uint32_t wp) { return row < 64 && wp < 32 ? crow_tile_code_offset(row, wp) : UINT32_MAX; }
-uint32_t crow_hip_tile_scale_offset(uint32_t row, uint32_t sb) { return row < 64 && sb < 16 ? crow_tile_scale_offset(row, sb) : UINT32_MAX; }
+uint32_t crow_hip_tile_code_offset(uint32_t row, uint32_t wp) { return row < 16 && wp < 32 ? crow_group_code_offset(row, wp) : UINT32_MAX; }
+uint32_t crow_hip_tile_scale_offset(uint32_t row, uint32_t sb) { return row < 16 && sb < 16 ? crow_group_scale_offset(row, sb) : UINT32_MAX; }
 
 static int layout_launch(const char* name, const void* a, const void* b, const void* c, uint32_t rows, uint32_t cols) {
     if (!g.ready) return CROW_ERR_NOT_INITIALIZED;

@@ -30,6 +30,11 @@ __device__ __forceinline__ uint4 stream_load(const uint4* p) {
     return make_uint4(v.x, v.y, v.z, v.w);
 }
 
+// the same for one dword per lane (the scale words of a 256-column group)
+__device__ __forceinline__ unsigned stream_load_u32(const unsigned* p) {
+    return __builtin_nontemporal_load((const __attribute__((address_space(1))) unsigned*)p);
+}
+
 // Library-owned scratch for kernels that split one output tile over several workgroups:
 // per-slice partial sums and one arrival counter per output tile.  Set once by crow_hip_init.
 struct Workspace {

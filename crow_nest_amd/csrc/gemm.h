@@ -7,9 +7,10 @@
 // is the CDNA4 form of the latter: weights decode to EXACT bf16 (e2m1 * ue4m3 has at most 6
 // significant bits), X is bf16, products are exact in f32, v_mfma_f32_16x16x32_bf16 accumulates.
 //
-// Data flow.  A wave owns one 64-row weight tile per panel and MT = 16 * TBK token rows.  Per 256-column panel:
-//   * the wave loads its 9216-byte weight tile straight into registers (the GEMV's loads); every code dword
-//     is the B operand of one "unit" (16 weight rows x 32 columns, layout.h) as it stands;
+// Data flow.  A wave owns a 64-row weight tile - four 16-row strips of the layout - per 256-column panel and MT = 16 * TBK token
+// rows.  Per panel:
+//   * the wave loads the panel's group of each of its four strips (4 x 2304 bytes) straight into registers; every code
+//     dword is the B operand of one "unit" (16 weight rows x 32 columns, layout.h) as it stands;
 //   * X[m0 .. m0 + MT][panel] is staged in LDS (row stride 528 B) and read back as A operands, 16 token rows x
 //     32 columns per 16-byte-per-lane read, each used for the four row groups of the tile;
 //   * per unit a lane turns its 8 codes into 8 bf16 values times the sub-block scale (cvt to f32, multiply,
@@ -35,36 +36,55 @@ __device__ __forceinline__ bf16x8 decode8_scaled(unsigned codes, float scale) {
     return __builtin_bit_cast(bf16x8, r);
 }
 
-// The tile's scale bytes as the GEMM needs them.  A lane (g, n) holds, for row groups j = 2 jp + (g & 1) only, the
-// scales of the sub-block half g >> 1 (layout.h); the other two row groups are in the neighbouring 16-lane group.
-// After the exchange `even` holds the words of the even group of each pair in both groups, `odd` those of the odd one.
+#define CROW_TILE_ROWS 64    // four strips
+#define CROW_PANEL_COLS 256  // one group per strip
+// the registers of one panel of a 64-row tile: per strip J one scale dword and two code quadwords
+struct PanelRegs {
+    unsigned sc[4];
+    uint4 cd[4][2];
+};
+// `w` = the tensor, `strips` / `groups` its strip and group counts; strips beyond the tensor re-read the last one (their rows
+// are never stored)
+__device__ __forceinline__ void load_panel(const unsigned char* w, int rt, int strips, int groups, int p, int lane, PanelRegs& r) {
+#pragma unroll
+    for (int J = 0; J < 4; J++) {
+        const int strip = 4 * rt + J < strips ? 4 * rt + J : strips - 1;
+        const unsigned char* g = w + ((size_t)strip * groups + p) * CROW_GROUP_BYTES;
+        r.sc[J] = stream_load_u32((const unsigned*)g + lane);
+        r.cd[J][0] = stream_load((const uint4*)(g + CROW_GROUP_SCALE_BYTES) + lane);
+        r.cd[J][1] = stream_load((const uint4*)(g + CROW_GROUP_SCALE_BYTES + 1024) + lane);
+    }
+}
+
+// The panel's scale bytes as the GEMM needs them.  A lane (g, n) holds, for each strip, the scales of segment g & 1 of every
+// pair, sub-block half g >> 1 (layout.h); the other segment's are in the neighbouring 16-lane group.  After the exchange `even`
+// holds the word of the even group of each 32-lane half in both groups, `odd` that of the odd one.
 struct TileScales {
     unsigned even[4], odd[4];
-    __device__ __forceinline__ void set(const uint4& sc) {
+    __device__ __forceinline__ void set(const unsigned (&sc)[4]) {
 #pragma unroll
-        for (int q = 0; q < 4; q++) {
-            const unsigned own = u4_get(sc, q);
-            const u32x2 sw = __builtin_amdgcn_permlane16_swap(own, own, false, false);
-            even[q] = sw.x;
-            odd[q] = sw.y;
+        for (int J = 0; J < 4; J++) {
+            const u32x2 sw = __builtin_amdgcn_permlane16_swap(sc[J], sc[J], false, false);
+            even[J] = sw.x;
+            odd[J] = sw.y;
         }
     }
-    // scale of this lane's operand of unit (row group J, segment S)
+    // scale of this lane's operand of unit (strip J, segment S of the panel): pair S / 2, segment S % 2
     template <int S, int J>
     __device__ __forceinline__ float get() const {
-        return e4m3_to_f32<S & 3>((J & 1) ? odd[2 * (J >> 1) + (S >> 2)] : even[2 * (J >> 1) + (S >> 2)]);
+        return e4m3_to_f32<(S >> 1)>((S & 1) ? odd[J] : even[J]);
     }
 };
 
 // one 32-column segment S of the panel: four units, TBK token blocks each
 template <int TBK, int S>
-__device__ __forceinline__ void gemm_segment(const uint4 (&cd)[CROW_STEPS], const TileScales& ts, const __bf16* xs_lane, f32x4 (&acc)[TBK][4]) {
+__device__ __forceinline__ void gemm_segment(const PanelRegs& r, const TileScales& ts, const __bf16* xs_lane, f32x4 (&acc)[TBK][4]) {
     bf16x8 A[TBK];
 #pragma unroll
     for (int tb = 0; tb < TBK; tb++) A[tb] = *(const bf16x8*)(xs_lane + tb * 16 * CROW_GEMM_XS_STRIDE + S * 32);
 #define CROW_GEMM_UNIT(J)                                                                                      \
     {                                                                                                          \
-        const bf16x8 B = decode8_scaled(u4_get(cd[S], J), ts.get<S, J>());                                     \
+        const bf16x8 B = decode8_scaled(u4_get(r.cd[J][S >> 2], S & 3), ts.get<S, J>());                       \
         _Pragma("unroll") for (int tb = 0; tb < TBK; tb++)                                                     \
             acc[tb][J] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(A[tb], B, acc[tb][J], 0, 0, 0);               \
     }
@@ -73,17 +93,17 @@ __device__ __forceinline__ void gemm_segment(const uint4 (&cd)[CROW_STEPS], cons
 }
 
 template <int TBK>
-__device__ __forceinline__ void gemm_panel(const uint4& sc, const uint4 (&cd)[CROW_STEPS], const __bf16* xs_lane, f32x4 (&acc)[TBK][4]) {
+__device__ __forceinline__ void gemm_panel(const PanelRegs& r, const __bf16* xs_lane, f32x4 (&acc)[TBK][4]) {
     TileScales ts;
-    ts.set(sc);
-    gemm_segment<TBK, 0>(cd, ts, xs_lane, acc);
-    gemm_segment<TBK, 1>(cd, ts, xs_lane, acc);
-    gemm_segment<TBK, 2>(cd, ts, xs_lane, acc);
-    gemm_segment<TBK, 3>(cd, ts, xs_lane, acc);
-    gemm_segment<TBK, 4>(cd, ts, xs_lane, acc);
-    gemm_segment<TBK, 5>(cd, ts, xs_lane, acc);
-    gemm_segment<TBK, 6>(cd, ts, xs_lane, acc);
-    gemm_segment<TBK, 7>(cd, ts, xs_lane, acc);
+    ts.set(r.sc);
+    gemm_segment<TBK, 0>(r, ts, xs_lane, acc);
+    gemm_segment<TBK, 1>(r, ts, xs_lane, acc);
+    gemm_segment<TBK, 2>(r, ts, xs_lane, acc);
+    gemm_segment<TBK, 3>(r, ts, xs_lane, acc);
+    gemm_segment<TBK, 4>(r, ts, xs_lane, acc);
+    gemm_segment<TBK, 5>(r, ts, xs_lane, acc);
+    gemm_segment<TBK, 6>(r, ts, xs_lane, acc);
+    gemm_segment<TBK, 7>(r, ts, xs_lane, acc);
 }
 
 // acc[tb][j][r] of lane (g, n): token m0 + 16 tb + 4 g + r, weight row 64 rt + 16 j + n
@@ -130,7 +150,7 @@ __device__ __forceinline__ void gemm_small_body(const unsigned char* __restrict_
 #pragma unroll
         for (int j = 0; j < 4; j++) acc[tb][j] = f32x4{0.f, 0.f, 0.f, 0.f};
 
-    const uint4* wt = (const uint4*)(w + (size_t)rt * panels * CROW_TILE_BYTES) + lane;
+    const int strips = (rows + CROW_STRIP_ROWS - 1) / CROW_STRIP_ROWS;
     // 16 TBK tokens x 256 columns = 512 TBK chunks of 16 bytes, 8 TBK per lane; wave-private.  Chunk i of this lane: token row
     // 2 i + lane / 32, 8 columns from 8 (lane % 32); its element offset in panel 0 is worked out once (32 bits: checked by
     // the entry points); rows beyond M read row M - 1, whose results are never stored.
@@ -155,18 +175,15 @@ __device__ __forceinline__ void gemm_small_body(const unsigned char* __restrict_
                 if (k0 + xq < k_dim) xv[i] = *(const uint4*)(x + (size_t)(xoff[i] + (unsigned)k0));
             }
         }
-        uint4 sc, cd[CROW_STEPS];
-        const uint4* t = wt + (size_t)p * (CROW_TILE_BYTES / 16);
-        sc = stream_load(t);
-#pragma unroll
-        for (int s = 0; s < CROW_STEPS; s++) cd[s] = stream_load(t + 64 * (s + 1));
+        PanelRegs pr;
+        load_panel(w, rt, strips, panels, p, lane, pr);
 #pragma unroll
         for (int i = 0; i < 8 * TBK; i++) {
             const int c = i * 64 + lane, r = c >> 5, q = c & 31;
             *(uint4*)(xs + r * CROW_GEMM_XS_STRIDE + q * 8) = xv[i];
         }
         __builtin_amdgcn_wave_barrier();
-        gemm_panel<TBK>(sc, cd, xs_lane, acc);
+        gemm_panel<TBK>(pr, xs_lane, acc);
         __builtin_amdgcn_wave_barrier();  // the tile is read before the next stage overwrites it
     }
     // the other waves -> wave 0 through LDS (each wave's own region is free now), added in wave order
@@ -234,13 +251,8 @@ __device__ __forceinline__ void gemm_pipe_body(const unsigned char* __restrict__
 #pragma unroll
         for (int j = 0; j < 4; j++) acc[tb][j] = f32x4{0.f, 0.f, 0.f, 0.f};
 
-    const uint4* wt = (const uint4*)(w + (size_t)(has_rows ? rt : 0) * panels * CROW_TILE_BYTES) + lane;
-    auto load_w = [&](int p, uint4& sc, uint4 (&cd)[CROW_STEPS]) {
-        const uint4* t = wt + (size_t)p * (CROW_TILE_BYTES / 16);
-        sc = stream_load(t);
-#pragma unroll
-        for (int s = 0; s < CROW_STEPS; s++) cd[s] = stream_load(t + 64 * (s + 1));
-    };
+    const int strips = (rows + CROW_STRIP_ROWS - 1) / CROW_STRIP_ROWS;
+    auto load_w = [&](int p, PanelRegs& r) { load_panel(w, has_rows ? rt : 0, strips, panels, p, lane, r); };
     // chunk c = i * 256 + thread: token row c / 32, 8 columns from 8 (c % 32).  The element offset of the chunk in panel 0 is
     // worked out once; rows beyond M read row M - 1 (their results are never stored), so whole panels load without masks.
     const int xq = ((int)threadIdx.x & 31) * 8;
@@ -272,9 +284,10 @@ __device__ __forceinline__ void gemm_pipe_body(const unsigned char* __restrict__
     };
     const int lane_off = (lane & 15) * CROW_GEMM_XS_STRIDE + (lane >> 4) * 8;
 
-    uint4 sc[2], cd[2][CROW_STEPS], xv[XCH];
+    PanelRegs pr[2];
+    uint4 xv[XCH];
     load_x(0, xv);
-    load_w(0, sc[0], cd[0]);
+    load_w(0, pr[0]);
     store_x(xs2, xv);
     __syncthreads();
     // two panels per trip so that the register sets swap roles without copies
@@ -286,9 +299,9 @@ __device__ __forceinline__ void gemm_pipe_body(const unsigned char* __restrict__
                 const bool more = pp + 1 < panels;
                 if (more) {
                     load_x(pp + 1, xv);
-                    load_w(pp + 1, sc[h ^ 1], cd[h ^ 1]);
+                    load_w(pp + 1, pr[h ^ 1]);
                 }
-                gemm_panel<TBK>(sc[h], cd[h], xs2 + h * XBUF + lane_off, acc);
+                gemm_panel<TBK>(pr[h], xs2 + h * XBUF + lane_off, acc);
                 if (more) store_x(xs2 + (h ^ 1) * XBUF, xv);
                 __syncthreads();  // the other buffer is written, and this one read, by every wave
             }
@@ -303,14 +316,15 @@ __device__ __forceinline__ void gemm_pipe_body(const unsigned char* __restrict__
 // Y[M][rows] f32 = X[M][k_dim] bf16 times the tiled NVFP4 tensor, times gs.  The argument list is
 // gemm_fp4_dense's (engine/src/kernels.rs:533-541) without the quantised-activation buffer: x is bf16.
 // grid (ceil(row_tiles / 4), ceil(M / MT)), block 256, MT = 64 / 128 for the two general entry points.
-// token blocks of 32: grid (row_tiles, ceil(M / 32)), block 256 (any multiple of 64 up to 512 works: the waves deal the panels)
+// token blocks of 32: grid (row_tiles, ceil(M / 32)), block 256 (or fewer whole waves: the waves deal the panels)
 extern "C" __global__ void __launch_bounds__(512) gemm_nvfp4_bf16_m32(const unsigned char* __restrict__ w, const unsigned short* __restrict__ x,
                                                                          const float* __restrict__ gs_ptr, float* __restrict__ y,
                                                                          const int* __restrict__ k_dim_p, const int* __restrict__ rows_p,
                                                                          const int* __restrict__ m_p) {
     __shared__ __attribute__((aligned(16))) __bf16 xs[4 * 32 * CROW_GEMM_XS_STRIDE];
     const int m = *m_p;
-    if (m < 1 || (unsigned long long)m * (unsigned long long)*k_dim_p > 0xffffffffull) {  // X is addressed with 32-bit element offsets
+    // four waves stage and reduce in the static LDS below; X is addressed with 32-bit element offsets
+    if (m < 1 || block_threads() > 256 || (unsigned long long)m * (unsigned long long)*k_dim_p > 0xffffffffull) {
         if (threadIdx.x == 0) atomicOr(crow::g_ws.status, crow::STATUS_BAD_SHAPE);
         return;
     }

@@ -7,37 +7,34 @@ using namespace crow;
 #define CROW_STATUS_BAD_SCALE_BYTE 8u
 
 // ------------------------------------------------------------------ container <-> tiled
-// One 64-thread block per tile (blockIdx.x = panel, blockIdx.y = row tile); thread l moves tile row l.
-// Load-time work: neither the strided 36-byte reads nor the scattered 4-byte tile writes are
-// coalesced, and they need not be.
+// One 64-thread block per group (blockIdx.x = group, blockIdx.y = strip); thread l moves the 36-byte container block
+// (strip row l % 16, block l / 16 of the group's four).  Load-time work: neither the strided 36-byte reads nor the
+// scattered 4-byte writes are coalesced, and they need not be.
 extern "C" __global__ void __launch_bounds__(64) repack_nvfp4(const unsigned char* __restrict__ src, unsigned char* __restrict__ dst,
                                                               const int* __restrict__ rows_p, const int* __restrict__ k_dim_p) {
     const int rows = *rows_p, k = *k_dim_p;
-    const int panels = (k + CROW_PANEL_COLS - 1) / CROW_PANEL_COLS, bpr = k / CROW_BLOCK_VALUES;
-    const int p = (int)blockIdx.x, rt = (int)blockIdx.y, lane = lane_id();
-    const int row = rt * CROW_TILE_ROWS + lane;
-    unsigned char* tile = dst + ((size_t)rt * panels + p) * CROW_TILE_BYTES;
+    const int groups = (k + CROW_GROUP_COLS - 1) / CROW_GROUP_COLS, bpr = k / CROW_BLOCK_VALUES;
+    const int gi = (int)blockIdx.x, strip = (int)blockIdx.y, lane = lane_id();
+    const int r = lane & 15, b = lane >> 4;
+    const int row = strip * CROW_STRIP_ROWS + r, blk = gi * 4 + b;
+    unsigned char* grp = dst + ((size_t)strip * groups + gi) * CROW_GROUP_BYTES;
+    unsigned q[9] = {0, 0, 0, 0, 0, 0, 0, 0, 0};
+    if (row < rows && blk < bpr) {
+        const unsigned* sq = (const unsigned*)(src + ((size_t)row * bpr + blk) * CROW_BLOCK_BYTES);
+#pragma unroll
+        for (int i = 0; i < 9; i++) q[i] = sq[i];
+    }
     bool bad = false;
 #pragma unroll
-    for (int b = 0; b < 4; b++) {
-        const int blk = p * 4 + b;
-        unsigned q[9] = {0, 0, 0, 0, 0, 0, 0, 0, 0};
-        if (row < rows && blk < bpr) {
-            const unsigned* sq = (const unsigned*)(src + ((size_t)row * bpr + blk) * CROW_BLOCK_BYTES);
-#pragma unroll
-            for (int i = 0; i < 9; i++) q[i] = sq[i];
-        }
-#pragma unroll
-        for (int i = 0; i < 4; i++) {
-            unsigned v = (q[0] >> (8 * i)) & 0xFFu;
-            if (v == 0xFFu) bad = true;
-            v &= 0x7Fu;
-            if (v == 0x7Fu) v = 0x7Eu;
-            tile[crow_tile_scale_offset((unsigned)lane, (unsigned)(4 * b + i))] = (unsigned char)v;
-        }
-#pragma unroll
-        for (int wd = 0; wd < 8; wd++) *(unsigned*)(tile + crow_tile_code_offset((unsigned)lane, (unsigned)(8 * b + wd))) = q[1 + wd];
+    for (int i = 0; i < 4; i++) {
+        unsigned v = (q[0] >> (8 * i)) & 0xFFu;
+        if (v == 0xFFu) bad = true;
+        v &= 0x7Fu;
+        if (v == 0x7Fu) v = 0x7Eu;
+        grp[crow_group_scale_offset((unsigned)r, (unsigned)(4 * b + i))] = (unsigned char)v;
     }
+#pragma unroll
+    for (int wd = 0; wd < 8; wd++) *(unsigned*)(grp + crow_group_code_offset((unsigned)r, (unsigned)(8 * b + wd))) = q[1 + wd];
     if (bad) atomicOr(g_ws.status, CROW_STATUS_BAD_SCALE_BYTE);
 }
 
@@ -46,47 +43,43 @@ extern "C" __global__ void __launch_bounds__(64) repack_nvfp4(const unsigned cha
 extern "C" __global__ void __launch_bounds__(64) unpack_nvfp4(const unsigned char* __restrict__ src, unsigned char* __restrict__ dst,
                                                               const int* __restrict__ rows_p, const int* __restrict__ k_dim_p) {
     const int rows = *rows_p, k = *k_dim_p;
-    const int panels = (k + CROW_PANEL_COLS - 1) / CROW_PANEL_COLS, bpr = k / CROW_BLOCK_VALUES;
-    const int p = (int)blockIdx.x, rt = (int)blockIdx.y, lane = lane_id();
-    const int row = rt * CROW_TILE_ROWS + lane;
-    if (row >= rows) return;
-    const unsigned char* tile = src + ((size_t)rt * panels + p) * CROW_TILE_BYTES;
+    const int groups = (k + CROW_GROUP_COLS - 1) / CROW_GROUP_COLS, bpr = k / CROW_BLOCK_VALUES;
+    const int gi = (int)blockIdx.x, strip = (int)blockIdx.y, lane = lane_id();
+    const int r = lane & 15, b = lane >> 4;
+    const int row = strip * CROW_STRIP_ROWS + r, blk = gi * 4 + b;
+    if (row >= rows || blk >= bpr) return;
+    const unsigned char* grp = src + ((size_t)strip * groups + gi) * CROW_GROUP_BYTES;
+    unsigned* q = (unsigned*)(dst + ((size_t)row * bpr + blk) * CROW_BLOCK_BYTES);
+    unsigned s4 = 0;
 #pragma unroll
-    for (int b = 0; b < 4; b++) {
-        const int blk = p * 4 + b;
-        if (blk < bpr) {
-            unsigned* q = (unsigned*)(dst + ((size_t)row * bpr + blk) * CROW_BLOCK_BYTES);
-            unsigned s4 = 0;
+    for (int i = 0; i < 4; i++) s4 |= (unsigned)grp[crow_group_scale_offset((unsigned)r, (unsigned)(4 * b + i))] << (8 * i);
+    q[0] = s4;
 #pragma unroll
-            for (int i = 0; i < 4; i++) s4 |= (unsigned)tile[crow_tile_scale_offset((unsigned)lane, (unsigned)(4 * b + i))] << (8 * i);
-            q[0] = s4;
-#pragma unroll
-            for (int wd = 0; wd < 8; wd++) q[1 + wd] = *(const unsigned*)(tile + crow_tile_code_offset((unsigned)lane, (unsigned)(8 * b + wd)));
-        }
-    }
+    for (int wd = 0; wd < 8; wd++) q[1 + wd] = *(const unsigned*)(grp + crow_group_code_offset((unsigned)r, (unsigned)(8 * b + wd)));
 }
 
 // Dequantise a tiled tensor to f32 [rows][k_dim]: w = e2m1(code) * f32(ue4m3(scale) * gs), the two
 // roundings of the reference decode in that order (engine/src/cnq.rs:1298-1308 with the scale rule of
-// cpu_nvfp4.rs:98-105 already applied by the repacker).  Same grid as repack_nvfp4.
+// cpu_nvfp4.rs:98-105 already applied by the repacker).  Same grid as repack_nvfp4: thread l decodes the 64 values of
+// strip row l % 16, container block l / 16 of the group.
 extern "C" __global__ void __launch_bounds__(64) dequant_nvfp4_tiled(const unsigned char* __restrict__ w, const float* __restrict__ gs_ptr,
                                                                      float* __restrict__ out, const int* __restrict__ rows_p,
                                                                      const int* __restrict__ k_dim_p) {
     const int rows = *rows_p, k = *k_dim_p;
-    const int panels = (k + CROW_PANEL_COLS - 1) / CROW_PANEL_COLS;
-    const int p = (int)blockIdx.x, rt = (int)blockIdx.y, lane = lane_id();
-    const int row = rt * CROW_TILE_ROWS + lane;
-    if (row >= rows) return;
+    const int groups = (k + CROW_GROUP_COLS - 1) / CROW_GROUP_COLS;
+    const int gi = (int)blockIdx.x, strip = (int)blockIdx.y, lane = lane_id();
+    const int r = lane & 15, b = lane >> 4;
+    const int row = strip * CROW_STRIP_ROWS + r, col_b = gi * CROW_GROUP_COLS + b * CROW_BLOCK_VALUES;
+    if (row >= rows || col_b >= k) return;
     const float gs = gs_ptr[0];
-    const unsigned char* tile = w + ((size_t)rt * panels + p) * CROW_TILE_BYTES;
-    for (int sb = 0; sb < 16; sb++) {
-        const int col0 = p * CROW_PANEL_COLS + sb * 16;
-        if (col0 >= k) break;
-        const unsigned byte = tile[crow_tile_scale_offset((unsigned)lane, (unsigned)sb)];
+    const unsigned char* grp = w + ((size_t)strip * groups + gi) * CROW_GROUP_BYTES;
+    for (int i = 0; i < 4; i++) {
+        const int sb = 4 * b + i;
+        const unsigned byte = grp[crow_group_scale_offset((unsigned)r, (unsigned)sb)];
         const float sf = __builtin_amdgcn_cvt_f32_fp8((int)byte, 0) * gs;
-        float* o = out + (size_t)row * k + col0;
+        float* o = out + (size_t)row * k + col_b + 16 * i;
         for (int d = 0; d < 2; d++) {
-            const unsigned wd = *(const unsigned*)(tile + crow_tile_code_offset((unsigned)lane, (unsigned)(2 * sb + d)));
+            const unsigned wd = *(const unsigned*)(grp + crow_group_code_offset((unsigned)r, (unsigned)(2 * sb + d)));
             for (int j = 0; j < 8; j++) {
                 const unsigned nib = (wd >> (4 * j)) & 0xFu;
                 const f32x2 v = __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(nib, 1.0f, 0);
@@ -289,14 +282,15 @@ extern "C" __global__ void __launch_bounds__(64) router_top10(const float* __res
 
 // Router and routed gate|up + SwiGLU in ONE launch: every block works out its token's routing itself (wave 0; the
 // logits row is 1 KB) instead of reading pointers a router launch left behind, which takes a launch (4 us back to back) off
-// the layer.  grid (1, inter / 64, T K), block 1024 as moe_gate_up_silu.  Block (row tile 0, pick 0) of each token writes
+// the layer.  grid (inter / 16, 1, T K), block as moe_gate_up_silu.  Block (strip 0, pick 0) of each token writes
 // ids, wts and dn_ptrs for moe_down_combine.  table[2 e] / table[2 e + 1] = gate|up / down slab of expert e.
 extern "C" __global__ void __launch_bounds__(1024) moe_route_gate_up_silu(const float* __restrict__ logits, const unsigned long long* __restrict__ table,
                                                                           const float* __restrict__ x, const float* __restrict__ gs_ptr,
                                                                           float* __restrict__ h, int* __restrict__ ids, float* __restrict__ wts,
                                                                           unsigned long long* __restrict__ dn_ptrs, const int* __restrict__ k_dim_p,
-                                                                          const int* __restrict__ x_stride_p, const int* __restrict__ inter_p) {
-    ENTER(logits, table, x, gs_ptr, h, ids, wts, dn_ptrs, k_dim_p, x_stride_p, inter_p);
+                                                                          const int* __restrict__ x_stride_p, const int* __restrict__ inter_p, int geo) {
+    ENTER();
+    const int pairs = geo & 0xFFFFF;
     __shared__ unsigned long long s_slab;
     const int E = g_geo.experts, K = g_geo.topk;
     if (E < 64 || E > 1024 || (E & (E - 1)) != 0 || K < 1 || K > 16 || K > E || table == nullptr) {
@@ -306,16 +300,21 @@ extern "C" __global__ void __launch_bounds__(1024) moe_route_gate_up_silu(const 
     const int combo = (int)blockIdx.z, t = combo / K, j = combo % K;
     if (threadIdx.x < 64) {  // wave 0
         int picked;
-        router_dispatch(E, logits, nullptr, ids, wts, nullptr, dn_ptrs, table, nullptr, nullptr, nullptr, K, t, blockIdx.y == 0 && j == 0, picked);
+        router_dispatch(E, logits, nullptr, ids, wts, nullptr, dn_ptrs, table, nullptr, nullptr, nullptr, K, t, blockIdx.x == 0 && j == 0, picked);
         const int e = __builtin_amdgcn_readlane(picked, j);
         if (threadIdx.x == 0) s_slab = table[2 * e];
     }
     __syncthreads();
-    const int inter = *inter_p, k = *k_dim_p;
+    const int inter = *inter_p;
     const unsigned char* w = (const unsigned char*)s_slab;
-    const size_t up_off = (size_t)(inter / CROW_TILE_ROWS) * ((k + CROW_PANEL_COLS - 1) / CROW_PANEL_COLS) * CROW_TILE_BYTES;
-    GemvArgs a{{w, w + up_off}, {gs_ptr, gs_ptr}, x + (size_t)t * *x_stride_p, 0, h + (size_t)combo * inter, 0, k, inter, 1, nullptr};
-    gemv_body<2, 1, false, EPI_SILU_GU, XRows<1, false>::value, true>(a, blockIdx.z, LDS, ws);
+    CROW_REFUSE_NULL_SLAB(w);  // a table with an empty entry: uniform over the block, after the only barrier before the body
+    if (inter % CROW_STRIP_ROWS != 0) {
+        if (threadIdx.x == 0) atomicOr(ws.status, STATUS_BAD_SHAPE);
+        return;
+    }
+    GemvArgs a = gemv_args(w, w + up_offset(inter, pairs), gs_ptr, gs_ptr, x + (size_t)t * *x_stride_p, 0, h, 0, pairs, k_dim_p, inter_p);
+    a.y_row0 = combo;
+    gemv_body<2, 1, false, EPI_SILU_GU>(a, blockIdx.z, LDS, ws);
 }
 
 // Sort the n routed combos of a batch by expert and cut them into tiles of at most four combos of one expert: the work of
@@ -468,13 +467,13 @@ extern "C" __global__ void __launch_bounds__(1024) argmax_k(const float* __restr
     }
 }
 
-// Stage 2 of the fused head: the greedy token from the per-row-tile candidates gemv_nvfp4_w_argmax left in
-// the workspace (ceil(rows / 64) of them).  grid (1), block 256.  Same total order as argmax_k.
+// Stage 2 of the fused head: the greedy token from the per-strip candidates gemv_nvfp4_w_argmax left in
+// the workspace (ceil(rows / 16) of them).  grid (1), block 256.  Same total order as argmax_k.
 extern "C" __global__ void __launch_bounds__(256) argmax_tiles(int* __restrict__ out, const int* __restrict__ rows_p) {
     __shared__ float sv[4];
     __shared__ int si[4];
     const Workspace ws = g_ws;
-    const int tiles = (*rows_p + CROW_TILE_ROWS - 1) / CROW_TILE_ROWS;
+    const int tiles = (*rows_p + CROW_STRIP_ROWS - 1) / CROW_STRIP_ROWS;
     Best b{-3.0e38f, 0};
     for (int t = (int)threadIdx.x; t < tiles && t < (int)ws.am_slots; t += 256) {
         const float v = ws.am_val[t];

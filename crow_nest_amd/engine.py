@@ -88,7 +88,7 @@ class Engine:
         if y is None:
             y = torch.empty((m, rows), dtype=torch.float32, device=self.dev)
         name = "gemv_nvfp4_wm" if x.dtype == torch.float32 else "gemv_nvfp4_wm_bf16"
-        gx, gy, gz, bx = launch_dims(name, rows, k)
+        gx, gy, gz, bx = launch_dims(name, rows, k, m)
         p = self.p
         launch_v(self.k.f(name), gx, gy, gz, bx, [w.w_ptr, x.data_ptr(), w.gs_ptr, y.data_ptr(), p.i32(k), p.i32(rows), p.i32(m)])
         return y
@@ -107,7 +107,7 @@ class Engine:
                      [mlp.gate.w_ptr, mlp.up.w_ptr, x.data_ptr(), mlp.gate.gs_ptr, mlp.up.gs_ptr, h.data_ptr(), p.i32(k), p.i32(inter)])
         else:
             name = "gemv_nvfp4_gum" if x.dtype == torch.float32 else "gemv_nvfp4_gum_bf16"
-            gx, gy, gz, bx = launch_dims(name, inter, k)
+            gx, gy, gz, bx = launch_dims(name, inter, k, t)
             launch_v(self.k.f(name), gx, gy, gz, bx,
                      [mlp.gate.w_ptr, mlp.up.w_ptr, x.data_ptr(), mlp.gate.gs_ptr, mlp.up.gs_ptr, h.data_ptr(), p.i32(k), p.i32(inter), p.i32(t)])
         return h
@@ -142,9 +142,18 @@ class Engine:
         return out
 
     # ------------------------------------------------------------------ routed experts
+    def _check_moe(self, moe: MoeW) -> None:
+        """The routed kernels index the table with expert ids of the kernel geometry: a table (or slab tensor) with fewer
+        experts would be read past its end.  Refused here, before any launch (the C++ mirror does the same)."""
+        e = self.geo.experts
+        if moe.gate_up.experts != e or moe.down.experts != e or moe.table.shape[0] != e:
+            raise ValueError(f"moe: the geometry has {e} experts, the weights {moe.gate_up.experts} / {moe.down.experts}, the table {moe.table.shape[0]}")
+
     def router(self, logits: torch.Tensor, moe: MoeW | None = None):
         t, e = logits.shape
         k = self.geo.topk
+        if moe is not None:
+            self._check_moe(moe)
         assert e == self.geo.experts and logits.dtype == torch.float32 and logits.is_contiguous()
         ids = torch.empty((t, k), dtype=torch.int32, device=self.dev)
         wts = torch.empty((t, k), dtype=torch.float32, device=self.dev)
@@ -171,6 +180,7 @@ class Engine:
         moe_down_grouped) and acc_combo.  The grouping idea of the reference's prefill path (kernels.rs:3322-3384)."""
         t, hdim = x.shape
         inter, topk, experts = self.geo.inter, self.geo.topk, self.geo.experts
+        self._check_moe(moe)
         assert hdim == self.geo.hidden and moe.gate_up.rows == 2 * inter and moe.down.rows == hdim
         p = self.p
         ids, wts, _, _ = self.router(logits, moe)
@@ -201,6 +211,7 @@ class Engine:
         takes the router into the gate|up launch (moe_route_gate_up_silu + moe_down_combine: two launches)."""
         t, hdim = x.shape
         inter, topk = self.geo.inter, self.geo.topk
+        self._check_moe(moe)
         assert hdim == self.geo.hidden and moe.gate_up.rows == 2 * inter and moe.down.rows == hdim
         p = self.p
         combos = t * topk

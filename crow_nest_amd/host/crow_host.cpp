@@ -201,7 +201,7 @@ void Engine::dense_proj(const Fp4& w, int t, uint64_t x, uint64_t y, bool x_bf16
 void Engine::proj_m(const Fp4& w, int m, uint64_t x, uint64_t y, bool x_bf16) {
     if (m < 1 || m > NVFP4_MMAX) throw Panic("proj_m: M = " + std::to_string(m) + " is outside 1..=" + std::to_string(NVFP4_MMAX));
     const char* name = x_bf16 ? "gemv_nvfp4_wm_bf16" : "gemv_nvfp4_wm";
-    launch_v(k.f(name), launch_dims(name, (uint32_t)w.rows, (uint32_t)w.cols), {w.w.ptr(), x, w.gs.ptr(), y, p.i32(w.cols), p.i32(w.rows), p.i32(m)});
+    launch_v(k.f(name), launch_dims(name, (uint32_t)w.rows, (uint32_t)w.cols, (uint32_t)m), {w.w.ptr(), x, w.gs.ptr(), y, p.i32(w.cols), p.i32(w.rows), p.i32(m)});
 }
 void Engine::gate_up(const MlpW& mlp, int t, uint64_t x, uint64_t h, bool x_bf16) {
     const int inter = mlp.gate.rows, kd = mlp.gate.cols;
@@ -213,7 +213,7 @@ void Engine::gate_up(const MlpW& mlp, int t, uint64_t x, uint64_t h, bool x_bf16
                  {mlp.gate.w.ptr(), mlp.up.w.ptr(), x, mlp.gate.gs.ptr(), mlp.up.gs.ptr(), h, p.i32(kd), p.i32(inter)});
     } else {
         const char* name = x_bf16 ? "gemv_nvfp4_gum_bf16" : "gemv_nvfp4_gum";
-        launch_v(k.f(name), launch_dims(name, (uint32_t)inter, (uint32_t)kd),
+        launch_v(k.f(name), launch_dims(name, (uint32_t)inter, (uint32_t)kd, (uint32_t)t),
                  {mlp.gate.w.ptr(), mlp.up.w.ptr(), x, mlp.gate.gs.ptr(), mlp.up.gs.ptr(), h, p.i32(kd), p.i32(inter), p.i32(t)});
     }
 }

@@ -45,7 +45,11 @@ enum crow_status {
     CROW_ERR_GEO = -8
 };
 
-/* launch geometry chosen by the library for a kernel and a problem (wave64 shapes stay out of the caller) */
+/* launch geometry chosen by the library for a kernel and a problem (wave64 shapes stay out of the caller).  The four words
+ * are to be handed to crow_hip_launch unchanged.  For the NVFP4 GEMV family `gy` is not a grid extent: it carries the problem
+ * (bits 0..19 = k_dim / 64, bits 20..23 = activation rows of the last token group or 0, bits 24..31 = column slices per
+ * strip); crow_hip_launch launches (gx, slices, gz) blocks and hands the low 24 bits to the kernel by value, so that a wave
+ * can address its weights before the words behind k_dim_p / m_p have arrived from memory. */
 typedef struct crow_dims {
     uint32_t gx, gy, gz, bx;
 } crow_dims;
@@ -71,17 +75,17 @@ int crow_hip_set_geo(int experts, int topk, int hidden, int inter);
 /* ---- launch ---- */
 int crow_hip_launch(crow_fn_t f, uint32_t gx, uint32_t gy, uint32_t gz, uint32_t bx, const uint64_t* vals,
                     uint32_t n_vals, void* stream);
-/* grid/block for `name` on a [rows, k_dim] tensor with `z` token rows (batched kernels) or combos
- * (routed kernels); 1 otherwise.  The choice depends on (rows, k_dim) only, never on z. */
+/* grid/block for `name` on a [rows, k_dim] tensor with `z` token rows (batched and verify kernels: the value *t_p / *m_p
+ * will hold) or combos (routed kernels); 1 otherwise.  The split of the work depends on (rows, k_dim) only, never on z. */
 int crow_hip_launch_dims(const char* name, uint32_t rows, uint32_t k_dim, uint32_t z, crow_dims* out);
-/* the same with the GEMV split forced: `s` column slices per row tile (blocks that hand their partial sums over through the
- * workspace) and `w` waves per block and tensor; 0 = the library's choice.  Every GEMV kernel is correct for every split:
+/* the same with the GEMV split forced: `s` column slices per 16-row strip (blocks that hand their partial sums over through
+ * the workspace) and `w` waves per block and tensor; 0 = the library's choice.  Every GEMV kernel is correct for every split:
  * this is for tuning and for tests.  Other kernels ignore s and w. */
 int crow_hip_launch_dims_split(const char* name, uint32_t rows, uint32_t k_dim, uint32_t z, uint32_t s, uint32_t w, crow_dims* out);
 /* the GEMM entry point (a name of the kernel table) that serves `m` token rows fastest on a tensor of `rows` rows: the
  * choice depends on how the blocks of each tiling fall on this device's compute units */
 const char* crow_hip_gemm_kernel(uint32_t rows, uint32_t m);
-/* reads and clears the device status word (synchronises the current stream): CROW_OK or CROW_ERR_* */
+/* reads and clears the device status word (waits for the whole device first: every stream): CROW_OK or CROW_ERR_* */
 int crow_hip_status(void);
 int crow_hip_reset_workspace(void);
 
@@ -128,9 +132,10 @@ int crow_hip_time_graph(void* graph_exec, void* stream, uint32_t iters, float* u
 /* ---- load-time repack (the one call the reference does not have) ---- */
 size_t crow_hip_container_bytes(uint32_t rows, uint32_t cols);
 size_t crow_hip_tiled_bytes(uint32_t rows, uint32_t cols);
-/* where the repacker puts things inside a 9216-byte tile (host arithmetic, no device needed): the byte offset of the code
- * dword of tile row `row` (0..63), tile columns 8 wp .. 8 wp + 7 (wp 0..31), and of the scale byte of tile row `row`,
- * 16-column sub-block sb (0..15).  UINT32_MAX for an argument out of range. */
+/* where the repacker puts things inside a 2304-byte group of 16 rows x 256 columns (host arithmetic, no device needed): the
+ * byte offset of the code dword of strip row `row` (0..15), group columns 8 wp .. 8 wp + 7 (wp 0..31), and of the scale byte
+ * of strip row `row`, 16-column sub-block sb (0..15).  Group (strip, gi) of a tensor starts at
+ * (strip * ceil(cols / 256) + gi) * 2304.  UINT32_MAX for an argument out of range. */
 uint32_t crow_hip_tile_code_offset(uint32_t row, uint32_t wp);
 uint32_t crow_hip_tile_scale_offset(uint32_t row, uint32_t sb);
 /* src_dev: container bytes [rows][cols/64][36] already on the device; dst_dev: crow_hip_tiled_bytes.

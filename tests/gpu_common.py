@@ -10,24 +10,58 @@ from refgen import normal_f32
 TOL = 1e-3  # north star: GEMV outputs within max relative error 1e-3 of the CPU path
 
 
-FLOOR = 1e-2  # outputs below 1 % of their row's rms are compared absolutely (1e-5 rms), see rel_err
+FLOOR = 1e-3  # outputs below 0.1 % of their row's rms are compared absolutely (1e-6 rms), see rel_err
 
 
-def rel_err(y: np.ndarray, ref: np.ndarray) -> float:
-    """max_i |y_i - ref_i| / max(|ref_i|, FLOOR * rms(ref)) per output row, worst row.
+# Two products in a row (gate / up + SwiGLU, then down; a routed layer): the second product's inputs already differ from the
+# CPU path's by the first one's summation order, and that difference - about 1e-6 of the row's rms after K ~ 3000 terms - is
+# carried to every output, also to those that cancel to almost nothing.  Such end-to-end comparisons floor at 1 % of the rms;
+# each single product inside them is held to FLOOR on its own (against the CPU path on the device's own inputs) and to the
+# gamma bound.  Measured on the 1024 -> 2816 -> 1024 FFN at four rows: 1.2e-3 at the 0.1 % floor (one near-zero output),
+# 1.2e-4 at the 1 % floor; the down product alone on the device's own h: below 1e-4 at the 0.1 % floor.
+FLOOR_CHAINED = 1e-2
+
+
+def floor_of(n_outputs: int) -> float:
+    """The floor for a comparison of n_outputs values at once.  Either path's f32 summation of K ~ 5000 terms leaves an
+    absolute error of about 2.5e-7 of the row's rms per output, so the largest of some ten thousand of them reaches 1e-6 rms -
+    which IS 1e-3 of the 0.1 % floor: beyond 2^14 outputs the plain floor tests the tail of that noise, not the kernel
+    (measured at K = 5120: 1.03e-3 on one of 38,400 outputs of a 200-token GEMM, 1.15e-3 on one of 32,768 of a 128-token one;
+    their gamma ratios are below 0.02).  Such comparisons floor at 1 % of the rms and hold the floorless gamma bound on
+    sampled rows as well.  (The one-token tests, the benchmark's config 0 with its 17,408 outputs included, stay on FLOOR.)"""
+    return FLOOR if n_outputs <= (1 << 14) else FLOOR_CHAINED
+
+
+def rel_err(y: np.ndarray, ref: np.ndarray, floor: float = FLOOR) -> float:
+    """max_i |y_i - ref_i| / max(|ref_i|, floor * rms(ref)) per output row, worst row.
 
     A dot product of K ~ 5000 terms summed in f32 carries an absolute error of about 1e-6 of the
     row's rms whatever the order (the CPU path against f64 shows the same); an output that happens
     to cancel to almost nothing therefore has no meaningful RELATIVE error, and is held to
-    TOL * FLOOR * rms instead.  Every GEMV test additionally holds the reference's own acceptance
-    bound gamma(K/16 + 10) * sum|w x| against an f64 evaluation (gamma_ratio), which has no floor."""
+    TOL * FLOOR * rms instead.  The GEMV tests additionally hold the reference's own acceptance
+    bound gamma(K/16 + 10) * sum|w x| against an f64 evaluation (gamma_ratio), which has no floor,
+    on all rows or on a sample of them."""
     y = np.asarray(y, np.float64).reshape(ref.shape)
     r = np.asarray(ref, np.float64)
     if r.ndim == 1:
         r, y = r[None], y[None]
     rms = np.sqrt((r * r).mean(axis=1, keepdims=True))
-    den = np.maximum(np.abs(r), FLOOR * np.maximum(rms, 1e-30))
+    den = np.maximum(np.abs(r), floor * np.maximum(rms, 1e-30))
     return float(np.max(np.abs(y - r) / den))
+
+
+def rel_l2(y: np.ndarray, ref: np.ndarray) -> float:
+    """||y - ref|| / ||ref|| over everything (the reference's GPU gate holds 1e-4: bin/mma_gate.rs:315)."""
+    y = np.asarray(y, np.float64).reshape(-1)
+    r = np.asarray(ref, np.float64).reshape(-1)
+    return float(np.linalg.norm(y - r) / max(np.linalg.norm(r), 1e-300))
+
+
+def gamma_rows(y, w, r0, n, cols, gs, x) -> float:
+    """gamma_ratio on rows r0 .. r0 + n - 1 of a container tensor `w` with `cols` columns; y = the outputs of those rows
+    ([n] or [tokens][n])."""
+    rb = cols // 64 * 36
+    return gamma_ratio(y, w[r0 * rb:(r0 + n) * rb], n, cols, gs, x)
 
 
 def gamma_ratio(y, w, rows, cols, gs, x) -> float:

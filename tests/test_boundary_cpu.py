@@ -42,7 +42,8 @@ def test_kernel_table_names_without_a_device():
     assert lib.crow_hip_get_function(b"no_such_kernel", C.byref(out)) == -2  # CROW_ERR_KERNEL_MISSING
     assert b"kernel missing" in lib.crow_hip_error_string(-2)
     assert lib.crow_hip_tiled_bytes(17408, 5120) == 17408 * 5120 // 64 * 36 == lib.crow_hip_container_bytes(17408, 5120)
-    assert lib.crow_hip_tiled_bytes(1, 64) == 9216  # one padded tile
+    assert lib.crow_hip_tiled_bytes(1, 64) == 2304  # one padded group: 16 rows x 256 columns
+    assert lib.crow_hip_tiled_bytes(151936, 5120) == lib.crow_hip_container_bytes(151936, 5120)
 
 
 def test_kernel_header_is_the_library_table():
@@ -77,8 +78,14 @@ def test_launch_dims_depend_on_the_matrix_only():
     d1, d4 = L.Dims(), L.Dims()
     assert lib.crow_hip_launch_dims(b"gemv_nvfp4_w", 17408, 5120, 1, C.byref(d1)) == 0
     assert lib.crow_hip_launch_dims(b"gemv_nvfp4_wm", 17408, 5120, 1, C.byref(d4)) == 0
-    assert (d1.gx, d1.gy, d1.gz, d1.bx) == (d4.gx, d4.gy, d4.gz, d4.bx)  # verify rows == decode row, bit for bit
-    assert d1.gy == 272 and d1.bx % 64 == 0
+    # verify rows == decode row, bit for bit: same grid, same block, same K word and slice count; only the row hint differs
+    assert (d1.gx, d1.gy & 0xFF0FFFFF, d1.gz, d1.bx) == (d4.gx, d4.gy & 0xFF0FFFFF, d4.gz, d4.bx)
+    assert d1.gx == 17408 // 16 and d1.bx == 5 * 64 and d1.gy == (5120 // 64) | (1 << 24)  # one block per strip, whole K inside it
+    assert (d4.gy >> 20) & 0xF == 1
+    assert lib.crow_hip_launch_dims(b"gemv_nvfp4_w", 5120, 17408, 1, C.byref(d1)) == 0
+    assert d1.gy >> 24 > 1 and d1.gy & 0xFFFFF == 17408 // 64  # a strip of 68 groups is cut into slices
+    assert lib.crow_hip_launch_dims(b"gemv_nvfp4_gu_bf16", 17408, 5120, 1, C.byref(d1)) == 0
+    assert d1.bx == 2 * 5 * 64 and d1.gy >> 24 == 1
     assert lib.crow_hip_launch_dims(b"gemv_nvfp4_w", 8, 96, 1, C.byref(d1)) == -7  # 96 columns: not whole blocks
 
 
@@ -110,28 +117,27 @@ def test_product_does_not_import_the_oracle():
                 assert "oracle" not in text.lower(), (dirpath, f)
 
 
-def test_tile_layout_is_a_bijection_and_matches_the_matrix_operand_shape():
-    """Every byte of a 9216-byte tile is owned by exactly one (row, column) item, and the placement is the one the kernels
-    assume: a lane's dword d of code segment s is row 16 d + lane % 16, columns 32 s + 8 (lane / 16) .. + 7; a lane's scale byte
-    8 jp + s is row 16 (2 jp + (g & 1)) + n, sub-block 2 s + (g >> 1)."""
+def test_group_layout_is_a_bijection_and_matches_the_matrix_operand_shape():
+    """Every byte of a 2304-byte group (16 rows x 256 columns) is owned by exactly one (row, column) item, and the placement is
+    the one the kernels assume: a lane's dword d of code half h is strip row lane % 16, pair 2 h + d / 2, segment d % 2, columns
+    8 (lane / 16) .. + 7 of that segment; a lane's scale byte jj is row lane % 16, pair jj, segment g & 1, half g >> 1."""
     lib = L.lib()
     seen = set()
-    for row in range(64):
+    for row in range(16):
         for wp in range(32):
             o = lib.crow_hip_tile_code_offset(row, wp)
-            s_, g = wp >> 2, wp & 3
-            lane, d = 16 * g + (row & 15), row >> 4
-            assert o == 1024 * (s_ + 1) + 16 * lane + 4 * d and o % 4 == 0
+            pair, seg, g = wp >> 3, (wp >> 2) & 1, wp & 3
+            lane, h, d = 16 * g + row, pair >> 1, 2 * (pair & 1) + seg
+            assert o == 256 + 1024 * h + 16 * lane + 4 * d and o % 4 == 0
             for b in range(4):
                 assert o + b not in seen
                 seen.add(o + b)
         for sb in range(16):
             o = lib.crow_hip_tile_scale_offset(row, sb)
-            j, n = row >> 4, row & 15
-            g, jp, s_ = 2 * (sb & 1) + (j & 1), j >> 1, sb >> 1
-            assert o == 16 * (16 * g + n) + 8 * jp + s_ and o < 1024
+            pair, seg, half = sb >> 2, (sb >> 1) & 1, sb & 1
+            g = 2 * half + seg
+            assert o == 4 * (16 * g + row) + pair and o < 256
             assert o not in seen
             seen.add(o)
-    assert seen == set(range(9216))
-    assert lib.crow_hip_tile_code_offset(64, 0) == 0xFFFFFFFF and lib.crow_hip_tile_scale_offset(0, 16) == 0xFFFFFFFF
-
+    assert seen == set(range(2304))
+    assert lib.crow_hip_tile_code_offset(16, 0) == 0xFFFFFFFF and lib.crow_hip_tile_scale_offset(0, 16) == 0xFFFFFFFF

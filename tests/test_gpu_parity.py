@@ -1,15 +1,16 @@
 """GPU parity: the HIP path (through the C ABI, via the host mirror) against the CPU oracle.
 
 Bars: dequantised weights bit-exact; integer / index results bit-exact; GEMV outputs within
-max relative error 1e-3 of the CPU path (TOL; the denominator floors at 1 % of the row's rms so that
+max relative error 1e-3 of the CPU path (TOL; the denominator floors at 0.1 % of the row's rms so that
 an output that cancels to ~0 does not divide by nothing - see gpu_common.rel_err), and additionally
-inside the reference's own fp32 bound gamma(K/16 + 10) * sum|w x| against an f64 evaluation.
+inside the reference's own fp32 bound gamma(K/16 + 10) * sum|w x| against an f64 evaluation
+(gamma_ratio; on sampled rows where the tensor is large).
 """
 import numpy as np
 import pytest
 import torch
 
-from gpu_common import TOL, gamma_ratio, quantized_normal, rel_err
+from gpu_common import FLOOR_CHAINED, TOL, floor_of, gamma_ratio, gamma_rows, quantized_normal, rel_err, rel_l2
 from oracle import oracle as orc
 from refgen import SplitMix64, normal_f32, random_nvfp4, scale_mix, synth_nvfp4
 
@@ -110,9 +111,10 @@ def test_gemv_w_against_the_cpu_path(eng, rows, cols):
     assert gamma_ratio(y, w, rows, cols, gs, x) <= 1.0
 
 
-@pytest.mark.parametrize("s,wv", [(1, 1), (1, 4), (3, 2), (5, 1), (20, 1), (2, 16)])
+@pytest.mark.parametrize("s,wv", [(1, 1), (1, 4), (1, 5), (3, 2), (5, 1), (20, 1), (2, 10), (1, 16)])
 def test_gemv_is_correct_for_every_split(eng, s, wv):
-    """Any (slices, waves) split gives an answer inside the bound; the same split gives the same bits."""
+    """Any (slices, waves) split gives an answer inside the bound; the same split gives the same bits.  (1, 1) and (1, 4) make
+    a wave walk more groups than it holds at once: the loop over register loads."""
     rows, cols = 300, 5120
     w = random_nvfp4(77, rows, cols)
     gs = 4.0e-4
@@ -122,7 +124,7 @@ def test_gemv_is_correct_for_every_split(eng, s, wv):
     f = _load(w, rows, cols, gs)
     xd, p = _dev(x), eng.p
     dims = launch_dims("gemv_nvfp4_w", rows, cols, 1, split=(s, wv))
-    assert dims[0] == s and dims[3] == 64 * wv
+    assert dims[1] >> 24 == s and dims[3] == 64 * wv and dims[1] & 0xFFFFF == cols // 64
     ys = []
     for _ in range(2):
         y = torch.empty((1, rows), dtype=torch.float32, device="cuda")
@@ -158,6 +160,7 @@ def test_ragged_shapes_drawn_at_random(eng):
         ref = orc.gemv(w, rows, cols, gs, xo)
         y = (eng.proj_m(f, m, xd) if (bf16 or m > 1) else eng.dense_proj(f, 1, xd)).cpu().numpy()
         assert rel_err(y, ref) <= TOL, case
+        assert gamma_ratio(y, w, rows, cols, gs, xo) <= 1.0, case
         h = eng.gate_up(MlpW(f, f2, f), m, xd).cpu().numpy()
         assert rel_err(h, orc.silu_mul(ref, orc.gemv(w2, rows, cols, gs2, xo))) <= TOL, case
     eng.check()
@@ -177,6 +180,7 @@ def test_split_launches_back_to_back_with_changing_inputs(eng):
     p = eng.p
     for s, wv in ((4, 4), (16, 1), (2, 8)):
         dims = launch_dims("gemv_nvfp4_w", rows, cols, 1, split=(s, wv))
+        assert dims[1] >> 24 == s
         y = torch.empty((n, rows), dtype=torch.float32, device="cuda")
         for i in range(n):
             launch_v(eng.k.f("gemv_nvfp4_w"), *dims, [f.w_ptr, xd[i].data_ptr(), f.gs_ptr, y[i].data_ptr(), p.i32(cols), p.i32(rows)])
@@ -200,6 +204,7 @@ def test_verify_rows_are_bit_identical_to_one_row_decode(eng):
         for j in range(m):
             assert np.array_equal(ym[j].view(np.uint32), one[j].view(np.uint32)), (m, j)
         assert rel_err(ym, orc.gemv(w, rows, cols, gs, x[:m])) <= TOL
+        assert gamma_ratio(ym, w, rows, cols, gs, x[:m]) <= 1.0
     eng.check()
 
 
@@ -218,7 +223,14 @@ def test_fused_gate_up_silu_and_down(eng, t):
     assert rel_err(h, h_ref) <= TOL
     y = eng.dense_ffn_w(mlp, _dev(x), t).cpu().numpy()
     y_ref = orc.ffn(wg, gs[0], wu, gs[1], wd, gs[2], H, I, x)
-    assert rel_err(y, y_ref) <= TOL
+    assert rel_err(y, y_ref, FLOOR_CHAINED) <= TOL  # two products in a row: see gpu_common.FLOOR_CHAINED
+    # each product on its own, at the plain floor and inside the bound of the reference's own gate: down on the device's own h,
+    # gate alone through proj_m
+    yd = eng.dense_proj(mlp.down, t, _dev(h)).cpu().numpy()
+    assert np.array_equal(yd.view(np.uint32), y.view(np.uint32))
+    assert rel_err(yd, orc.gemv(wd, H, I, gs[2], h)) <= TOL
+    assert gamma_ratio(yd, wd, H, I, gs[2], h) <= 1.0
+    assert gamma_ratio(eng.proj_m(mlp.gate, t, _dev(x)).cpu().numpy(), wg, I, H, gs[0], x) <= 1.0
     # bf16 activations (benchmark config 1: bf16 X): the oracle gets the exactly widened values
     xb, xw = _bf16_dev(x)
     hb = eng.gate_up(mlp, t, xb.reshape(t, H).contiguous()).cpu().numpy()
@@ -235,6 +247,63 @@ def test_batched_token_rows(eng):
     x = normal_f32(4, 1, t * cols).reshape(t, cols)
     y = eng.dense_proj(f, t, _dev(x)).cpu().numpy()
     assert rel_err(y, orc.gemv(w, rows, cols, gs, x)) <= TOL
+    eng.check()
+
+
+def test_record_kernel_entry_points_by_their_own_names(eng):
+    """gemv_fp4 (kernels.rs:118-151), gemv_fp4_b1k (:1302-1337), gemv_fp4_bs (:1022-1058, its own y stride word) and the
+    one-row bf16 twin gemv_nvfp4_w_bf16 (kernels_p2.rs:355-368), each launched through the C ABI under its own name on a
+    ragged shape, against the CPU path and inside its f32 bound."""
+    from crow_nest_amd.kernels import launch_dims, launch_v
+    rows, cols = 203, 1984  # a partial last strip, a partial last group
+    w = random_nvfp4(808, rows, cols)
+    gs = 9.0e-4
+    f = _load(w, rows, cols, gs)
+    p = eng.p
+    x = normal_f32(9, 1, 5 * cols).reshape(5, cols)
+    xd = _dev(x)
+    ref = orc.gemv(w, rows, cols, gs, x)
+    # gemv_fp4: one row
+    y = torch.full((rows,), 7.0, dtype=torch.float32, device="cuda")
+    launch_v(eng.k.f("gemv_fp4"), *launch_dims("gemv_fp4", rows, cols), [f.w_ptr, xd[2].data_ptr(), f.gs_ptr, y.data_ptr(), p.i32(cols), p.i32(rows)])
+    eng.check()
+    assert rel_err(y.cpu().numpy(), ref[2]) <= TOL and gamma_ratio(y.cpu().numpy(), w, rows, cols, gs, x[2]) <= 1.0
+    # gemv_nvfp4_w_bf16: one bf16 row
+    xb, xw = _bf16_dev(x[3])
+    y = torch.full((rows,), 7.0, dtype=torch.float32, device="cuda")
+    launch_v(eng.k.f("gemv_nvfp4_w_bf16"), *launch_dims("gemv_nvfp4_w_bf16", rows, cols), [f.w_ptr, xb.data_ptr(), f.gs_ptr, y.data_ptr(), p.i32(cols), p.i32(rows)])
+    eng.check()
+    assert rel_err(y.cpu().numpy(), orc.gemv(w, rows, cols, gs, xw)[0]) <= TOL and gamma_ratio(y.cpu().numpy(), w, rows, cols, gs, xw) <= 1.0
+    # ... and it is the M = 1 case of the verify twin, bit for bit
+    y1 = eng.proj_m(f, 1, xb.reshape(1, cols)).cpu().numpy()[0]
+    assert np.array_equal(y1.view(np.uint32), y.cpu().numpy().view(np.uint32))
+    # gemv_fp4_b1k: five token rows (a full group of four and a last group of one)
+    yb = torch.full((5, rows), 7.0, dtype=torch.float32, device="cuda")
+    launch_v(eng.k.f("gemv_fp4_b1k"), *launch_dims("gemv_fp4_b1k", rows, cols, 5), [f.w_ptr, xd.data_ptr(), f.gs_ptr, yb.data_ptr(), p.i32(cols), p.i32(rows), p.i32(5)])
+    eng.check()
+    assert rel_err(yb.cpu().numpy(), ref) <= TOL and gamma_ratio(yb.cpu().numpy(), w, rows, cols, gs, x) <= 1.0
+    # gemv_fp4_bs: seven ... here five rows into a wider buffer; the gap columns stay untouched
+    stride = rows + 37
+    ys = torch.full((5, stride), 7.0, dtype=torch.float32, device="cuda")
+    launch_v(eng.k.f("gemv_fp4_bs"), *launch_dims("gemv_fp4_bs", rows, cols, 5),
+             [f.w_ptr, xd.data_ptr(), f.gs_ptr, ys.data_ptr(), p.i32(cols), p.i32(stride), p.i32(rows), p.i32(5)])
+    eng.check()
+    got = ys.cpu().numpy()
+    assert np.array_equal(got[:, :rows].view(np.uint32), yb.cpu().numpy().view(np.uint32))  # the same bodies: the same bits
+    assert bool((got[:, rows:] == 7.0).all())
+    # a stride shorter than a row is refused, nothing written
+    from crow_nest_amd.lib import CrowHipError
+    ys.fill_(7.0)
+    launch_v(eng.k.f("gemv_fp4_bs"), *launch_dims("gemv_fp4_bs", rows, cols, 5),
+             [f.w_ptr, xd.data_ptr(), f.gs_ptr, ys.data_ptr(), p.i32(cols), p.i32(rows - 1), p.i32(rows), p.i32(5)])
+    with pytest.raises(CrowHipError) as ei:
+        eng.check()
+    assert ei.value.code == -7 and bool((ys == 7.0).all())
+    # dims made for one token count, the word behind t_p saying another: refused
+    launch_v(eng.k.f("gemv_fp4_b"), *launch_dims("gemv_fp4_b", rows, cols, 5), [f.w_ptr, xd.data_ptr(), f.gs_ptr, ys.data_ptr(), p.i32(cols), p.i32(rows), p.i32(4)])
+    with pytest.raises(CrowHipError) as ei:
+        eng.check()
+    assert ei.value.code == -7 and bool((ys == 7.0).all())
     eng.check()
 
 
@@ -359,8 +428,50 @@ def test_moe_layer_both_launch_sequences(eng, t):
         eng.check()
         assert np.array_equal(ids.cpu().numpy(), ids_ref)
         assert np.allclose(wts.cpu().numpy(), w_ref, rtol=2e-6, atol=0)
-        assert rel_err(y.cpu().numpy(), y_ref) <= TOL, fused
+        assert rel_err(y.cpu().numpy(), y_ref, FLOOR_CHAINED) <= TOL, fused  # products in a row: gpu_common.FLOOR_CHAINED
     eng.check()
+
+
+def test_routed_expert_products_inside_the_bound(eng):
+    """The two products of a routed layer on their own, per combo: gemv_fp4_ptrb on the gate|up slabs and on the down slabs
+    (kernels.rs:195-233), and the fused moe_gate_up_silu, against the CPU path on the same expert's container bytes, at the
+    plain floor and inside the f32 bound."""
+    from crow_nest_amd.engine import expert_table
+    from crow_nest_amd.kernels import launch_dims, launch_v
+    from crow_nest_amd.weights import load_expert_slabs
+    E, H, I, K = 256, 2048, 512, 8
+    gu = random_nvfp4(41, E * 2 * I, H, scale_lo=0x30, scale_hi=0x48, p7f=0)
+    dn = random_nvfp4(42, E * H, I, scale_lo=0x30, scale_hi=0x48, p7f=0)
+    gs_gu, gs_dn = 2.0e-3, 3.0e-3
+    s_gu, s_dn = load_expert_slabs(gu, E, 2 * I, H, gs_gu), load_expert_slabs(dn, E, H, I, gs_dn)
+    table = expert_table(s_gu, s_dn)
+    t = 2
+    picks = np.array([[3, 200, 17, 255, 0, 96, 41, 128], [200, 5, 6, 7, 250, 3, 64, 1]], np.int64)
+    x = (normal_f32(5, 900, t * H) * np.float32(0.1)).reshape(t, H)
+    hin = (normal_f32(5, 901, t * K * I) * np.float32(0.3)).reshape(t * K, I)
+    p = eng.p
+    gup = table[torch.from_numpy(picks.reshape(-1)).cuda(), 0].contiguous()
+    dnp = table[torch.from_numpy(picks.reshape(-1)).cuda(), 1].contiguous()
+    xd, hd = _dev(x), _dev(hin)
+    h1 = torch.empty((t * K, 2 * I), dtype=torch.float32, device="cuda")
+    launch_v(eng.k.f("gemv_fp4_ptrb"), *launch_dims("gemv_fp4_ptrb", 2 * I, H, t * K),
+             [gup.data_ptr(), xd.data_ptr(), s_gu.gs.data_ptr(), h1.data_ptr(), p.i32(H), p.i32(K), p.i32(H), p.i32(2 * I)])
+    h2 = torch.empty((t * K, I), dtype=torch.float32, device="cuda")
+    launch_v(eng.k.f("moe_gate_up_silu"), *launch_dims("moe_gate_up_silu", I, H, t * K),
+             [gup.data_ptr(), xd.data_ptr(), s_gu.gs.data_ptr(), h2.data_ptr(), p.i32(H), p.i32(K), p.i32(H), p.i32(I)])
+    eo = torch.empty((t * K, H), dtype=torch.float32, device="cuda")
+    launch_v(eng.k.f("gemv_fp4_ptrb"), *launch_dims("gemv_fp4_ptrb", H, I, t * K),
+             [dnp.data_ptr(), hd.data_ptr(), s_dn.gs.data_ptr(), eo.data_ptr(), p.i32(I), p.i32(1), p.i32(I), p.i32(H)])
+    eng.check()
+    h1n, h2n, eon = h1.cpu().numpy(), h2.cpu().numpy(), eo.cpu().numpy()
+    per_gu, per_dn = 2 * I * H // 64 * 36, H * I // 64 * 36
+    for c in range(t * K):
+        e = int(picks.reshape(-1)[c])
+        wgu, wdn = gu[e * per_gu:(e + 1) * per_gu], dn[e * per_dn:(e + 1) * per_dn]
+        r1 = orc.gemv(wgu, 2 * I, H, gs_gu, x[c // K])[0]
+        assert rel_err(h1n[c], r1) <= TOL and gamma_ratio(h1n[c], wgu, 2 * I, H, gs_gu, x[c // K]) <= 1.0, c
+        assert rel_err(h2n[c], orc.silu_mul(r1[None, :I], r1[None, I:])[0]) <= TOL, c
+        assert rel_err(eon[c], orc.gemv(wdn, H, I, gs_dn, hin[c])[0]) <= TOL and gamma_ratio(eon[c], wdn, H, I, gs_dn, hin[c]) <= 1.0, c
 
 
 def test_moe_layer_other_geometries_drawn_at_random(eng):
@@ -396,7 +507,7 @@ def test_moe_layer_other_geometries_drawn_at_random(eng):
                 eng.check()
                 assert np.array_equal(ids.cpu().numpy(), ids_ref), (case, fused)
                 assert np.allclose(wts.cpu().numpy(), w_ref, rtol=2e-6, atol=0), (case, fused)
-                assert rel_err(y.cpu().numpy(), y_ref) <= TOL, (case, fused)
+                assert rel_err(y.cpu().numpy(), y_ref, FLOOR_CHAINED) <= TOL, (case, fused)
     finally:
         eng.set_geo(keep)
     eng.check()
@@ -435,10 +546,10 @@ def test_moe_layer_grouped_by_expert(eng, t):
             want.append((e, start + q, min(4, c - q), 0))
         start += c
     assert tl.tolist() == [list(w_) for w_ in want]
-    assert rel_err(y.cpu().numpy(), y_ref) <= TOL
+    assert rel_err(y.cpu().numpy(), y_ref, FLOOR_CHAINED) <= TOL
     # the ungrouped sequence gives the same layer
     _, _, y2 = eng.moe_run(moe, _dev(x), _dev(logits), fused=True)
-    assert rel_err(y2.cpu().numpy(), y_ref) <= TOL
+    assert rel_err(y2.cpu().numpy(), y_ref, FLOOR_CHAINED) <= TOL
     eng.check()
 
 
@@ -452,9 +563,9 @@ def test_config0_full_size(eng):
     y = eng.dense_proj(f, 1, _dev(x)).cpu().numpy()[0]
     eng.check()
     ref = orc.gemv(w, rows, cols, gs, x, threads=8)[0]
-    assert rel_err(y, ref) <= TOL
-    sub = slice(0, 512)
-    assert gamma_ratio(y[sub], w[:512 * cols // 64 * 36], 512, cols, gs, x) <= 1.0
+    assert rel_err(y, ref) <= TOL and rel_l2(y, ref) <= 1e-4
+    for r0 in (0, 8704 - 256, rows - 512):
+        assert gamma_rows(y[r0:r0 + 512], w, r0, 512, cols, gs, x) <= 1.0, r0
     # dequantised weights bit-exact on a slab of the full tensor
     from crow_nest_amd.weights import dequant
     d = dequant(f)[:256].cpu().numpy().reshape(-1)
@@ -484,11 +595,26 @@ def test_config1_full_size_properties(eng):
     for t in range(T):
         h1 = eng.gate_up(mlp, 1, xb[t:t + 1].contiguous()).cpu().numpy()
         assert np.array_equal(h1.view(np.uint32)[0], h.view(np.uint32)[t]), t
+    # the two-row launch (its own bodies of the gate / up and down kernels): rows 1..2 of the four, bit for bit and against the CPU path
+    h2 = eng.gate_up(mlp, 2, xb[1:3].contiguous())
+    eng.check()
+    assert np.array_equal(h2.cpu().numpy().view(np.uint32), h.view(np.uint32)[1:3])
+    r0 = 8704 - 64
+    assert rel_err(h2.cpu().numpy()[:, r0:r0 + 128], orc.silu_mul(orc.gemv(wg[r0 * rb:(r0 + 128) * rb], 128, H, gg, xw[1:3], threads=8),
+                                                                   orc.gemv(wu[r0 * rb:(r0 + 128) * rb], 128, H, gu, xw[1:3], threads=8))) <= TOL
+    # the gate product alone (bf16 X, four rows) inside the reference's own bound on sampled rows
+    g4 = eng.proj_m(mlp.gate, T, xb).cpu().numpy()
+    for r0 in (0, I - 256):
+        assert gamma_rows(g4[:, r0:r0 + 256], wg, r0, 256, H, gg, xw) <= 1.0, r0
     y = eng.dense_proj(mlp.down, T, h4).cpu().numpy()
     eng.check()
     rbd = I // 64 * 36
     for r0 in (0, H - 256):
         assert rel_err(y[:, r0:r0 + 256], orc.gemv(wd[r0 * rbd:(r0 + 256) * rbd], 256, I, gd, h, threads=8)) <= TOL, r0
+        assert gamma_rows(y[:, r0:r0 + 256], wd, r0, 256, I, gd, h) <= 1.0, r0
+    y2 = eng.dense_proj(mlp.down, 2, h2).cpu().numpy()
+    eng.check()
+    assert np.array_equal(y2.view(np.uint32), y.view(np.uint32)[1:3])
     y8 = eng.dense_proj(mlp.down, T, (h4 * 8.0).contiguous()).cpu().numpy()
     assert np.array_equal(y8.view(np.uint32), (y * np.float32(8.0)).view(np.uint32))
     for t in (0, 3):
@@ -513,6 +639,7 @@ def test_config3_full_size_head(eng):
     for r0 in (0, 75968 - 100, rows - 256):
         ref = orc.gemv(w[r0 * rb:(r0 + 256) * rb], 256, cols, gs, x, threads=8)[0]
         assert rel_err(got[r0:r0 + 256], ref) <= TOL, r0
+        assert gamma_rows(got[r0:r0 + 256], w, r0, 256, cols, gs, x) <= 1.0, r0
     assert int(idx.item()) == orc.argmax_ref(got) == int(np.argmax(got))
     logits2, idx2 = eng.lm_head_row(f, _dev(x), fused=False)
     assert np.array_equal(logits2.cpu().numpy().reshape(-1).view(np.uint32), got.view(np.uint32))
@@ -550,7 +677,8 @@ def test_gemm_ragged_shapes_drawn_at_random(eng):
         for kernel in (None, forced):
             y = eng.gemm(f, m, xb.reshape(m, cols).contiguous(), kernel=kernel).cpu().numpy()
             eng.check()
-            assert rel_err(y, ref) <= TOL, (case, kernel)
+            assert rel_err(y, ref, floor_of(y.size)) <= TOL, (case, kernel)
+            assert gamma_ratio(y[:2], w, rows, cols, gs, xw.reshape(m, cols)[:2]) <= 1.0, (case, kernel)
 
 
 def test_gemm_m16_full_size_cross_block_split(eng):
@@ -573,13 +701,15 @@ def _gemm_case(eng, m, rows, cols, kernel):
     y = eng.gemm(f, m, xb.reshape(m, cols).contiguous(), kernel=kernel).cpu().numpy()
     eng.check()
     ref = orc.gemv(w, rows, cols, gs, xw.reshape(m, cols), threads=8)
-    assert rel_err(y, ref) <= TOL
+    assert rel_err(y, ref, floor_of(y.size)) <= TOL
     assert gamma_ratio(y[:4], w, rows, cols, gs, xw.reshape(m, cols)[:4]) <= 1.0
 
 
-def test_gemm_full_size_sampled_rows(eng):
-    """Benchmark config 4 (batched GEMM) at M = 512 on the full [17408, 5120] tensor; the CPU path checks 768 sampled rows."""
-    rows, cols, m = 17408, 5120, 512
+@pytest.mark.parametrize("m", [512, 128])
+def test_gemm_full_size_sampled_rows(eng, m):
+    """Benchmark config 4 (batched GEMM) at M = 512 and M = 128 on the full [17408, 5120] tensor; the CPU path checks 768 sampled rows."""
+    rows, cols = 17408, 5120
+    print(f"case m={m}", flush=True)
     w, gs = quantized_normal(0, 0, rows, cols)
     f = _load(w, rows, cols, gs)
     xb, xw = _bf16_dev(normal_f32(0, 40, m * cols))
@@ -588,7 +718,8 @@ def test_gemm_full_size_sampled_rows(eng):
     rb = cols // 64 * 36
     for r0 in (0, 8704 - 128, 17408 - 256):
         ref = orc.gemv(w[r0 * rb:(r0 + 256) * rb], 256, cols, gs, xw.reshape(m, cols), threads=8)
-        assert rel_err(y[:, r0:r0 + 256], ref) <= TOL, r0
+        assert rel_err(y[:, r0:r0 + 256], ref, floor_of(3 * ref.size)) <= TOL, r0
+        assert gamma_rows(y[:8, r0:r0 + 256], w, r0, 256, cols, gs, xw.reshape(m, cols)[:8]) <= 1.0, r0
     # linearity, a size-independent property: rows of X scaled by powers of two scale Y exactly
     x2 = (xb.reshape(m, cols).float() * 4.0).to(torch.bfloat16).contiguous()
     y2 = eng.gemm(f, m, x2).cpu().numpy()
@@ -630,7 +761,7 @@ def test_container_tensors_load_dequantise_and_multiply(eng):
     x = normal_f32(12, 0, 2 * 64).reshape(2, 64) * np.float32(40.0)
     y = eng.dense_ffn_w(MlpW(g, u, d), _dev(x), 2).cpu().numpy()
     ref = orc.ffn(graw, gt.global_scale, uraw, ut.global_scale, draw, dt.global_scale, 64, 128, x)
-    assert rel_err(y, ref) <= TOL
+    assert rel_err(y, ref, FLOOR_CHAINED) <= TOL
     eng.check()
     c.close()
 
@@ -653,7 +784,7 @@ def test_captured_sequence_replays_match_eager_launches(eng):
     seq = [("gemv_nvfp4_gu", launch_dims("gemv_nvfp4_gu", I, H), [g_.w_ptr, u_.w_ptr, x.data_ptr(), g_.gs_ptr, u_.gs_ptr, hbuf.data_ptr(), p.i32(H), p.i32(I)]),
            ("gemv_nvfp4_w", launch_dims("gemv_nvfp4_w", H, I), [d_.w_ptr, hbuf.data_ptr(), d_.gs_ptr, y.data_ptr(), p.i32(I), p.i32(H)]),
            ("gemv_nvfp4_w_argmax", launch_dims("gemv_nvfp4_w_argmax", V, H), [h_.w_ptr, y.data_ptr(), h_.gs_ptr, logits.data_ptr(), p.i32(H), p.i32(V), tok.data_ptr()]),
-           ("argmax_tiles", (1, 1, 1, 256), [tok.data_ptr(), p.i32(V)])]
+           ("argmax_tiles", launch_dims("argmax_tiles", V, H), [tok.data_ptr(), p.i32(V)])]
 
     def eager():
         for name, dims, vals in seq:
@@ -680,7 +811,7 @@ def test_captured_sequence_replays_match_eager_launches(eng):
     # and the replayed result is the CPU path's
     xr = normal_f32(50, 3, H) * np.float32(0.05)
     ref = orc.ffn(wg, 2e-3, wu, 1.5e-3, wd, 1.1e-3, H, I, xr.reshape(1, H))[0]
-    assert rel_err(y.cpu().numpy(), ref) <= TOL
+    assert rel_err(y.cpu().numpy(), ref, FLOOR_CHAINED) <= TOL
     gr.close()
     eng.check()
 
@@ -699,10 +830,20 @@ def test_launches_with_a_wrong_block_shape_are_refused(eng):
     gx, gy, gz, bx = launch_dims("gemv_nvfp4_w", rows, cols)
     with pytest.raises(CrowHipError):
         launch_v(eng.k.f("gemv_nvfp4_w"), gx, gy, gz, 100, [f.w_ptr, x.data_ptr(), f.gs_ptr, y.data_ptr(), p.i32(cols), p.i32(rows)])
-    launch_v(eng.k.f("gemv_nvfp4_gu"), 1, 2, 1, 192, [f.w_ptr, f.w_ptr, x.data_ptr(), f.gs_ptr, f.gs_ptr, y.data_ptr(), p.i32(cols), p.i32(rows)])
+    gx, gy, gz, bx = launch_dims("gemv_nvfp4_gu", rows, cols)
+    launch_v(eng.k.f("gemv_nvfp4_gu"), gx, gy, gz, 192, [f.w_ptr, f.w_ptr, x.data_ptr(), f.gs_ptr, f.gs_ptr, y.data_ptr(), p.i32(cols), p.i32(rows)])
     with pytest.raises(CrowHipError):
         eng.check()
     assert float(y.min()) == 7.0 == float(y.max())
+    # the 32-token GEMM entry stages and reduces in LDS sized for four waves: a larger block is refused, nothing written
+    xb = torch.zeros((20, cols), dtype=torch.bfloat16, device="cuda")
+    yg = torch.full((20, rows), 7.0, dtype=torch.float32, device="cuda")
+    gx, gy, gz, bx = launch_dims("gemm_nvfp4_bf16_m32", rows, cols, 20)
+    for bad_bx in (512, 320):
+        launch_v(eng.k.f("gemm_nvfp4_bf16_m32"), gx, gy, gz, bad_bx, [f.w_ptr, xb.data_ptr(), f.gs_ptr, yg.data_ptr(), p.i32(cols), p.i32(rows), p.i32(20)])
+        with pytest.raises(CrowHipError) as ei:
+            eng.check()
+        assert ei.value.code == -7 and bool((yg == 7.0).all())
     eng.check()
 
 
@@ -740,6 +881,44 @@ def test_an_unsupported_geometry_is_refused_and_an_empty_pointer_table_is_not_fo
     with pytest.raises(CrowHipError) as ei:
         eng.check()
     assert ei.value.code == -8 and float(y.min()) == 7.0 == float(y.max())  # y += 0 from every combo
+    # the kernels that take their slabs from the expert TABLE: a table whose entries are zeros is not followed either
+    E = eng.geo.experts
+    table0 = torch.zeros((E, 2), dtype=torch.int64, device="cuda")
+    tiles = torch.tensor([[3, 0, 2, 0]], dtype=torch.int32, device="cuda")
+    n_tiles = torch.ones(1, dtype=torch.int32, device="cuda")
+    perm = torch.tensor([1, 0], dtype=torch.int32, device="cuda")
+    xk = torch.zeros((1, H), dtype=torch.float32, device="cuda")
+    eo = torch.full((K, H), 7.0, dtype=torch.float32, device="cuda")
+    launch_v(eng.k.f("moe_gate_up_silu_grouped"), *launch_dims("moe_gate_up_silu_grouped", I, H, 1),
+             [tiles.data_ptr(), n_tiles.data_ptr(), perm.data_ptr(), table0.data_ptr(), xk.data_ptr(), gs.data_ptr(), h2.data_ptr(),
+              p.i32(H), p.i32(K), p.i32(H), p.i32(I)])
+    with pytest.raises(CrowHipError) as ei:
+        eng.check()
+    assert ei.value.code == -8 and float(h2.min()) == 7.0 == float(h2.max())
+    launch_v(eng.k.f("moe_down_grouped"), *launch_dims("moe_down_grouped", H, I, 1),
+             [tiles.data_ptr(), n_tiles.data_ptr(), perm.data_ptr(), table0.data_ptr(), h2.data_ptr(), gs.data_ptr(), eo.data_ptr(), p.i32(I), p.i32(H)])
+    with pytest.raises(CrowHipError) as ei:
+        eng.check()
+    assert ei.value.code == -8 and float(eo.min()) == 7.0 == float(eo.max())
+    logits = _dev(normal_f32(6, 77, E).reshape(1, E))
+    ids = torch.full((1, K), -1, dtype=torch.int32, device="cuda")
+    wr = torch.zeros((1, K), dtype=torch.float32, device="cuda")
+    dn = torch.zeros((1, K), dtype=torch.int64, device="cuda")
+    launch_v(eng.k.f("moe_route_gate_up_silu"), *launch_dims("moe_route_gate_up_silu", I, H, K),
+             [logits.data_ptr(), table0.data_ptr(), xk.data_ptr(), gs.data_ptr(), h2.data_ptr(), ids.data_ptr(), wr.data_ptr(), dn.data_ptr(),
+              p.i32(H), p.i32(H), p.i32(I)])
+    with pytest.raises(CrowHipError) as ei:
+        eng.check()
+    assert ei.value.code == -8 and float(h2.min()) == 7.0 == float(h2.max())
+    # the host mirror refuses a table that does not cover the geometry's experts before anything is launched
+    from crow_nest_amd.engine import MoeW
+    from crow_nest_amd.weights import ExpertSlabs
+    few = ExpertSlabs(torch.zeros(16, dtype=torch.uint8, device="cuda"), gs, E // 2, 2 * I, H, 8)
+    few_dn = ExpertSlabs(torch.zeros(16, dtype=torch.uint8, device="cuda"), gs, E // 2, H, I, 8)
+    bad = MoeW(few, few_dn, torch.zeros((E // 2, 2), dtype=torch.int64, device="cuda"))
+    for run in (lambda: eng.moe_run(bad, xk, logits), lambda: eng.moe_run_grouped(bad, xk, logits), lambda: eng.router(logits, bad)):
+        with pytest.raises(ValueError, match="experts"):
+            run()
     eng.check()
 
 
@@ -753,11 +932,21 @@ def test_verify_kernels_refuse_more_than_four_rows(eng):
     x = torch.zeros(5 * cols, dtype=torch.float32, device="cuda")
     y = torch.full((5 * rows,), 7.0, dtype=torch.float32, device="cuda")
     p = eng.p
-    launch_v(eng.k.f("gemv_nvfp4_wm"), *launch_dims("gemv_nvfp4_wm", rows, cols), [f.w_ptr, x.data_ptr(), f.gs_ptr, y.data_ptr(), p.i32(cols), p.i32(rows), p.i32(5)])
+    with pytest.raises(CrowHipError) as ei:  # asked for by its own name, five rows are refused on the host
+        launch_dims("gemv_nvfp4_wm", rows, cols, 5)
+    assert ei.value.code == -7  # CROW_ERR_SHAPE
+    # dims made for four rows (or for an unknown count), the word behind m_p saying five: refused by the kernel
+    for z in (4, 1):
+        launch_v(eng.k.f("gemv_nvfp4_wm"), *launch_dims("gemv_nvfp4_wm", rows, cols, z), [f.w_ptr, x.data_ptr(), f.gs_ptr, y.data_ptr(), p.i32(cols), p.i32(rows), p.i32(5)])
+        with pytest.raises(CrowHipError) as ei:
+            status()
+        assert ei.value.code == -7
+        assert bool((y == 7.0).all())
+    # and a launch whose dims were made for another K stores nothing either
+    launch_v(eng.k.f("gemv_nvfp4_wm"), *launch_dims("gemv_nvfp4_wm", rows, cols // 2, 2), [f.w_ptr, x.data_ptr(), f.gs_ptr, y.data_ptr(), p.i32(cols), p.i32(rows), p.i32(2)])
     with pytest.raises(CrowHipError) as ei:
         status()
-    assert ei.value.code == -7  # CROW_ERR_SHAPE
-    assert bool((y == 7.0).all())
+    assert ei.value.code == -7 and bool((y == 7.0).all())
     eng.check()
 
 
