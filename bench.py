@@ -218,9 +218,9 @@ def main() -> int:
         others["config0_gemv_17408x5120_f32x"] = entry(l0.us(), W_BYTES + K * 4 + N * 4 + 4)
         # config 1 at verify widths
         for m in (2, 4):
-            lg = Launch(eng, "gemv_nvfp4_gum_bf16", N, K, 1,
+            lg = Launch(eng, "gemv_nvfp4_gum_bf16", N, K, m,
                         [[s["gate"].data_ptr(), s["up"].data_ptr(), xkb.data_ptr(), gs1.data_ptr(), gs1.data_ptr(), ybuf.data_ptr(), p.i32(K), p.i32(N), p.i32(m)] for s in sets])
-            ld = Launch(eng, "gemv_nvfp4_wm", K, N, 1,
+            ld = Launch(eng, "gemv_nvfp4_wm", K, N, m,
                         [[s["down"].data_ptr(), xf.data_ptr(), gs1.data_ptr(), ybuf.data_ptr(), p.i32(N), p.i32(K), p.i32(m)] for s in sets])
             others[f"config1_gate_up_silu_M{m}"] = entry(lg.us(), alg_bytes_gate_up(m))
             others[f"config1_down_M{m}"] = entry(ld.us(), alg_bytes_down(m))
@@ -232,6 +232,7 @@ def main() -> int:
         l3 = Launch(eng, "gemv_nvfp4_w_argmax", V, K, 1, [[hd.data_ptr(), xk.data_ptr(), gs1.data_ptr(), ybuf.data_ptr(), p.i32(K), p.i32(V), idx.data_ptr()] for hd in heads])
         from crow_nest_amd.kernels import time_sequence
         seq3 = [(l3.f, l3.dims, l3.raw), (eng.k.f("argmax_tiles"), (1, 1, 1, 256), [[idx.data_ptr(), p.i32(V)]])]
+        status()
         time_sequence(seq3, 4, 10)
         others["config3_lm_head_151936x5120_argmax"] = entry(min(time_sequence(seq3, 4, 100) for _ in range(3)), V * K // 64 * 36 + K * 4 + V * 4 + 4)
         others["config3_lm_head_151936x5120_argmax"]["launches"] = 2

@@ -17,17 +17,18 @@ struct FnEntry {
     const void* stub;
     int nargs;
     unsigned lds_fixed;  // dynamic LDS of a launch (kernels outside the GEMV family)
-    // GEMV family (gemv.h): tensors per block (0 = not of the family), and the dynamic LDS of a block as a function of the most
-    // groups one of its waves owns: zero area + one staging area per wave
+    // GEMV family (gemv.h): tensors per block (0 = not of the family), and the dynamic LDS of a block: the zero area + one
+    // staging area per wave
     int nr;
-    int (*lds_zero)(int most);
-    int (*lds_per_wave)(int most);
+    int max_waves;  // per block (the kernel's launch bound)
+    int lds_per_wave;
 };
 
-#define CROW_FN(name, nargs) {#name, (const void*)&name, nargs, 0u, 0, nullptr, nullptr}
+#define CROW_FN(name, nargs) {#name, (const void*)&name, nargs, 0u, 0, 16, 0}
 // NR tensors per block, bodies for 1 .. MMAX activation rows, bf16 or f32 activations
+// (the bodies for several f32 rows need more registers than a block of sixteen waves leaves each: they run in blocks of eight)
 #define CROW_GEMV(name, nargs, NR, MMAX, XBF16) \
-    {#name, (const void*)&name, nargs, 0u, NR, &crow::StagingAlloc<MMAX, XBF16>::zero_bytes, &crow::StagingAlloc<MMAX, XBF16>::per_wave}
+    {#name, (const void*)&name, nargs, 0u, NR, (MMAX > 1 && !XBF16) ? 8 : 16, crow::crow_gemv_lds_per_wave(MMAX, XBF16)}
 const FnEntry g_table[] = {
     CROW_GEMV(gemv_nvfp4_w, 6, 1, 1, false),       CROW_GEMV(gemv_nvfp4_w_bf16, 6, 1, 1, true),  CROW_GEMV(gemv_nvfp4_w_argmax, 7, 1, 1, false),
     CROW_GEMV(gemv_nvfp4_gu, 8, 2, 1, false),      CROW_GEMV(gemv_nvfp4_gu_bf16, 8, 2, 1, true),
@@ -41,10 +42,10 @@ const FnEntry g_table[] = {
     CROW_FN(argmax_k, 3),          CROW_FN(argmax_tiles, 2),        CROW_FN(dequant_fp4_flat, 4),    CROW_FN(repack_nvfp4, 4),
     CROW_FN(unpack_nvfp4, 4),      CROW_FN(dequant_nvfp4_tiled, 5),
     // shared-X GEMM blocks: two staged X tiles of MT rows x 528 bytes
-    {"gemm_nvfp4_bf16", (const void*)&gemm_nvfp4_bf16, 7, 2u * 128u * 528u, 0, nullptr, nullptr},
-    {"gemm_nvfp4_bf16_m64", (const void*)&gemm_nvfp4_bf16_m64, 7, 2u * 64u * 528u, 0, nullptr, nullptr},
-    {"gemm_nvfp4_bf16_m48", (const void*)&gemm_nvfp4_bf16_m48, 7, 2u * 48u * 528u, 0, nullptr, nullptr},
-    {"gemm_nvfp4_bf16_m96", (const void*)&gemm_nvfp4_bf16_m96, 7, 2u * 96u * 528u, 0, nullptr, nullptr},
+    {"gemm_nvfp4_bf16", (const void*)&gemm_nvfp4_bf16, 7, 2u * 128u * 528u, 0, 16, 0},
+    {"gemm_nvfp4_bf16_m64", (const void*)&gemm_nvfp4_bf16_m64, 7, 2u * 64u * 528u, 0, 16, 0},
+    {"gemm_nvfp4_bf16_m48", (const void*)&gemm_nvfp4_bf16_m48, 7, 2u * 48u * 528u, 0, 16, 0},
+    {"gemm_nvfp4_bf16_m96", (const void*)&gemm_nvfp4_bf16_m96, 7, 2u * 96u * 528u, 0, 16, 0},
     CROW_FN(gemm_nvfp4_bf16_m32, 7), CROW_FN(gemm_nvfp4_bf16_m16, 7), CROW_FN(gemv_bf16_w, 5),
     CROW_FN(gemv_bf16, 5), CROW_FN(gemv_bf16_b, 5), CROW_FN(gemv_b, 5), CROW_FN(gemv_bf16_ws, 5), CROW_FN(gemv_bf16_bs, 6),
 };
@@ -94,7 +95,7 @@ int launch_entry(const FnEntry* e, dim3 grid, dim3 block, const uint64_t* vals, 
     if (!e || !vals) return CROW_ERR_BAD_ARGUMENT;
     if ((int)n != e->nargs) return CROW_ERR_ARG_COUNT;
     // whole wavefronts only: every kernel derives its wave count (and its LDS layout) from block.x / 64
-    if (grid.x == 0 || grid.y == 0 || grid.z == 0 || block.x == 0 || block.x > 1024 || block.x % 64 != 0) return CROW_ERR_BAD_ARGUMENT;
+    if (grid.x == 0 || grid.y == 0 || grid.z == 0 || block.x == 0 || block.x > 64u * (unsigned)e->max_waves || block.x % 64 != 0) return CROW_ERR_BAD_ARGUMENT;
     void* args[17];
     for (uint32_t i = 0; i < n; i++) args[i] = (void*)&vals[i];
     size_t lds = e->lds_fixed;
@@ -104,11 +105,7 @@ int launch_entry(const FnEntry* e, dim3 grid, dim3 block, const uint64_t* vals, 
         const int pairs = (int)(word & 0xFFFFFu), slices = (int)(word >> 24) == 0 ? 1 : (int)(word >> 24);
         const int waves = (int)(block.x / 64), wpt = waves / e->nr;
         if (pairs == 0 || wpt == 0) return CROW_ERR_BAD_ARGUMENT;
-        const int groups = (pairs + CROW_GROUP_PAIRS - 1) / CROW_GROUP_PAIRS;
-        // (moe_down_combine's waves are the token's picks: each owns all groups of its strip)
-        int most = e->stub == (const void*)&moe_down_combine ? groups : crow::crow_most_groups(groups, slices * wpt);
-        if (most > CROW_GEMV_GMAX) most = CROW_GEMV_GMAX;
-        lds = (size_t)e->lds_zero(most) + (size_t)waves * (size_t)e->lds_per_wave(most);
+        lds = (size_t)CROW_GEMV_ZERO_BYTES + (size_t)waves * (size_t)e->lds_per_wave;
         if (lds > g.lds_cap) return CROW_ERR_SHAPE;
         geo = (int)(word & 0xFFFFFFu);
         grid.y = (unsigned)slices;
@@ -163,8 +160,8 @@ int crow_hip_init(int device) {
     // a GEMV block of 16 waves, and the GEMM's two staged X tiles, need more dynamic LDS than the default per-block limit
     for (int i = 0; i < g_table_n; i++) {
         size_t most = g_table[i].lds_fixed;
-        if (g_table[i].nr != 0) {  // the GEMV family: a block of sixteen waves at the longest staged rows, within the device's limit
-            most = (size_t)g_table[i].lds_zero(CROW_GEMV_GMAX) + 16 * (size_t)g_table[i].lds_per_wave(CROW_GEMV_GMAX);
+        if (g_table[i].nr != 0) {  // the GEMV family: the largest block the kernel takes, within the device's limit
+            most = (size_t)CROW_GEMV_ZERO_BYTES + (size_t)g_table[i].max_waves * (size_t)g_table[i].lds_per_wave;
             if (most > g.lds_cap) most = g.lds_cap;
         }
         if (most > 48 * 1024 &&
@@ -325,18 +322,11 @@ int crow_hip_launch_dims_split(const char* name, uint32_t rows, uint32_t k_dim, 
             return CROW_OK;
         }
         if (verify && z > 4) return CROW_ERR_SHAPE;
-        const uint32_t wmax = 16u / (uint32_t)e->nr;  // waves per tensor in a block of at most 1024 threads
-        // A wave takes at most four groups (9 KB of loads, all in flight from its first instruction).  One block holds a
-        // strip when that needs no more waves than a block has; longer strips are cut into slices of four waves.
-        const uint32_t units = (groups + CROW_GEMV_GMAX - 1) / CROW_GEMV_GMAX;
-        uint32_t w, s;
-        if (units <= wmax) {
-            w = units;
-            s = 1;
-        } else {
-            w = 4;
-            s = (units + w - 1) / w;
-        }
+        const uint32_t wmax = (uint32_t)e->max_waves / (uint32_t)e->nr;  // waves per tensor in a block
+        // A wave walks its run of groups with four of them (9 KB) in flight; few long walks beat many short ones (measured:
+        // every wave pays its start, its staging set-up and the block's meeting in LDS once).  One block holds a whole strip
+        // whatever K is: there is no cross-block split unless it is asked for.
+        uint32_t w = (groups + 3 * CROW_GEMV_RING - 1) / (3 * CROW_GEMV_RING), s = 1;  // about twelve groups (27 KB) per wave
         if (force_s > 0) s = force_s;
         if (force_w > 0) w = force_w;
         if (w > wmax) w = wmax;

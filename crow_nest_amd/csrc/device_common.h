@@ -30,6 +30,9 @@ __device__ __forceinline__ uint4 stream_load(const uint4* p) {
     return make_uint4(v.x, v.y, v.z, v.w);
 }
 
+__device__ __forceinline__ u32x4 stream_load_v(const uint4* p) {
+    return __builtin_nontemporal_load((const __attribute__((address_space(1))) u32x4*)p);
+}
 // the same for one dword per lane (the scale words of a 256-column group)
 __device__ __forceinline__ unsigned stream_load_u32(const unsigned* p) {
     return __builtin_nontemporal_load((const __attribute__((address_space(1))) unsigned*)p);

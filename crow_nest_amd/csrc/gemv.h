@@ -1,8 +1,8 @@
 // NVFP4 GEMV family for gfx950: y[m][row] = gs * sum_k W[row][k] * x[m][k], M <= 4 activation rows.
 //
 // Mapping.  A workgroup owns one 16-row STRIP of the tensor (layout.h) and, for K up to 16384, ALL of its columns: wave w of
-// the block takes a run of consecutive 256-column groups, at most four (9 KB) at a time, and the block's waves meet in
-// LDS.  Nothing crosses workgroups, so there is no workspace, no arrival counter and no device-scope ordering on this path.
+// the block walks a run of consecutive 256-column groups, four of them (9 KB) in flight at any time, and the block's waves
+// meet in LDS.  Nothing crosses workgroups, so there is no workspace, no arrival counter and no device-scope ordering on this path.
 // Only tensors whose strip does not fit one block's waves (K > 16384, e.g. the 17408-column down projection) are cut into S
 // column slices whose blocks hand their 16 sums over through the library workspace (slice_hand_over below).
 // The weights are read exactly once, as non-temporal loads that cover 1024 contiguous bytes per instruction, issued
@@ -30,8 +30,9 @@
 // added as (hi + mid) + lo before the scale FMA: every product w * term is exact in f32, so the only roundings are the f32
 // additions, as in any f32 dot product.
 //
-// Each wave stages its own activation slice in LDS (bf16 rows, 512 bytes per group) while its weight loads are in flight and
-// reads its A operands from there with one 16-byte read per lane; lanes whose operand row is zero read a zeroed area instead.
+// Each wave stages its own activation slice in LDS, group by group (bf16 rows, 512 bytes per group, two groups deep), while
+// its weight loads are in flight, and reads its A operands from there with one 16-byte read per lane; lanes whose operand
+// row is zero read a zeroed area instead.
 //
 // FP32 accumulation order (per output row and activation row), documented because it differs from the reference CPU path's
 // 8-lane order (cpu_nvfp4.rs:22-31) and from its GPU kernel of record (kernels_p2.rs:304-347); all three are within the same
@@ -51,9 +52,9 @@
 // unit u = slice * W + wave.
 //
 // Dynamic LDS of a block (bytes; the launcher sizes it from the block size):
-//   [0, ZERO)                       zeros (as long as a staged row)
-//   [ZERO + wave * XR * ROW, ...)   the wave's activation staging, XR rows of ROW bytes; when a wave has finished its groups,
-//                                   the first 64 M bytes of its area carry its 16 M sums to wave 0
+//   [0, 640)                        zeros
+//   [640 + wave * 2 * XR * 560, ..) the wave's activation staging: two slots of XR rows of 560 bytes; when a wave has finished
+//                                   its groups, the first 64 M bytes of its area carry its 16 M sums to wave 0
 #pragma once
 #include "device_common.h"
 
@@ -89,45 +90,24 @@ __device__ __forceinline__ GemvArgs gemv_args(const unsigned char* w0, const uns
     return a;
 }
 
-// most groups of 256 columns a wave holds in registers at once (9 dwords each)
-#define CROW_GEMV_GMAX 4
-// A staged activation row holds the groups of one batch, 512 bytes each.  The 48 bytes of padding start four consecutive rows
+// A wave keeps this many 256-column groups (2304 bytes each) in flight: a ring of register slots that is refilled group by
+// group as the wave walks along its strip.
+#define CROW_GEMV_RING 4
+// One staged activation row of one group: 512 bytes of bf16 values.  The 48 bytes of padding start four consecutive rows
 // 48 bytes apart modulo the 128-byte bank cycle, so that the operand reads of a set's rows miss each other.
-#define CROW_GEMV_ROW_PAD 48
+#define CROW_GEMV_XROW_BYTES 560
+#define CROW_GEMV_ZERO_BYTES 640  // a zeroed row (512 bytes + what a zero lane's reads reach past the last pair's offset)
 
-// How many groups a wave stages at once (SG; the rest follow in batches while it computes) and how many rows (XR): one bf16
-// row per token, or three (hi, mid, lo) per f32 token.  One-row kernels stage everything up front, while the weight loads are
-// in flight; the others in batches that keep the registers carrying activations to LDS, and a compute unit's 160 KB, within
-// what twenty-odd resident waves can share.  The row length follows the launch: `most` = the most groups any wave of the
-// launch owns, so a K = 2048 strip on four waves stages rows of two groups, not four.
+// The staging a wave needs for M activation rows: XR rows per group (one bf16 row per token, or three - hi, mid, lo - per f32
+// token), two groups deep (the next group is staged while the current one is multiplied).
 template <int M, bool XBF16>
 struct Staging {
-    static constexpr int SG = XBF16 ? (M == 1 ? CROW_GEMV_GMAX : 2) : (M == 1 ? CROW_GEMV_GMAX : 1);
     static constexpr int XR = XBF16 ? M : 3 * M;
-    CROW_HD static constexpr int batch(int most) { return most < SG ? most : SG; }
-    CROW_HD static constexpr int row_bytes(int most) { return batch(most) * 512 + CROW_GEMV_ROW_PAD; }
-    CROW_HD static constexpr int zero_bytes(int most) { return batch(most) * 512 + 64; }  // a zero lane's reads reach 64 bytes past the last pair's offset
-    CROW_HD static constexpr int per_wave(int most) { return XR * row_bytes(most); }
+    static constexpr int SLOT = XR * CROW_GEMV_XROW_BYTES;
+    static constexpr int PER_WAVE = 2 * SLOT;  // also carries the wave's 16 M sums to wave 0 afterwards (>= 256 bytes)
 };
-// the dynamic LDS of a block whose entry point dispatches over 1 .. MMAX activation rows: sized for the widest of its bodies
-template <int MMAX, bool XBF16>
-struct StagingAlloc {
-    CROW_HD static constexpr int zero_bytes(int most) {
-        const int a = Staging<MMAX, XBF16>::zero_bytes(most), b = StagingAlloc<MMAX - 1, XBF16>::zero_bytes(most);
-        return a > b ? a : b;
-    }
-    CROW_HD static constexpr int per_wave(int most) {
-        const int a = Staging<MMAX, XBF16>::per_wave(most), b = StagingAlloc<MMAX - 1, XBF16>::per_wave(most);
-        return a > b ? a : b;
-    }
-};
-template <bool XBF16>
-struct StagingAlloc<0, XBF16> {
-    CROW_HD static constexpr int zero_bytes(int) { return 0; }
-    CROW_HD static constexpr int per_wave(int) { return 256; }  // the 16 x 4 sums a wave hands to wave 0
-};
-// the most groups a wave of a launch owns: `groups` dealt to `units` = slices * waves-per-tensor
-CROW_HD static constexpr int crow_most_groups(int groups, int units) { return (groups + units - 1) / units; }
+// the dynamic LDS of a block: the zero area, then one staging area per wave, sized for the widest body of the entry point
+CROW_HD static constexpr int crow_gemv_lds_per_wave(int mmax, bool xbf16) { return 2 * (xbf16 ? mmax : 3 * mmax) * CROW_GEMV_XROW_BYTES; }
 
 typedef __attribute__((address_space(3))) unsigned char* lds_p;
 __device__ __forceinline__ void lds_store16(lds_p p, unsigned a, unsigned b, unsigned c, unsigned d) {
@@ -145,97 +125,19 @@ __device__ __forceinline__ bf16x8 decode8(unsigned codes) {
     return __builtin_bit_cast(bf16x8, r);
 }
 
-// the registers of up to GMAX groups: one scale dword and two code quadwords per group
-struct GroupRegs {
-    unsigned sc[CROW_GEMV_GMAX];
-    uint4 cd[CROW_GEMV_GMAX][2];
-};
-// `first` = address of the wave's first group; loads of groups >= n are not issued (n is wave-uniform)
-__device__ __forceinline__ void load_groups(const unsigned char* first, int n, int lane, GroupRegs& r) {
-#pragma unroll
-    for (int g = 0; g < CROW_GEMV_GMAX; g++) {
-        if (g < n) {
-            const unsigned char* p = first + (size_t)g * CROW_GROUP_BYTES;
-            r.sc[g] = stream_load_u32((const unsigned*)p + lane);
-            r.cd[g][0] = stream_load((const uint4*)(p + CROW_GROUP_SCALE_BYTES) + lane);
-            r.cd[g][1] = stream_load((const uint4*)(p + CROW_GROUP_SCALE_BYTES + 1024) + lane);
-        }
-    }
+// x = hi + mid + lo exactly: each term keeps the next 8 significant bits (truncation; the subtractions are exact)
+__device__ __forceinline__ void split3(float f, unsigned& hi, unsigned& mid, unsigned& lo) {
+    hi = __float_as_uint(f) & 0xffff0000u;
+    const float r1 = __fsub_rn(f, __uint_as_float(hi));
+    mid = __float_as_uint(r1) & 0xffff0000u;
+    const float r2 = __fsub_rn(r1, __uint_as_float(mid));
+    lo = __float_as_uint(r2) & 0xffff0000u;
 }
 
-// The activation slice of a batch of SG groups, fetched into registers and then written to the wave's LDS rows.
-template <int M, bool XBF16>
-struct XStage;
-template <int M>
-struct XStage<M, true> {
-    static constexpr int SG = Staging<M, true>::SG;
-    uint2 v[M][SG];
-    // columns col0 + 256 gg + 4 lane .. + 3 of token row t, for the batch's first n groups
-    __device__ __forceinline__ void fetch(const void* x, const size_t (&xoff)[M], int col0, int k_dim, int n, int lane) {
-#pragma unroll
-        for (int t = 0; t < M; t++)
-#pragma unroll
-            for (int gg = 0; gg < SG; gg++) {
-                const int col = col0 + CROW_GROUP_COLS * gg + 4 * lane;
-                v[t][gg] = make_uint2(0, 0);
-                if (gg < n && col < k_dim) v[t][gg] = *(const uint2*)((const unsigned short*)x + xoff[t] + col);
-            }
-    }
-    __device__ __forceinline__ void store(lds_p xw, int ROW, int n, int lane) const {
-#pragma unroll
-        for (int t = 0; t < M; t++)
-#pragma unroll
-            for (int gg = 0; gg < SG; gg++)
-                if (gg < n) lds_store8(xw + t * ROW + 512 * gg + 8 * lane, v[t][gg].x, v[t][gg].y);
-    }
-};
-template <int M>
-struct XStage<M, false> {
-    static constexpr int SG = Staging<M, false>::SG;
-    float4 v[M][SG];
-    __device__ __forceinline__ void fetch(const void* x, const size_t (&xoff)[M], int col0, int k_dim, int n, int lane) {
-#pragma unroll
-        for (int t = 0; t < M; t++)
-#pragma unroll
-            for (int gg = 0; gg < SG; gg++) {
-                const int col = col0 + CROW_GROUP_COLS * gg + 4 * lane;
-                v[t][gg] = make_float4(0.f, 0.f, 0.f, 0.f);
-                if (gg < n && col < k_dim) v[t][gg] = *(const float4*)((const float*)x + xoff[t] + col);
-            }
-    }
-    // x = hi + mid + lo exactly: each term keeps the next 8 significant bits (truncation; the subtractions are exact)
-    __device__ __forceinline__ static void split(float f, unsigned& hi, unsigned& mid, unsigned& lo) {
-        hi = __float_as_uint(f) & 0xffff0000u;
-        const float r1 = __fsub_rn(f, __uint_as_float(hi));
-        mid = __float_as_uint(r1) & 0xffff0000u;
-        const float r2 = __fsub_rn(r1, __uint_as_float(mid));
-        lo = __float_as_uint(r2) & 0xffff0000u;
-    }
-    __device__ __forceinline__ void store(lds_p xw, int ROW, int n, int lane) const {
-#pragma unroll
-        for (int t = 0; t < M; t++)
-#pragma unroll
-            for (int gg = 0; gg < SG; gg++) {
-                if (gg < n) {
-                    unsigned h[4], m[4], l[4];
-                    split(v[t][gg].x, h[0], m[0], l[0]);
-                    split(v[t][gg].y, h[1], m[1], l[1]);
-                    split(v[t][gg].z, h[2], m[2], l[2]);
-                    split(v[t][gg].w, h[3], m[3], l[3]);
-                    // bf16 pairs: high halves of (odd element, even element)
-                    lds_p row = xw + (3 * t) * ROW + 512 * gg + 8 * lane;
-                    lds_store8(row, __builtin_amdgcn_perm(h[1], h[0], 0x07060302u), __builtin_amdgcn_perm(h[3], h[2], 0x07060302u));
-                    lds_store8(row + ROW, __builtin_amdgcn_perm(m[1], m[0], 0x07060302u), __builtin_amdgcn_perm(m[3], m[2], 0x07060302u));
-                    lds_store8(row + 2 * ROW, __builtin_amdgcn_perm(l[1], l[0], 0x07060302u), __builtin_amdgcn_perm(l[3], l[2], 0x07060302u));
-                }
-            }
-    }
-};
-
 // One 256-column group: four pairs.  `a1[q]`, `a2[q]` are this lane's LDS addresses of its A1 / A2 operand for pair 0 of the
-// staged batch, set q (or of the zero area); OFF = byte offset of the group inside the staged batch.
-template <int M, bool XBF16, int OFF>
-__device__ __forceinline__ void group_multiply(unsigned sc, const uint4 (&cd)[2], const lds_p (&a1)[XBF16 ? 1 : (3 * M + 3) / 4],
+// group's staging slot, set q (or of the zero area).
+template <int M, bool XBF16>
+__device__ __forceinline__ void group_multiply(unsigned sc, const u32x4 (&cd)[2], const lds_p (&a1)[XBF16 ? 1 : (3 * M + 3) / 4],
                                                const lds_p (&a2)[XBF16 ? 1 : (3 * M + 3) / 4], float (&acc)[M]) {
     constexpr int NSET = XBF16 ? 1 : (3 * M + 3) / 4;
     typedef __attribute__((address_space(3))) const u32x4* lds_v4;
@@ -244,10 +146,10 @@ __device__ __forceinline__ void group_multiply(unsigned sc, const uint4 (&cd)[2]
         bf16x8 A1[NSET], A2[NSET];
 #pragma unroll
         for (int q = 0; q < NSET; q++) {
-            A1[q] = __builtin_bit_cast(bf16x8, *(lds_v4)(a1[q] + OFF + 128 * jj));
-            A2[q] = __builtin_bit_cast(bf16x8, *(lds_v4)(a2[q] + OFF + 128 * jj));
+            A1[q] = __builtin_bit_cast(bf16x8, *(lds_v4)(a1[q] + 128 * jj));
+            A2[q] = __builtin_bit_cast(bf16x8, *(lds_v4)(a2[q] + 128 * jj));
         }
-        const uint4& c = cd[jj >> 1];
+        const u32x4 c = cd[jj >> 1];
         const bf16x8 B0 = decode8((jj & 1) ? c.z : c.x), B1 = decode8((jj & 1) ? c.w : c.y);
         const float sv = jj == 0 ? e4m3_to_f32<0>(sc) : (jj == 1 ? e4m3_to_f32<1>(sc) : (jj == 2 ? e4m3_to_f32<2>(sc) : e4m3_to_f32<3>(sc)));
         f32x4 D[NSET];
@@ -268,6 +170,217 @@ __device__ __forceinline__ void group_multiply(unsigned sc, const uint4 (&cd)[2]
         }
     }
 }
+
+// A wave's walk along its strip: groups first .. first + count - 1, RING of them in flight at any time.
+//
+//   issue<J>(g)    requests group g into ring slot J: its activations (4 columns per lane and token; every lane always loads -
+//                  a lane whose columns lie beyond K reads the row's last four instead and drops them when staging - so no load
+//                  sits behind a branch and the compiler can count the loads in flight exactly) and its 2304 weight bytes
+//   stage<J>(g)    writes slot J's activations as bf16 rows into LDS staging slot J % 2
+//   multiply<J>()  four pairs of matrix instructions on slot J against LDS slot J % 2
+//
+// Steady state, per group: stage the NEXT group (its activations were requested right behind the current group's weights, so
+// they are here once those are), multiply the current one, refill its slot with the group RING further on.  Everything is
+// unrolled by RING so that every register index, LDS offset and wait count is static; the walk ends in one of RING tails, chosen
+// by how many groups are left to request.
+template <int M, bool XBF16>
+struct StripWalk {
+    typedef Staging<M, XBF16> St;
+    static constexpr int NSET = XBF16 ? 1 : (3 * M + 3) / 4;
+    typedef typename std::conditional<XBF16, u32x2, f32x4>::type XV;  // plain vector types: they live in registers
+    unsigned sc[CROW_GEMV_RING];
+    u32x4 cd[CROW_GEMV_RING][2];
+    XV xv[CROW_GEMV_RING][M];
+    lds_p a1[2][NSET], a2[2][NSET];  // this lane's operand addresses in the two staging slots (or in the zero area)
+    lds_p xw;
+    const unsigned char* wl;  // the lane's view of the wave's first group
+    const unsigned char* xl;  // the lane's view of the wave's first column of activation row 0
+    size_t xoff[M];           // byte offsets of the activation rows
+    int col_lane, k_dim, lane;
+    float acc[M];
+
+    __device__ __forceinline__ void init(const unsigned char* strip, int first, int k_dim_, const void* x, const size_t (&xoff_elems)[M], lds_p xw_,
+                                         lds_p zero) {
+        lane = lane_id();
+        xw = xw_;
+        k_dim = k_dim_;
+        wl = strip + (size_t)first * CROW_GROUP_BYTES;
+        col_lane = first * CROW_GROUP_COLS + 4 * lane;
+        xl = (const unsigned char*)x;
+#pragma unroll
+        for (int m = 0; m < M; m++) {
+            xoff[m] = xoff_elems[m] * (XBF16 ? 2 : 4);
+            acc[m] = 0.0f;
+        }
+        // this lane as a holder of A operand row i = lane % 16, K group g = lane / 16 (K indices 8 g .. 8 g + 7)
+        const int g = lane >> 4, i = lane & 15, r4 = i & 3;
+        const bool half_ok = (g >> 1) == (i >> 3);      // the row's 16-column half is this K group's half
+        const bool second = ((i >> 2) & 1) != 0;        // rows 4..7, 12..15 belong to A2 (segment 1 of the pair: 64 bytes on)
+#pragma unroll
+        for (int s = 0; s < 2; s++)
+#pragma unroll
+            for (int q = 0; q < NSET; q++) {
+                const int row = 4 * q + r4;
+                const bool live = half_ok && row < St::XR;
+                lds_p data = xw + s * St::SLOT + row * CROW_GEMV_XROW_BYTES + 16 * g;
+                a1[s][q] = (live && !second) ? data : zero + 16 * g;
+                a2[s][q] = (live && second) ? data + 64 : zero + 16 * g;
+            }
+    }
+    // activations of group g into x slot J (g % RING == J)
+    template <int J>
+    __device__ __forceinline__ void issue_x(int g) {
+        const int col = col_lane + g * CROW_GROUP_COLS;
+        const size_t o = (size_t)(col < k_dim ? col : k_dim - 4) * (XBF16 ? 2 : 4);
+#pragma unroll
+        for (int t = 0; t < M; t++) xv[J][t] = *(const __attribute__((address_space(1))) XV*)(xl + xoff[t] + o);
+    }
+    // weights of group g into slot J
+    template <int J>
+    __device__ __forceinline__ void issue_w(int g) {
+        const unsigned char* p = wl + (size_t)g * CROW_GROUP_BYTES;
+        sc[J] = stream_load_u32((const unsigned*)p + lane);
+        cd[J][0] = stream_load_v((const uint4*)(p + CROW_GROUP_SCALE_BYTES) + lane);
+        cd[J][1] = stream_load_v((const uint4*)(p + CROW_GROUP_SCALE_BYTES + 1024) + lane);
+    }
+    template <int J>
+    __device__ __forceinline__ void stage(int g) {
+        const bool in = col_lane + g * CROW_GROUP_COLS < k_dim;
+        lds_p slot = xw + (J & 1) * St::SLOT + 8 * lane;
+#pragma unroll
+        for (int t = 0; t < M; t++) {
+            if constexpr (XBF16) {
+                lds_store8(slot + t * CROW_GEMV_XROW_BYTES, in ? xv[J][t].x : 0u, in ? xv[J][t].y : 0u);
+            } else {
+                unsigned h[4], m[4], l[4];
+                split3(in ? xv[J][t].x : 0.f, h[0], m[0], l[0]);
+                split3(in ? xv[J][t].y : 0.f, h[1], m[1], l[1]);
+                split3(in ? xv[J][t].z : 0.f, h[2], m[2], l[2]);
+                split3(in ? xv[J][t].w : 0.f, h[3], m[3], l[3]);
+                // bf16 pairs: high halves of (odd element, even element)
+                lds_p row = slot + (3 * t) * CROW_GEMV_XROW_BYTES;
+                lds_store8(row, __builtin_amdgcn_perm(h[1], h[0], 0x07060302u), __builtin_amdgcn_perm(h[3], h[2], 0x07060302u));
+                lds_store8(row + CROW_GEMV_XROW_BYTES, __builtin_amdgcn_perm(m[1], m[0], 0x07060302u), __builtin_amdgcn_perm(m[3], m[2], 0x07060302u));
+                lds_store8(row + 2 * CROW_GEMV_XROW_BYTES, __builtin_amdgcn_perm(l[1], l[0], 0x07060302u), __builtin_amdgcn_perm(l[3], l[2], 0x07060302u));
+            }
+        }
+        __builtin_amdgcn_wave_barrier();  // (the wave's LDS accesses execute in order: this only keeps the compiler from reordering them)
+    }
+    template <int J>
+    __device__ __forceinline__ void multiply() {
+        group_multiply<M, XBF16>(sc[J], cd[J], a1[J & 1], a2[J & 1], acc);
+        __builtin_amdgcn_wave_barrier();
+        // a group is one scheduling region: without the fence the scheduler pulls the decodes of several groups forward in the
+        // long straight-line tails of the walk and runs out of registers there
+        __builtin_amdgcn_sched_barrier(0);
+    }
+
+    // groups g .. g + N - 1 (N <= RING) are requested into slots 0 .. N - 1 - activations first, so that they do not queue
+    // behind the weights
+    template <int N>
+    __device__ __forceinline__ void start(int g) {
+        if (N > 0) issue_x<0>(g);
+        if (N > 1) issue_x<1>(g + 1);
+        if (N > 2) issue_x<2>(g + 2);
+        if (N > 3) issue_x<3>(g + 3);
+        if (N > 0) issue_w<0>(g);
+        if (N > 1) issue_w<1>(g + 1);
+        if (N > 2) issue_w<2>(g + 2);
+        if (N > 3) issue_w<3>(g + 3);
+    }
+    // On entry: the weights of groups g0 .. g0 + 3 are in (or on their way to) slots 0..3, group g0 is staged, the activations of
+    // g0 + 1 .. g0 + 4 are in (or on their way to) their x slots.  The quad multiplies its four groups and, if REFILL, requests
+    // the weights of the next four into the slots it frees.  The activations of groups g0 + 5 .. g0 + 8 are requested in any case,
+    // each as soon as its x slot has been staged: a request for a group beyond the wave's run reads columns that exist (or the
+    // row's last four) and is never used.  On return group g0 + 4 is staged if REFILL.
+    template <bool REFILL>
+    __device__ __forceinline__ void quad(int g0) {
+        stage<1>(g0 + 1);
+        issue_x<1>(g0 + 5);
+        multiply<0>();
+        if (REFILL) issue_w<0>(g0 + 4);
+        stage<2>(g0 + 2);
+        issue_x<2>(g0 + 6);
+        multiply<1>();
+        if (REFILL) issue_w<1>(g0 + 5);
+        stage<3>(g0 + 3);
+        issue_x<3>(g0 + 7);
+        multiply<2>();
+        if (REFILL) issue_w<2>(g0 + 6);
+        if (REFILL) {
+            stage<0>(g0 + 4);
+            issue_x<0>(g0 + 8);
+        }
+        multiply<3>();
+        if (REFILL) issue_w<3>(g0 + 7);
+    }
+    // the last N < RING groups g0 .. g0 + N - 1 sit in slots 0 .. N - 1, group g0 is staged
+    template <int N>
+    __device__ __forceinline__ void rest(int g0) {
+        if (N > 1) stage<1>(g0 + 1);
+        if (N > 0) multiply<0>();
+        if (N > 2) stage<2>(g0 + 2);
+        if (N > 1) multiply<1>();
+        if (N > 2) multiply<2>();
+    }
+    template <int N>
+    __device__ __forceinline__ void remainder(int g) {
+        start<N>(g);
+        stage<0>(g);
+        rest<N>(g);
+    }
+    // The whole walk over `count` groups: the full quads as a pipeline (every quad's loads in flight while the one before is
+    // multiplied), then what is left (count % 4 groups) on its own.  `mid` is whatever the block has to do between a wave's
+    // first requests and its first use of LDS (zeroing the zero area, a block barrier): it runs once, after the first loads
+    // have left.  Paths with different loads in flight never meet before a wait that matters, so the waits count exactly.
+    template <class Mid>
+    __device__ __forceinline__ void go(int count, Mid mid) {
+        const int nq = count >> 2, r = count & 3;
+        if (nq > 0) {
+            start<4>(0);
+            mid();
+            stage<0>(0);
+            issue_x<0>(4);
+            // (one copy of each body, and no branch whose two sides begin alike: the compiler hoists what two successors of a
+            // branch have in common, here every decode of the ring, above the branch - and runs out of registers there)
+            int q = 0;
+            for (; q + 1 < nq; q++) quad<true>(4 * q);
+            quad<false>(4 * q);
+            if (r == 3) remainder<3>(4 * nq);
+            else if (r == 2) remainder<2>(4 * nq);
+            else if (r == 1) remainder<1>(4 * nq);
+        } else if (r == 3) {
+            start<3>(0);
+            mid();
+            stage<0>(0);
+            rest<3>(0);
+        } else if (r == 2) {
+            start<2>(0);
+            mid();
+            stage<0>(0);
+            rest<2>(0);
+        } else if (r == 1) {
+            start<1>(0);
+            mid();
+            stage<0>(0);
+            rest<1>(0);
+        } else {
+            mid();
+        }
+    }
+    // out[m] in every lane l = the wave's partial dot product of strip row l % 16 with activation row m.
+    // lane (g, n) holds sub-block class 2 (g & 1) + (g >> 1) of row n: classes (0 + 1) + (2 + 3) = (g0 + g2) + (g1 + g3)
+    __device__ __forceinline__ void finish(float (&out)[M]) const {
+#pragma unroll
+        for (int m = 0; m < M; m++) {
+            const unsigned a = __float_as_uint(acc[m]);
+            const u32x2 sw = __builtin_amdgcn_permlane32_swap(a, a, false, false);  // .x = lanes 0..31's value, .y = lanes 32..63's
+            const unsigned b = __float_as_uint(__fadd_rn(__uint_as_float(sw.x), __uint_as_float(sw.y)));
+            const u32x2 sq = __builtin_amdgcn_permlane16_swap(b, b, false, false);  // .x = the even 16-lane group's value, .y = the odd one's
+            out[m] = __fadd_rn(__uint_as_float(sq.x), __uint_as_float(sq.y));
+        }
+    }
+};
 
 // Ordering point of the cross-block hand-over.  Every access to the shared partials and counters is an agent-scope atomic:
 // on gfx950 such a store / load / read-modify-write carries the coherence bit that makes it bypass the per-die L2 for
@@ -327,78 +440,15 @@ __device__ __forceinline__ bool slice_hand_over(float (&v)[NV], unsigned tile_id
     return true;
 }
 
-// out[m] in every lane l = the wave's partial dot product of strip row l % 16 with activation row m, over groups
-// first .. first + count - 1 of the strip whose group 0 is at `strip`.  `xw` is the wave's own staging area, `zero` the block's
-// zeroed area, `most` the most groups any wave of the launch owns (it fixes the staged row length).
-template <int M, bool XBF16>
-__device__ __forceinline__ void strip_accumulate(const unsigned char* strip, int first, int count, int most, int k_dim, const void* x,
-                                                 const size_t (&xoff)[M], lds_p xw, lds_p zero, float (&out)[M]) {
-    typedef Staging<M, XBF16> St;
-    constexpr int NSET = XBF16 ? 1 : (3 * M + 3) / 4, SG = St::SG;
-    const int ROW = St::row_bytes(most);
-    const int lane = lane_id();
-    // this lane as a holder of A operand row i = lane % 16, K group g = lane / 16 (K indices 8 g .. 8 g + 7)
-    const int g = lane >> 4, i = lane & 15, r4 = i & 3;
-    const bool half_ok = (g >> 1) == (i >> 3);      // the row's 16-column half is this K group's half
-    const bool second = ((i >> 2) & 1) != 0;        // rows 4..7, 12..15 belong to A2 (segment 1 of the pair: 64 bytes on)
-    lds_p a1[NSET], a2[NSET];
-#pragma unroll
-    for (int q = 0; q < NSET; q++) {
-        const int row = 4 * q + r4;
-        const bool live = half_ok && row < St::XR;
-        lds_p data = xw + row * ROW + 16 * g;
-        a1[q] = (live && !second) ? data : zero + 16 * g;
-        a2[q] = (live && second) ? data + 64 : zero + 16 * g;
-    }
-    float acc[M];
-#pragma unroll
-    for (int m = 0; m < M; m++) acc[m] = 0.0f;
-    for (int c0 = 0; c0 < count; c0 += CROW_GEMV_GMAX) {  // one trip unless the wave owns more than GMAX groups
-        const int n = count - c0 < CROW_GEMV_GMAX ? count - c0 : CROW_GEMV_GMAX;
-        const int g0 = first + c0;
-        XStage<M, XBF16> xs;
-        // fetched before the weight loads are issued so that its data does not queue behind them
-        xs.fetch(x, xoff, g0 * CROW_GROUP_COLS, k_dim, n < SG ? n : SG, lane);
-        GroupRegs r;
-        load_groups(strip + (size_t)g0 * CROW_GROUP_BYTES, n, lane, r);
-#pragma unroll
-        for (int b0 = 0; b0 < CROW_GEMV_GMAX; b0 += SG) {
-            if (b0 < n) {
-                const int nb = n - b0 < SG ? n - b0 : SG;
-                xs.store(xw, ROW, nb, lane);
-                __builtin_amdgcn_wave_barrier();  // the reads below follow the writes above in program order (same wave)
-                if (b0 + SG < n) xs.fetch(x, xoff, (g0 + b0 + SG) * CROW_GROUP_COLS, k_dim, n - b0 - SG < SG ? n - b0 - SG : SG, lane);
-#define CROW_GROUP(GG)                                                                                                               \
-    if (GG < SG && b0 + GG < CROW_GEMV_GMAX && b0 + GG < n)                                                                          \
-        group_multiply<M, XBF16, 512 * (GG < SG ? GG : 0)>(r.sc[b0 + GG < CROW_GEMV_GMAX ? b0 + GG : 0], r.cd[b0 + GG < CROW_GEMV_GMAX ? b0 + GG : 0], \
-                                                           a1, a2, acc);
-                CROW_GROUP(0) CROW_GROUP(1) CROW_GROUP(2) CROW_GROUP(3)
-#undef CROW_GROUP
-                __builtin_amdgcn_wave_barrier();  // ... and the next batch's writes follow these reads
-            }
-        }
-    }
-    // lane (g, n) holds sub-block class 2 (g & 1) + (g >> 1) of row n: classes (0 + 1) + (2 + 3) = (g0 + g2) + (g1 + g3)
-#pragma unroll
-    for (int m = 0; m < M; m++) {
-        const unsigned a = __float_as_uint(acc[m]);
-        const u32x2 sw = __builtin_amdgcn_permlane32_swap(a, a, false, false);  // .x = lanes 0..31's value, .y = lanes 32..63's
-        const unsigned b = __float_as_uint(__fadd_rn(__uint_as_float(sw.x), __uint_as_float(sw.y)));
-        const u32x2 sq = __builtin_amdgcn_permlane16_swap(b, b, false, false);  // .x = the even 16-lane group's value, .y = the odd one's
-        out[m] = __fadd_rn(__uint_as_float(sq.x), __uint_as_float(sq.y));
-    }
-}
-
 typedef __attribute__((address_space(3))) float* lds_f;
 
 // The body every GEMV entry point runs.  The caller has already offset the pointers in `a` for its token group / combo `z`,
 // which only indexes the workspace here.  `lds` is the block's dynamic LDS, laid out as described at the top of the file and
-// sized by the launcher for StagingAlloc<M_ALLOC, XBF16>: entry points that dispatch over M size it for their widest body.
+// sized by the launcher for M_ALLOC rows: entry points that dispatch over M size it for their widest body.
 template <int NR, int M, bool XBF16, int EPI, int M_ALLOC = M>
 __device__ __forceinline__ void gemv_body(const GemvArgs& a, unsigned z, lds_p lds, const Workspace& ws) {
-    typedef Staging<M, XBF16> St;
-    typedef StagingAlloc<M_ALLOC, XBF16> Alloc;
     static_assert(M <= M_ALLOC, "the allocation covers this body");
+    constexpr int AREA = crow_gemv_lds_per_wave(M_ALLOC, XBF16);
     const int lane = lane_id();
     const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6)), waves = block_threads() >> 6;  // wave-uniform on purpose
     const int strip = (int)blockIdx.x, strips = (int)gridDim.x;
@@ -410,8 +460,10 @@ __device__ __forceinline__ void gemv_body(const GemvArgs& a, unsigned z, lds_p l
     const int unit = slice * wpt + (wave - r_own * wpt), units = slices * wpt;
     // the strip's groups in runs of floor(groups / units), the first groups % units runs one longer
     const int base = groups / units, rem = groups - base * units;
-    const int count = base + (unit < rem ? 1 : 0), first = unit * base + (unit < rem ? unit : rem);
-    const int most = base + (rem > 0 ? 1 : 0);
+    // (a two-tensor block launched with an odd number of waves has one wave too many: it takes nothing, and the launch is
+    // refused at the store - not here, where the refusal would sit between a wave's start and its first weight load)
+    const bool extra_wave = NR == 2 && wave - r_own * wpt >= wpt;
+    const int count = extra_wave ? 0 : base + (unit < rem ? 1 : 0), first = unit * base + (unit < rem ? unit : rem);
     const unsigned char* wsel = r_own != 0 ? a.w[1] : a.w[0];  // a select, never an indexed read
     const unsigned char* strip_p = wsel + (size_t)strip * groups * CROW_GROUP_BYTES;
     // element offsets of this launch's activation rows, and which output row each of them writes
@@ -428,19 +480,17 @@ __device__ __forceinline__ void gemv_body(const GemvArgs& a, unsigned z, lds_p l
             yrow[m] = a.y_row0 + m;
         }
     }
-    if (NR == 2 && (waves & 1)) {  // the two tensors take half of the block's waves each (uniform over the block: nobody waits at a barrier)
-        if (threadIdx.x == 0) atomicOr(ws.status, STATUS_BAD_SHAPE);
-        return;
-    }
     lds_p zero = lds;
-    const int area_bytes = Alloc::per_wave(most);
-    lds_p areas = lds + Alloc::zero_bytes(most);
-    for (int o = 16 * (int)threadIdx.x; o < St::zero_bytes(most); o += 16 * (waves << 6)) lds_store16(zero + o, 0, 0, 0, 0);
-    if (waves > 1) __syncthreads();
-    else __builtin_amdgcn_wave_barrier();
-
+    lds_p areas = lds + CROW_GEMV_ZERO_BYTES;
+    StripWalk<M, XBF16> walk;
+    walk.init(strip_p, first, k_dim, a.x, xoff, areas + wave * AREA, zero);
+    walk.go(count, [&]() {  // (the wave's first loads have left by now)
+        for (int o = 16 * (int)threadIdx.x; o < CROW_GEMV_ZERO_BYTES; o += 16 * (waves << 6)) lds_store16(zero + o, 0, 0, 0, 0);
+        if (waves > 1) __syncthreads();
+        else __builtin_amdgcn_wave_barrier();
+    });
     float part[M];
-    strip_accumulate<M, XBF16>(strip_p, first, count, most, k_dim, a.x, xoff, areas + wave * area_bytes, zero, part);
+    walk.finish(part);
 
     // waves of the block -> wave 0: lane l of wave 0 takes output (m = l / 16, n = l % 16) and adds the waves' sums in wave order
     float v[NR];
@@ -450,15 +500,15 @@ __device__ __forceinline__ void gemv_body(const GemvArgs& a, unsigned z, lds_p l
     if (waves > 1) {
         if (lane < 16) {
 #pragma unroll
-            for (int m = 0; m < M; m++) ((lds_f)(areas + wave * area_bytes))[m * 16 + lane] = part[m];
+            for (int m = 0; m < M; m++) ((lds_f)(areas + wave * AREA))[m * 16 + lane] = part[m];
         }
         __syncthreads();
         if (wave > 0) return;
         if (mo < M) {
 #pragma unroll
             for (int r = 0; r < NR; r++) {
-                v[r] = ((lds_f)(areas + (r * wpt) * area_bytes))[lane];
-                for (int w = 1; w < wpt; w++) v[r] += ((lds_f)(areas + (r * wpt + w) * area_bytes))[lane];
+                v[r] = ((lds_f)(areas + (r * wpt) * AREA))[lane];
+                for (int w = 1; w < wpt; w++) v[r] += ((lds_f)(areas + (r * wpt + w) * AREA))[lane];
             }
         }
     } else {
@@ -471,7 +521,8 @@ __device__ __forceinline__ void gemv_body(const GemvArgs& a, unsigned z, lds_p l
     if (slices > 1 && !slice_hand_over<NR>(v, z * (unsigned)strips + (unsigned)strip, slice, slices, ws, lane)) return;
 
     const int rows = *a.rows_p;
-    if (*a.k_dim_p != k_dim || (a.count_p != nullptr && *a.count_p != a.count_expect)) {  // the launch geometry was made for another problem: nothing is stored
+    // the launch geometry was made for another problem, or the two tensors cannot share the block's waves evenly: nothing is stored
+    if (*a.k_dim_p != k_dim || (a.count_p != nullptr && *a.count_p != a.count_expect) || (NR == 2 && (waves & 1))) {
         if (lane == 0) atomicOr(ws.status, STATUS_BAD_SHAPE);
         return;
     }

@@ -19,36 +19,52 @@ using namespace crow;
 // The block's dynamic LDS (zeros, activation staging, wave hand-over: gemv.h); the launcher sizes it.
 extern __shared__ uint4 crow_dyn_lds[];
 #define LDS ((lds_p)crow_dyn_lds)
-// First statement of every GEMV entry point: the workspace descriptor is fetched with the kernel arguments, in the
-// first scalar round trip, not behind the first use of it.
+// First statement of every GEMV entry point: the workspace descriptor and ALL kernel arguments are requested together and
+// waited for once - one scalar round trip between the start of a wave and its first weight load.  Left alone the compiler
+// fetches each argument where it is first used, behind whatever wait comes before: two or three dependent round trips.
+template <typename T>
+__device__ __forceinline__ void crow_need_one(T v) {
+    asm volatile("" ::"s"(v));
+}
+__device__ __forceinline__ void crow_need_now() {}
+template <typename T, typename... R>
+__device__ __forceinline__ void crow_need_now(T v, R... rest) {
+    crow_need_one(v);
+    crow_need_now(rest...);
+}
 #define ENTER(...)                \
     const Workspace ws = g_ws;    \
-    __builtin_amdgcn_sched_barrier(0)
+    crow_need_now(ws.status, block_threads(), (int)gridDim.y, __VA_ARGS__)
+// One-row kernels are compiled for at least this many resident waves per SIMD (it bounds their registers): six on bf16
+// activations, five on f32 ones (whose sixteen registers of activations in flight do not fit the tighter bound).  Blocks are
+// five waves per tensor at K = 5120, so five and six waves per SIMD hold the same four blocks per compute unit.
+#define CROW_ONE_ROW_BF16
+#define CROW_ONE_ROW_F32
 
 // ------------------------------------------------------------------ dense GEMV (decode, one row)
 // reference: gemv_nvfp4_w, engine/src/kernels_p2.rs:355-368
-extern "C" __global__ void __launch_bounds__(1024) gemv_nvfp4_w(const unsigned char* __restrict__ w, const float* __restrict__ x,
+extern "C" __global__ void CROW_ONE_ROW_F32 __launch_bounds__(1024) gemv_nvfp4_w(const unsigned char* __restrict__ w, const float* __restrict__ x,
                                                                 const float* __restrict__ gs_ptr, float* __restrict__ y,
                                                                 const int* __restrict__ k_dim_p, const int* __restrict__ rows_p, int geo) {
-    ENTER();
+    ENTER(w, x, gs_ptr, y, k_dim_p, rows_p, geo);
     const int pairs = geo & 0xFFFFF;
     GemvArgs a = gemv_args(w, nullptr, gs_ptr, nullptr, x, 0, y, 0, pairs, k_dim_p, rows_p);
     gemv_body<1, 1, false, EPI_SCALE>(a, 0, LDS, ws);
 }
 // the same product on bf16 activations (exact widening), for models that keep their activations in bf16
-extern "C" __global__ void __launch_bounds__(1024) gemv_nvfp4_w_bf16(const unsigned char* __restrict__ w, const unsigned short* __restrict__ x,
+extern "C" __global__ void CROW_ONE_ROW_BF16 __launch_bounds__(1024) gemv_nvfp4_w_bf16(const unsigned char* __restrict__ w, const unsigned short* __restrict__ x,
                                                                      const float* __restrict__ gs_ptr, float* __restrict__ y,
                                                                      const int* __restrict__ k_dim_p, const int* __restrict__ rows_p, int geo) {
-    ENTER();
+    ENTER(w, x, gs_ptr, y, k_dim_p, rows_p, geo);
     const int pairs = geo & 0xFFFFF;
     GemvArgs a = gemv_args(w, nullptr, gs_ptr, nullptr, x, 0, y, 0, pairs, k_dim_p, rows_p);
     gemv_body<1, 1, true, EPI_SCALE>(a, 0, LDS, ws);
 }
 // reference: gemv_fp4, engine/src/kernels.rs:118-151 (+ rows_p: the reference's grid.x is the row count)
-extern "C" __global__ void __launch_bounds__(1024) gemv_fp4(const unsigned char* __restrict__ w, const float* __restrict__ x,
+extern "C" __global__ void CROW_ONE_ROW_F32 __launch_bounds__(1024) gemv_fp4(const unsigned char* __restrict__ w, const float* __restrict__ x,
                                                             const float* __restrict__ gs_ptr, float* __restrict__ y,
                                                             const int* __restrict__ k_dim_p, const int* __restrict__ rows_p, int geo) {
-    ENTER();
+    ENTER(w, x, gs_ptr, y, k_dim_p, rows_p, geo);
     const int pairs = geo & 0xFFFFF;
     GemvArgs a = gemv_args(w, nullptr, gs_ptr, nullptr, x, 0, y, 0, pairs, k_dim_p, rows_p);
     gemv_body<1, 1, false, EPI_SCALE>(a, 0, LDS, ws);
@@ -59,11 +75,11 @@ extern "C" __global__ void __launch_bounds__(1024) gemv_fp4(const unsigned char*
 // ceil(rows / 16) candidates instead of re-reading all logits.  Together they replace lm_head_row +
 // argmax_k (engine/src/gen.rs:4766-4784, engine/src/kernels.rs:4238-4260), same tie rule.
 // out_idx is only a flag here (non-null selects the fused epilogue); argmax_tiles writes it.
-extern "C" __global__ void __launch_bounds__(1024) gemv_nvfp4_w_argmax(const unsigned char* __restrict__ w, const float* __restrict__ x,
+extern "C" __global__ void CROW_ONE_ROW_F32 __launch_bounds__(1024) gemv_nvfp4_w_argmax(const unsigned char* __restrict__ w, const float* __restrict__ x,
                                                                        const float* __restrict__ gs_ptr, float* __restrict__ y,
                                                                        const int* __restrict__ k_dim_p, const int* __restrict__ rows_p,
                                                                        int* __restrict__ out_idx, int geo) {
-    ENTER();
+    ENTER(w, x, gs_ptr, y, k_dim_p, rows_p, out_idx, geo);
     const int pairs = geo & 0xFFFFF;
     GemvArgs a = gemv_args(w, nullptr, gs_ptr, nullptr, x, 0, y, 0, pairs, k_dim_p, rows_p);
     a.argmax_out = out_idx;
@@ -72,22 +88,22 @@ extern "C" __global__ void __launch_bounds__(1024) gemv_nvfp4_w_argmax(const uns
 
 // ------------------------------------------------------------------ fused gate/up + SiLU (decode)
 // reference: gemv_nvfp4_gu, engine/src/kernels_p2.rs:372-389
-extern "C" __global__ void __launch_bounds__(1024) gemv_nvfp4_gu(const unsigned char* __restrict__ wg, const unsigned char* __restrict__ wu,
+extern "C" __global__ void CROW_ONE_ROW_F32 __launch_bounds__(1024) gemv_nvfp4_gu(const unsigned char* __restrict__ wg, const unsigned char* __restrict__ wu,
                                                                  const float* __restrict__ x, const float* __restrict__ gs_g,
                                                                  const float* __restrict__ gs_u, float* __restrict__ y,
                                                                  const int* __restrict__ k_dim_p, const int* __restrict__ rows_p, int geo) {
-    ENTER();
+    ENTER(wg, wu, x, gs_g, gs_u, y, k_dim_p, rows_p, geo);
     const int pairs = geo & 0xFFFFF;
     GemvArgs a = gemv_args(wg, wu, gs_g, gs_u, x, 0, y, 0, pairs, k_dim_p, rows_p);
     gemv_body<2, 1, false, EPI_SILU_GU>(a, 0, LDS, ws);
 }
 
 // the same on bf16 activations (exact widening)
-extern "C" __global__ void __launch_bounds__(1024) gemv_nvfp4_gu_bf16(const unsigned char* __restrict__ wg, const unsigned char* __restrict__ wu,
+extern "C" __global__ void CROW_ONE_ROW_BF16 __launch_bounds__(1024) gemv_nvfp4_gu_bf16(const unsigned char* __restrict__ wg, const unsigned char* __restrict__ wu,
                                                                       const unsigned short* __restrict__ x, const float* __restrict__ gs_g,
                                                                       const float* __restrict__ gs_u, float* __restrict__ y,
                                                                       const int* __restrict__ k_dim_p, const int* __restrict__ rows_p, int geo) {
-    ENTER();
+    ENTER(wg, wu, x, gs_g, gs_u, y, k_dim_p, rows_p, geo);
     const int pairs = geo & 0xFFFFF;
     GemvArgs a = gemv_args(wg, wu, gs_g, gs_u, x, 0, y, 0, pairs, k_dim_p, rows_p);
     gemv_body<2, 1, true, EPI_SILU_GU>(a, 0, LDS, ws);
@@ -119,22 +135,22 @@ __device__ __forceinline__ int rows_of(GemvArgs& a, int geo, const int* m_p) {
 }
 // x [M][k_dim] and y [M][rows] in place: the strides are K (by value) and the row count (needed before the first store only)
 // reference: gemv_nvfp4_wm, engine/src/kernels_p2.rs:472-497
-extern "C" __global__ void __launch_bounds__(1024) gemv_nvfp4_wm(const unsigned char* __restrict__ w, const float* __restrict__ x,
+extern "C" __global__ void __launch_bounds__(512) gemv_nvfp4_wm(const unsigned char* __restrict__ w, const float* __restrict__ x,
                                                                  const float* __restrict__ gs_ptr, float* __restrict__ y,
                                                                  const int* __restrict__ k_dim_p, const int* __restrict__ rows_p,
                                                                  const int* __restrict__ m_p, int geo) {
-    ENTER();
+    ENTER(w, x, gs_ptr, y, k_dim_p, rows_p, m_p, geo);
     const int pairs = geo & 0xFFFFF;
     GemvArgs a = gemv_args(w, nullptr, gs_ptr, nullptr, x, (size_t)pairs * CROW_PAIR_COLS, y, 0, pairs, k_dim_p, rows_p);
     gemv_m_dispatch<1, false, EPI_SCALE>(a, rows_of(a, geo, m_p), 0, LDS, ws);
 }
 // reference: gemv_nvfp4_gum, engine/src/kernels_p2.rs:499-530
-extern "C" __global__ void __launch_bounds__(1024) gemv_nvfp4_gum(const unsigned char* __restrict__ wg, const unsigned char* __restrict__ wu,
+extern "C" __global__ void __launch_bounds__(512) gemv_nvfp4_gum(const unsigned char* __restrict__ wg, const unsigned char* __restrict__ wu,
                                                                    const float* __restrict__ x, const float* __restrict__ gs_g,
                                                                    const float* __restrict__ gs_u, float* __restrict__ y,
                                                                    const int* __restrict__ k_dim_p, const int* __restrict__ rows_p,
                                                                    const int* __restrict__ m_p, int geo) {
-    ENTER();
+    ENTER(wg, wu, x, gs_g, gs_u, y, k_dim_p, rows_p, m_p, geo);
     const int pairs = geo & 0xFFFFF;
     GemvArgs a = gemv_args(wg, wu, gs_g, gs_u, x, (size_t)pairs * CROW_PAIR_COLS, y, 0, pairs, k_dim_p, rows_p);
     gemv_m_dispatch<2, false, EPI_SILU_GU>(a, rows_of(a, geo, m_p), 0, LDS, ws);
@@ -144,7 +160,7 @@ extern "C" __global__ void __launch_bounds__(1024) gemv_nvfp4_wm_bf16(const unsi
                                                                       const float* __restrict__ gs_ptr, float* __restrict__ y,
                                                                       const int* __restrict__ k_dim_p, const int* __restrict__ rows_p,
                                                                       const int* __restrict__ m_p, int geo) {
-    ENTER();
+    ENTER(w, x, gs_ptr, y, k_dim_p, rows_p, m_p, geo);
     const int pairs = geo & 0xFFFFF;
     GemvArgs a = gemv_args(w, nullptr, gs_ptr, nullptr, x, (size_t)pairs * CROW_PAIR_COLS, y, 0, pairs, k_dim_p, rows_p);
     gemv_m_dispatch<1, true, EPI_SCALE>(a, rows_of(a, geo, m_p), 0, LDS, ws);
@@ -154,7 +170,7 @@ extern "C" __global__ void __launch_bounds__(1024) gemv_nvfp4_gum_bf16(const uns
                                                                        const float* __restrict__ gs_u, float* __restrict__ y,
                                                                        const int* __restrict__ k_dim_p, const int* __restrict__ rows_p,
                                                                        const int* __restrict__ m_p, int geo) {
-    ENTER();
+    ENTER(wg, wu, x, gs_g, gs_u, y, k_dim_p, rows_p, m_p, geo);
     const int pairs = geo & 0xFFFFF;
     GemvArgs a = gemv_args(wg, wu, gs_g, gs_u, x, (size_t)pairs * CROW_PAIR_COLS, y, 0, pairs, k_dim_p, rows_p);
     gemv_m_dispatch<2, true, EPI_SILU_GU>(a, rows_of(a, geo, m_p), 0, LDS, ws);
@@ -184,25 +200,25 @@ __device__ __forceinline__ void gemv_tokens(const unsigned char* w, const float*
     }
     gemv_m_dispatch<1, false, EPI_SCALE>(a, m, blockIdx.z, LDS, ws);
 }
-extern "C" __global__ void __launch_bounds__(1024) gemv_fp4_b(const unsigned char* __restrict__ w, const float* __restrict__ x,
+extern "C" __global__ void __launch_bounds__(512) gemv_fp4_b(const unsigned char* __restrict__ w, const float* __restrict__ x,
                                                               const float* __restrict__ gs_ptr, float* __restrict__ y,
                                                               const int* __restrict__ k_dim_p, const int* __restrict__ rows_p,
                                                               const int* __restrict__ t_p, int geo) {
-    ENTER();
+    ENTER(w, x, gs_ptr, y, k_dim_p, rows_p, t_p, geo);
     gemv_tokens(w, x, gs_ptr, y, geo, k_dim_p, rows_p, t_p, 0, ws);
 }
-extern "C" __global__ void __launch_bounds__(1024) gemv_fp4_b1k(const unsigned char* __restrict__ w, const float* __restrict__ x,
+extern "C" __global__ void __launch_bounds__(512) gemv_fp4_b1k(const unsigned char* __restrict__ w, const float* __restrict__ x,
                                                                 const float* __restrict__ gs_ptr, float* __restrict__ y,
                                                                 const int* __restrict__ k_dim_p, const int* __restrict__ rows_p,
                                                                 const int* __restrict__ t_p, int geo) {
-    ENTER();
+    ENTER(w, x, gs_ptr, y, k_dim_p, rows_p, t_p, geo);
     gemv_tokens(w, x, gs_ptr, y, geo, k_dim_p, rows_p, t_p, 0, ws);
 }
-extern "C" __global__ void __launch_bounds__(1024) gemv_fp4_bs(const unsigned char* __restrict__ w, const float* __restrict__ x,
+extern "C" __global__ void __launch_bounds__(512) gemv_fp4_bs(const unsigned char* __restrict__ w, const float* __restrict__ x,
                                                                const float* __restrict__ gs_ptr, float* __restrict__ y,
                                                                const int* __restrict__ k_dim_p, const int* __restrict__ y_stride_p,
                                                                const int* __restrict__ rows_p, const int* __restrict__ t_p, int geo) {
-    ENTER();
+    ENTER(w, x, gs_ptr, y, k_dim_p, y_stride_p, rows_p, t_p, geo);
     const int y_stride = *y_stride_p;
     if (y_stride < *rows_p) {  // rows of y would overlap: refuse (uniform over the launch)
         if (threadIdx.x == 0) atomicOr(ws.status, STATUS_BAD_SHAPE);
@@ -222,11 +238,11 @@ extern "C" __global__ void __launch_bounds__(1024) gemv_fp4_bs(const unsigned ch
     }
 // reference: gemv_fp4_ptrb, engine/src/kernels.rs:195-233.  grid.z = combo; ptrs[combo] is the
 // device address of that combo's expert matrix in the tiled layout; x row = combo / x_div.
-extern "C" __global__ void __launch_bounds__(1024) gemv_fp4_ptrb(const unsigned long long* __restrict__ ptrs, const float* __restrict__ x,
+extern "C" __global__ void CROW_ONE_ROW_F32 __launch_bounds__(1024) gemv_fp4_ptrb(const unsigned long long* __restrict__ ptrs, const float* __restrict__ x,
                                                                  const float* __restrict__ gs_ptr, float* __restrict__ y,
                                                                  const int* __restrict__ k_dim_p, const int* __restrict__ x_div_p,
                                                                  const int* __restrict__ x_stride_p, const int* __restrict__ rows_p, int geo) {
-    ENTER();
+    ENTER(ptrs, x, gs_ptr, y, k_dim_p, x_div_p, x_stride_p, rows_p, geo);
     const int pairs = geo & 0xFFFFF;
     const int combo = (int)blockIdx.z;
     const unsigned char* w = (const unsigned char*)ptrs[combo];
@@ -242,11 +258,11 @@ extern "C" __global__ void __launch_bounds__(1024) gemv_fp4_ptrb(const unsigned 
 __device__ __forceinline__ size_t up_offset(int inter, int pairs) {
     return (size_t)(inter / CROW_STRIP_ROWS) * ((pairs + CROW_GROUP_PAIRS - 1) / CROW_GROUP_PAIRS) * CROW_GROUP_BYTES;
 }
-extern "C" __global__ void __launch_bounds__(1024) moe_gate_up_silu(const unsigned long long* __restrict__ ptrs, const float* __restrict__ x,
+extern "C" __global__ void CROW_ONE_ROW_F32 __launch_bounds__(1024) moe_gate_up_silu(const unsigned long long* __restrict__ ptrs, const float* __restrict__ x,
                                                                     const float* __restrict__ gs_ptr, float* __restrict__ h,
                                                                     const int* __restrict__ k_dim_p, const int* __restrict__ x_div_p,
                                                                     const int* __restrict__ x_stride_p, const int* __restrict__ inter_p, int geo) {
-    ENTER();
+    ENTER(ptrs, x, gs_ptr, h, k_dim_p, x_div_p, x_stride_p, inter_p, geo);
     const int pairs = geo & 0xFFFFF;
     const int combo = (int)blockIdx.z, inter = *inter_p;  // (arrives with ptrs[combo]: no round trip of its own)
     const unsigned char* w = (const unsigned char*)ptrs[combo];
@@ -263,39 +279,39 @@ extern "C" __global__ void __launch_bounds__(1024) moe_gate_up_silu(const unsign
 // Fused routed down projection + weighted combine: y[t][row] += sum_j rw[t][j] * (gs * <down_{e(t,j)} row, h[t K + j]>),
 // j ascending, each product and each add rounded on its own - the arithmetic of gemv_fp4_ptrb(down)
 // followed by acc_combo (engine/src/gen.rs:4527-4531, engine/src/kernels.rs:1583-1592) in one launch.
-// grid (ceil(H / 16), 1, T), block 64 * topk: wave j of a block takes combo t K + j and ALL columns of its strip
-// (1024 columns at a time; longer rows loop).
+// grid (ceil(H / 16), 1, T), block 64 * topk: wave j of a block takes combo t K + j and ALL columns of its strip.
 extern "C" __global__ void __launch_bounds__(1024) moe_down_combine(const unsigned long long* __restrict__ ptrs, const float* __restrict__ h,
                                                                     const float* __restrict__ gs_ptr, const float* __restrict__ rw,
                                                                     float* __restrict__ y, const int* __restrict__ k_dim_p,
                                                                     const int* __restrict__ rows_p, int geo) {
-    ENTER();
+    ENTER(ptrs, h, gs_ptr, rw, y, k_dim_p, rows_p, geo);
     const int pairs = geo & 0xFFFFF;
-    typedef Staging<1, false> St;
+    constexpr int AREA = crow_gemv_lds_per_wave(1, false);
     const int topk = block_threads() >> 6;
     if (topk != g_geo.topk || topk > 16) {
         if (threadIdx.x == 0) atomicOr(ws.status, STATUS_BAD_GEO);
         return;
     }
     const int k = pairs * CROW_PAIR_COLS, groups = (pairs + CROW_GROUP_PAIRS - 1) / CROW_GROUP_PAIRS;
-    const int most = groups < CROW_GEMV_GMAX ? groups : CROW_GEMV_GMAX;
     const int t = (int)blockIdx.z, strip = (int)blockIdx.x, j = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6)), lane = lane_id();
     const int combo = t * topk + j;
     // dynamic LDS: zeros, then one f32 one-row staging area per wave; a wave's weighted result for wave 0 goes where its staged
     // activations were
-    lds_p zero = LDS, areas = LDS + St::zero_bytes(most);
-    const int area_bytes = St::per_wave(most);
-    for (int o = 16 * (int)threadIdx.x; o < St::zero_bytes(most); o += 16 * (topk << 6)) lds_store16(zero + o, 0, 0, 0, 0);
-    __syncthreads();
+    lds_p zero = LDS, areas = LDS + CROW_GEMV_ZERO_BYTES;
     const unsigned char* w = (const unsigned char*)ptrs[combo];
-    float acc[1] = {0.0f};
     const size_t xoff[1] = {0};
-    if (w != nullptr) {
-        strip_accumulate<1, false>(w + (size_t)strip * groups * CROW_GROUP_BYTES, 0, groups, most, k, h + (size_t)combo * k, xoff, areas + j * area_bytes, zero, acc);
-    } else if (lane == 0) {  // a routing launch that refused its geometry left zeros behind: no weights to read; the wave
-        atomicOr(ws.status, STATUS_BAD_GEO);  // still joins the barrier below
-    }
-    if (lane < 16) ((lds_f)(areas + j * area_bytes))[lane] = rw[combo] * (acc[0] * gs_ptr[0]);
+    StripWalk<1, false> walk;
+    // a routing launch that refused its geometry left zeros behind: no weights to read; the wave still joins the barriers below
+    const int count = w != nullptr ? groups : 0;
+    walk.init(w + (size_t)strip * groups * CROW_GROUP_BYTES, 0, k, h + (size_t)combo * k, xoff, areas + j * AREA, zero);
+    walk.go(count, [&]() {
+        for (int o = 16 * (int)threadIdx.x; o < CROW_GEMV_ZERO_BYTES; o += 16 * (topk << 6)) lds_store16(zero + o, 0, 0, 0, 0);
+        __syncthreads();
+    });
+    float acc[1];
+    walk.finish(acc);
+    if (w == nullptr && lane == 0) atomicOr(ws.status, STATUS_BAD_GEO);
+    if (lane < 16) ((lds_f)(areas + j * AREA))[lane] = rw[combo] * (acc[0] * gs_ptr[0]);
     __syncthreads();
     const int rows = *rows_p, row = strip * CROW_STRIP_ROWS + lane;
     if (j != 0 || lane >= 16 || row >= rows) return;
@@ -304,7 +320,7 @@ extern "C" __global__ void __launch_bounds__(1024) moe_down_combine(const unsign
         return;
     }
     float sum = 0.0f;
-    for (int q = 0; q < topk; q++) sum = __fadd_rn(sum, ((lds_f)(areas + q * area_bytes))[lane]);
+    for (int q = 0; q < topk; q++) sum = __fadd_rn(sum, ((lds_f)(areas + q * AREA))[lane]);
     y[(size_t)t * rows + row] += sum;
 }
 
@@ -316,13 +332,13 @@ extern "C" __global__ void __launch_bounds__(1024) moe_down_combine(const unsign
 // blocks of tiles >= *n_tiles_p leave at once.  tiles[z] = (expert, first position in perm, combos, 0); table[2 e] /
 // table[2 e + 1] = gate|up / down slab of expert e (the router's table).  Row m of a tile is combo c = perm[first + m]:
 // it reads activation row c / *x_div_p and writes output row c.
-extern "C" __global__ void __launch_bounds__(1024) moe_gate_up_silu_grouped(const int4* __restrict__ tiles, const int* __restrict__ n_tiles_p,
+extern "C" __global__ void __launch_bounds__(512) moe_gate_up_silu_grouped(const int4* __restrict__ tiles, const int* __restrict__ n_tiles_p,
                                                                              const int* __restrict__ perm, const unsigned long long* __restrict__ table,
                                                                              const float* __restrict__ x, const float* __restrict__ gs_ptr,
                                                                              float* __restrict__ h, const int* __restrict__ k_dim_p,
                                                                              const int* __restrict__ x_div_p, const int* __restrict__ x_stride_p,
                                                                              const int* __restrict__ inter_p, int geo) {
-    ENTER();
+    ENTER(tiles, n_tiles_p, perm, table, x, gs_ptr, h, k_dim_p, x_div_p, x_stride_p, inter_p, geo);
     const int pairs = geo & 0xFFFFF;
     const int z = (int)blockIdx.z;
     if (z >= *n_tiles_p) return;
@@ -339,12 +355,12 @@ extern "C" __global__ void __launch_bounds__(1024) moe_gate_up_silu_grouped(cons
     gemv_m_dispatch<2, false, EPI_SILU_GU>(a, tl.z, blockIdx.z, LDS, ws);
 }
 // down slabs: x = h [combos][k_dim], y = eo [combos][rows]; acc_combo then adds the weighted rows per token
-extern "C" __global__ void __launch_bounds__(1024) moe_down_grouped(const int4* __restrict__ tiles, const int* __restrict__ n_tiles_p,
+extern "C" __global__ void __launch_bounds__(512) moe_down_grouped(const int4* __restrict__ tiles, const int* __restrict__ n_tiles_p,
                                                                     const int* __restrict__ perm, const unsigned long long* __restrict__ table,
                                                                     const float* __restrict__ h, const float* __restrict__ gs_ptr,
                                                                     float* __restrict__ eo, const int* __restrict__ k_dim_p,
                                                                     const int* __restrict__ rows_p, int geo) {
-    ENTER();
+    ENTER(tiles, n_tiles_p, perm, table, h, gs_ptr, eo, k_dim_p, rows_p, geo);
     const int pairs = geo & 0xFFFFF;
     const int z = (int)blockIdx.z;
     if (z >= *n_tiles_p) return;
