@@ -323,10 +323,20 @@ int crow_hip_launch_dims_split(const char* name, uint32_t rows, uint32_t k_dim, 
         }
         if (verify && z > 4) return CROW_ERR_SHAPE;
         const uint32_t wmax = (uint32_t)e->max_waves / (uint32_t)e->nr;  // waves per tensor in a block
-        // A wave walks its run of groups with four of them (9 KB) in flight; few long walks beat many short ones (measured:
-        // every wave pays its start, its staging set-up and the block's meeting in LDS once).  One block holds a whole strip
-        // whatever K is: there is no cross-block split unless it is asked for.
-        uint32_t w = (groups + 3 * CROW_GEMV_RING - 1) / (3 * CROW_GEMV_RING), s = 1;  // about twelve groups (27 KB) per wave
+        // A wave walks its run of groups with four of them (9 KB) in flight; few long walks beat many short ones (every wave
+        // pays its start, its staging set-up and the block's meeting in LDS once), as long as the launch still has a few
+        // thousand waves.  Measured on MI355X: [17408, 5120] one tensor 3 waves per strip (7 groups each), two tensors 2 + 2
+        // (10 groups each); [5120, 17408] (68 groups, only 320 strips) 5 slices of 4 waves, which meet through the workspace.
+        // A strip stays inside one block up to 64 groups (K = 16384).
+        uint32_t w, s;
+        if (groups <= 64) {
+            const uint32_t per_wave = e->nr == 2 ? 10 : 7;
+            w = (groups + per_wave - 1) / per_wave;
+            s = 1;
+        } else {
+            w = 4;
+            s = (groups + 13) / 14;
+        }
         if (force_s > 0) s = force_s;
         if (force_w > 0) w = force_w;
         if (w > wmax) w = wmax;
