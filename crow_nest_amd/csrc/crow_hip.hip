@@ -65,7 +65,6 @@ struct State {
 
 const unsigned long long PARTIAL_FLOATS = 16ull << 20;  // 64 MiB of split-K partial sums
 const unsigned COUNTER_SLOTS = 1u << 16;
-const unsigned AM_SLOTS = 1u << 16;
 // tile counters, then the status word
 const unsigned COUNTER_WORDS = COUNTER_SLOTS + 1;
 
@@ -136,21 +135,19 @@ int crow_hip_init(int device) {
     crow::Workspace ws{};
     ws.partial_floats = PARTIAL_FLOATS;
     ws.counter_slots = COUNTER_SLOTS;
-    ws.am_slots = AM_SLOTS;
     int* scalars = nullptr;
     // one failure path: everything allocated so far is released again
     auto fail = [&](hipError_t why) {
         (void)hipFree(ws.partials);
         (void)hipFree(ws.counters);
-        (void)hipFree(ws.am_val);
-        (void)hipFree(ws.am_idx);
+        (void)hipFree(ws.am_key);
         (void)hipFree(scalars);
         return (int)why;
     };
     if ((e = hipMalloc((void**)&ws.partials, PARTIAL_FLOATS * sizeof(float))) != hipSuccess) return fail(e);
     if ((e = hipMalloc((void**)&ws.counters, COUNTER_WORDS * sizeof(unsigned))) != hipSuccess) return fail(e);
-    if ((e = hipMalloc((void**)&ws.am_val, AM_SLOTS * sizeof(float))) != hipSuccess) return fail(e);
-    if ((e = hipMalloc((void**)&ws.am_idx, AM_SLOTS * sizeof(int))) != hipSuccess) return fail(e);
+    if ((e = hipMalloc((void**)&ws.am_key, sizeof(unsigned long long))) != hipSuccess) return fail(e);
+    if ((e = hipMemset(ws.am_key, 0, sizeof(unsigned long long))) != hipSuccess) return fail(e);
     if ((e = hipMalloc((void**)&scalars, 16 * sizeof(int))) != hipSuccess) return fail(e);
     if ((e = hipMemset(ws.counters, 0, COUNTER_WORDS * sizeof(unsigned))) != hipSuccess) return fail(e);
     ws.status = ws.counters + COUNTER_SLOTS;
@@ -182,8 +179,7 @@ int crow_hip_shutdown(void) {
     (void)hipDeviceSynchronize();
     (void)hipFree(g.ws.partials);
     (void)hipFree(g.ws.counters);
-    (void)hipFree(g.ws.am_val);
-    (void)hipFree(g.ws.am_idx);
+    (void)hipFree(g.ws.am_key);
     (void)hipFree(g.scalars);
     g = State{};
     return CROW_OK;
@@ -349,7 +345,6 @@ int crow_hip_launch_dims_split(const char* name, uint32_t rows, uint32_t k_dim, 
         const uint32_t hint = verify ? z : (tokens ? (z - 1) % 4 + 1 : 0);
         *out = crow_dims{strips, pairs | (hint << 20) | (s << 24), gz, 64u * w * (uint32_t)e->nr};
         if (s > 1 && ((unsigned long long)strips * gz * s * 2 * 64 > PARTIAL_FLOATS || (unsigned long long)strips * gz > COUNTER_SLOTS)) return CROW_ERR_WORKSPACE;
-        if (strcmp(name, "gemv_nvfp4_w_argmax") == 0 && strips > AM_SLOTS) return CROW_ERR_WORKSPACE;
         return CROW_OK;
     }
     if (strncmp(name, "gemm_nvfp4_bf16", 15) == 0) {  // z = M token rows
@@ -377,7 +372,7 @@ int crow_hip_launch_dims_split(const char* name, uint32_t rows, uint32_t k_dim, 
     if (strcmp(name, "router_top10") == 0) { *out = crow_dims{z, 1, 1, 64}; return CROW_OK; }
     if (strcmp(name, "moe_group") == 0) { *out = crow_dims{1, 1, 1, 1024}; return CROW_OK; }
     if (strcmp(name, "argmax_k") == 0) { *out = crow_dims{1, 1, 1, 1024}; return CROW_OK; }
-    if (strcmp(name, "argmax_tiles") == 0) { *out = crow_dims{1, 1, 1, 256}; return CROW_OK; }
+    if (strcmp(name, "argmax_tiles") == 0) { *out = crow_dims{1, 1, 1, 64}; return CROW_OK; }
     if (strcmp(name, "acc_combo") == 0) { *out = crow_dims{(rows + 255) / 256, z, 1, 256}; return CROW_OK; }  // rows = hidden
     if (strcmp(name, "silu_mul_combo") == 0 || strcmp(name, "dequant_fp4_flat") == 0) {  // rows = element count
         *out = crow_dims{(rows + 255) / 256, 1, 1, 256};
@@ -402,6 +397,7 @@ int crow_hip_status(void) {
     (void)hipMemset(g.ws.status, 0, sizeof st);
     // a launch that bailed out may have left arrival counters behind
     (void)hipMemset(g.ws.counters, 0, COUNTER_WORDS * sizeof(unsigned));
+    (void)hipMemset(g.ws.am_key, 0, sizeof(unsigned long long));  // ... or a head's candidates without their stage 2
     if (st & CROW_STATUS_BAD_SCALE_BYTE) return CROW_ERR_SCALE_BYTE;
     if (st & crow::STATUS_WORKSPACE_TOO_SMALL) return CROW_ERR_WORKSPACE;
     if (st & crow::STATUS_BAD_GEO) return CROW_ERR_GEO;
@@ -412,6 +408,7 @@ int crow_hip_reset_workspace(void) {
     if (!g.ready) return CROW_ERR_NOT_INITIALIZED;
     hipError_t e = hipDeviceSynchronize();
     if (e != hipSuccess) return (int)e;
+    if ((e = hipMemset(g.ws.am_key, 0, sizeof(unsigned long long))) != hipSuccess) return (int)e;
     return hip_rc(hipMemset(g.ws.counters, 0, COUNTER_WORDS * sizeof(unsigned)));
 }
 

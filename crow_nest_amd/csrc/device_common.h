@@ -46,9 +46,7 @@ struct Workspace {
     unsigned long long partial_floats;  // capacity of `partials`
     unsigned counter_slots;             // capacity of `counters`
     unsigned* status;                   // device word: non-zero = a launch did not fit the workspace
-    float* am_val;                      // fused lm_head argmax: one (value, index) candidate per row tile
-    int* am_idx;
-    unsigned am_slots;
+    unsigned long long* am_key;         // fused lm_head argmax: the best (value, index) so far as one ordered 64-bit key; 0 = none
 };
 __device__ Workspace g_ws;
 
@@ -98,6 +96,19 @@ struct Best {
 __device__ __forceinline__ bool better(float v, int i, float bv, int bi) {
     const unsigned ki = __brev((unsigned)i & 1023u), kb = __brev((unsigned)bi & 1023u);
     return v > bv || (v == bv && (ki < kb || (ki == kb && i < bi)));
+}
+// The same order as ONE unsigned 64-bit key, larger = better: the value's bits made monotonic (sign flipped for positive
+// floats, all bits for negative ones) above the complement of (bit-reversed (i mod 1024), i / 1024).  A 64-bit atomic maximum
+// over such keys is the tournament, whatever the arrival order.  No key of a real candidate is 0.
+__device__ __forceinline__ unsigned long long best_key(float v, int i) {
+    const unsigned u = __float_as_uint(v);
+    const unsigned hi = (u & 0x80000000u) ? ~u : (u | 0x80000000u);
+    const unsigned tie = ((__brev((unsigned)i & 1023u) >> 22) << 22) | ((unsigned)i >> 10);
+    return ((unsigned long long)hi << 32) | (unsigned long long)(0xFFFFFFFFu - tie);
+}
+__device__ __forceinline__ int best_key_index(unsigned long long key) {
+    const unsigned tie = 0xFFFFFFFFu - (unsigned)(key & 0xFFFFFFFFull);
+    return (int)(((tie & 0x3FFFFFu) << 10) | (__brev(tie >> 22) >> 22));
 }
 __device__ __forceinline__ Best wave_best(Best b) {
     for (int o = 32; o > 0; o >>= 1) {

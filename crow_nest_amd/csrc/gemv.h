@@ -528,20 +528,13 @@ __device__ __forceinline__ void gemv_body(const GemvArgs& a, unsigned z, lds_p l
     }
     const int row = strip * CROW_STRIP_ROWS + n;
     if (EPI == EPI_SCALE && a.argmax_out != nullptr) {
-        // fused head, stage 1: logits out and one (value, index) candidate per strip into the workspace, plain stores, no
-        // waiting.  Stage 2 is argmax_tiles.
+        // fused head, stage 1: logits out, and the strip's best (value, index) folded into the library's key word with one
+        // 64-bit atomic maximum that nobody waits for.  Stage 2 (argmax_tiles) decodes the key and clears it.
         const float val = v[0] * a.gs[0][0];
         const bool live = mo == 0 && row < rows;
         if (live) a.y[row] = val;
         const Best b = wave_best(Best{live ? val : -3.0e38f, live ? row : 0});
-        if ((unsigned)strips > ws.am_slots) {
-            if (lane == 0) atomicOr(ws.status, STATUS_WORKSPACE_TOO_SMALL);
-            return;
-        }
-        if (lane == 0) {
-            ws.am_val[strip] = b.v;
-            ws.am_idx[strip] = b.i;
-        }
+        if (lane == 0) __hip_atomic_fetch_max(ws.am_key, best_key(b.v, b.i), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         return;
     }
     if (mo >= M || row >= rows) return;

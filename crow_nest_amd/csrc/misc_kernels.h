@@ -467,37 +467,15 @@ extern "C" __global__ void __launch_bounds__(1024) argmax_k(const float* __restr
     }
 }
 
-// Stage 2 of the fused head: the greedy token from the per-strip candidates gemv_nvfp4_w_argmax left in
-// the workspace (ceil(rows / 16) of them).  grid (1), block 256.  Same total order as argmax_k.
+// Stage 2 of the fused head: the greedy token out of the key word gemv_nvfp4_w_argmax's blocks folded their candidates into
+// (device_common.h: same total order as argmax_k), and the word cleared for the next head.  grid (1), block 64.
+// (rows_p is unused: kept so that the call site's value list stays as it was.)
 extern "C" __global__ void __launch_bounds__(256) argmax_tiles(int* __restrict__ out, const int* __restrict__ rows_p) {
-    __shared__ float sv[4];
-    __shared__ int si[4];
-    const Workspace ws = g_ws;
-    const int tiles = (*rows_p + CROW_STRIP_ROWS - 1) / CROW_STRIP_ROWS;
-    Best b{-3.0e38f, 0};
-    for (int t = (int)threadIdx.x; t < tiles && t < (int)ws.am_slots; t += 256) {
-        const float v = ws.am_val[t];
-        const int i = ws.am_idx[t];
-        if (better(v, i, b.v, b.i)) {
-            b.v = v;
-            b.i = i;
-        }
-    }
-    b = wave_best(b);
-    const int wave = (int)(threadIdx.x >> 6);
-    if (lane_id() == 0) {
-        sv[wave] = b.v;
-        si[wave] = b.i;
-    }
-    __syncthreads();
-    if (threadIdx.x == 0) {
-        for (int w = 1; w < 4; w++)
-            if (better(sv[w], si[w], b.v, b.i)) {
-                b.v = sv[w];
-                b.i = si[w];
-            }
-        out[0] = b.i;
-    }
+    if (threadIdx.x != 0) return;
+    unsigned long long* key = g_ws.am_key;
+    const unsigned long long k = __hip_atomic_load(key, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    out[0] = k != 0ull ? best_key_index(k) : 0;
+    __hip_atomic_store(key, 0ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
 // ------------------------------------------------------------------ BF16 and F32 keeps
