@@ -22,13 +22,14 @@ struct FnEntry {
     int nr;
     int max_waves;  // per block (the kernel's launch bound)
     int lds_per_wave;
+    bool takes_ws;  // the launcher appends the scratch descriptor (every kernel of the GEMV family, and argmax_tiles)
 };
 
-#define CROW_FN(name, nargs) {#name, (const void*)&name, nargs, 0u, 0, 16, 0}
+#define CROW_FN(name, nargs) {#name, (const void*)&name, nargs, 0u, 0, 16, 0, false}
 // NR tensors per block, bodies for 1 .. MMAX activation rows, bf16 or f32 activations
 // (the bodies for several f32 rows need more registers than a block of sixteen waves leaves each: they run in blocks of eight)
 #define CROW_GEMV(name, nargs, NR, MMAX, XBF16) \
-    {#name, (const void*)&name, nargs, 0u, NR, (MMAX > 1 && !XBF16) ? 8 : 16, crow::crow_gemv_lds_per_wave(MMAX, XBF16)}
+    {#name, (const void*)&name, nargs, 0u, NR, (MMAX > 1 && !XBF16) ? 8 : 16, crow::crow_gemv_lds_per_wave(MMAX, XBF16), true}
 const FnEntry g_table[] = {
     CROW_GEMV(gemv_nvfp4_w, 6, 1, 1, false),       CROW_GEMV(gemv_nvfp4_w_bf16, 6, 1, 1, true),  CROW_GEMV(gemv_nvfp4_w_argmax, 7, 1, 1, false),
     CROW_GEMV(gemv_nvfp4_gu, 8, 2, 1, false),      CROW_GEMV(gemv_nvfp4_gu_bf16, 8, 2, 1, true),
@@ -39,13 +40,13 @@ const FnEntry g_table[] = {
     CROW_GEMV(moe_route_gate_up_silu, 11, 2, 1, false), CROW_GEMV(moe_gate_up_silu_grouped, 11, 2, 4, false), CROW_GEMV(moe_down_grouped, 9, 1, 4, false),
     CROW_FN(moe_group, 6),
     CROW_FN(router_top10, 10),     CROW_FN(silu_mul_combo, 3),      CROW_FN(acc_combo, 3),
-    CROW_FN(argmax_k, 3),          CROW_FN(argmax_tiles, 2),        CROW_FN(dequant_fp4_flat, 4),    CROW_FN(repack_nvfp4, 4),
+    CROW_FN(argmax_k, 3),          {"argmax_tiles", (const void*)&argmax_tiles, 2, 0u, 0, 4, 0, true},        CROW_FN(dequant_fp4_flat, 4),    CROW_FN(repack_nvfp4, 4),
     CROW_FN(unpack_nvfp4, 4),      CROW_FN(dequant_nvfp4_tiled, 5),
     // shared-X GEMM blocks: two staged X tiles of MT rows x 528 bytes
-    {"gemm_nvfp4_bf16", (const void*)&gemm_nvfp4_bf16, 7, 2u * 128u * 528u, 0, 16, 0},
-    {"gemm_nvfp4_bf16_m64", (const void*)&gemm_nvfp4_bf16_m64, 7, 2u * 64u * 528u, 0, 16, 0},
-    {"gemm_nvfp4_bf16_m48", (const void*)&gemm_nvfp4_bf16_m48, 7, 2u * 48u * 528u, 0, 16, 0},
-    {"gemm_nvfp4_bf16_m96", (const void*)&gemm_nvfp4_bf16_m96, 7, 2u * 96u * 528u, 0, 16, 0},
+    {"gemm_nvfp4_bf16", (const void*)&gemm_nvfp4_bf16, 7, 2u * 128u * 528u, 0, 16, 0, false},
+    {"gemm_nvfp4_bf16_m64", (const void*)&gemm_nvfp4_bf16_m64, 7, 2u * 64u * 528u, 0, 16, 0, false},
+    {"gemm_nvfp4_bf16_m48", (const void*)&gemm_nvfp4_bf16_m48, 7, 2u * 48u * 528u, 0, 16, 0, false},
+    {"gemm_nvfp4_bf16_m96", (const void*)&gemm_nvfp4_bf16_m96, 7, 2u * 96u * 528u, 0, 16, 0, false},
     CROW_FN(gemm_nvfp4_bf16_m32, 7), CROW_FN(gemm_nvfp4_bf16_m16, 7), CROW_FN(gemv_bf16_w, 5),
     CROW_FN(gemv_bf16, 5), CROW_FN(gemv_bf16_b, 5), CROW_FN(gemv_b, 5), CROW_FN(gemv_bf16_ws, 5), CROW_FN(gemv_bf16_bs, 6),
 };
@@ -89,16 +90,19 @@ const FnEntry* entry_of(crow_fn_t f) {
 // The launch dimensions of the GEMV family carry the problem in `gy` (crow_hip_launch_dims writes it, callers pass it on
 // unchanged): bits 0..19 = K / 64, bits 20..23 = activation rows of the last token group (0 = not given), bits 24..31 = S, the
 // number of column slices per strip.  The real grid is (gx, S, gz); the low 24 bits reach the kernel by value.
-int launch_entry(const FnEntry* e, dim3 grid, dim3 block, const uint64_t* vals, uint32_t n, hipStream_t s) {
+// `ws`: the scratch memory the launch may use, handed by value to the kernels that take one.
+int launch_entry(const FnEntry* e, dim3 grid, dim3 block, const uint64_t* vals, uint32_t n, hipStream_t s, const crow::Workspace& ws) {
     if (!g.ready) return CROW_ERR_NOT_INITIALIZED;
     if (!e || !vals) return CROW_ERR_BAD_ARGUMENT;
     if ((int)n != e->nargs) return CROW_ERR_ARG_COUNT;
     // whole wavefronts only: every kernel derives its wave count (and its LDS layout) from block.x / 64
     if (grid.x == 0 || grid.y == 0 || grid.z == 0 || block.x == 0 || block.x > 64u * (unsigned)e->max_waves || block.x % 64 != 0) return CROW_ERR_BAD_ARGUMENT;
-    void* args[17];
+    void* args[18];
     for (uint32_t i = 0; i < n; i++) args[i] = (void*)&vals[i];
+    uint32_t na = n;
     size_t lds = e->lds_fixed;
     int geo = 0;
+    crow::Workspace ws_arg = ws;
     if (e->nr != 0) {
         const unsigned word = grid.y;
         const int pairs = (int)(word & 0xFFFFFu), slices = (int)(word >> 24) == 0 ? 1 : (int)(word >> 24);
@@ -106,10 +110,15 @@ int launch_entry(const FnEntry* e, dim3 grid, dim3 block, const uint64_t* vals, 
         if (pairs == 0 || wpt == 0) return CROW_ERR_BAD_ARGUMENT;
         lds = (size_t)CROW_GEMV_ZERO_BYTES + (size_t)waves * (size_t)e->lds_per_wave;
         if (lds > g.lds_cap) return CROW_ERR_SHAPE;
+        // a split launch must fit the scratch memory it is given (the kernels check again and report through the status word)
+        if (slices > 1 && ((unsigned long long)grid.x * grid.z * (unsigned)slices * (unsigned)e->nr * 64ull > ws.partial_floats ||
+                           (unsigned long long)grid.x * grid.z > ws.counter_slots))
+            return CROW_ERR_WORKSPACE;
         geo = (int)(word & 0xFFFFFFu);
         grid.y = (unsigned)slices;
-        args[n] = (void*)&geo;
+        args[na++] = (void*)&geo;
     }
+    if (e->takes_ws) args[na++] = (void*)&ws_arg;
     const hipError_t rc = hipLaunchKernel(e->stub, grid, block, args, lds, s);
     if (rc != hipSuccess) (void)hipGetLastError();  // reported here: not left behind for an unrelated later call to find
     return hip_rc(rc);
@@ -254,7 +263,7 @@ int crow_hip_launch(crow_fn_t f, uint32_t gx, uint32_t gy, uint32_t gz, uint32_t
                     void* stream) {
     const FnEntry* e = entry_of(f);
     if (!e) return CROW_ERR_KERNEL_MISSING;
-    return launch_entry(e, dim3(gx, gy, gz), dim3(bx, 1, 1), vals, n_vals, stream ? (hipStream_t)stream : g.stream);
+    return launch_entry(e, dim3(gx, gy, gz), dim3(bx, 1, 1), vals, n_vals, stream ? (hipStream_t)stream : g.stream, g.ws);
 }
 
 // Which GEMM entry point for m token rows on a [rows, *] tensor.  Up to 16 rows: the K-split body over blocks; up to 96:
@@ -470,7 +479,7 @@ int crow_hip_time_launches(crow_fn_t f, uint32_t gx, uint32_t gy, uint32_t gz, u
     if ((rc = hipEventCreate(&b)) != hipSuccess) return (int)rc;
     int out = hip_rc(hipEventRecord(a, g.stream));
     for (uint32_t i = 0; i < iters && out == CROW_OK; i++)
-        out = launch_entry(e, dim3(gx, gy, gz), dim3(bx), vals + (size_t)(i % n_sets) * n_vals, n_vals, g.stream);
+        out = launch_entry(e, dim3(gx, gy, gz), dim3(bx), vals + (size_t)(i % n_sets) * n_vals, n_vals, g.stream, g.ws);
     if (out == CROW_OK) out = hip_rc(hipEventRecord(b, g.stream));
     if (out == CROW_OK) out = hip_rc(hipEventSynchronize(b));
     float ms = 0.0f;
@@ -499,7 +508,7 @@ int crow_hip_time_sequence(uint32_t n_kernels, const crow_fn_t* fns, const crow_
     for (uint32_t i = 0; i < iters && out == CROW_OK; i++) {
         const uint64_t* v = vals + (size_t)(i % n_sets) * per_set;
         for (uint32_t k = 0; k < n_kernels && out == CROW_OK; k++) {
-            out = launch_entry((const FnEntry*)(void*)fns[k], dim3(dims[k].gx, dims[k].gy, dims[k].gz), dim3(dims[k].bx), v, n_vals[k], g.stream);
+            out = launch_entry((const FnEntry*)(void*)fns[k], dim3(dims[k].gx, dims[k].gy, dims[k].gz), dim3(dims[k].bx), v, n_vals[k], g.stream, g.ws);
             v += n_vals[k];
         }
     }
@@ -598,7 +607,7 @@ static int layout_launch(const char* name, const void* a, const void* b, const v
     if (c) vals[n++] = (uint64_t)c;
     vals[n++] = (uint64_t)sc;
     vals[n++] = (uint64_t)(sc + 1);
-    rc = launch_entry(find(name), dim3(d.gx, d.gy, d.gz), dim3(d.bx), vals, n, g.stream);
+    rc = launch_entry(find(name), dim3(d.gx, d.gy, d.gz), dim3(d.bx), vals, n, g.stream, g.ws);
     if (rc != CROW_OK) return rc;
     return crow_hip_status();
 }

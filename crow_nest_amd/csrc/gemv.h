@@ -528,13 +528,19 @@ __device__ __forceinline__ void gemv_body(const GemvArgs& a, unsigned z, lds_p l
     }
     const int row = strip * CROW_STRIP_ROWS + n;
     if (EPI == EPI_SCALE && a.argmax_out != nullptr) {
-        // fused head, stage 1: logits out, and the strip's best (value, index) folded into the library's key word with one
+        // fused head, stage 1: logits out, and the strip's best (value, index) folded into the caller's key word with a
         // 64-bit atomic maximum that nobody waits for.  Stage 2 (argmax_tiles) decodes the key and clears it.
         const float val = v[0] * a.gs[0][0];
         const bool live = mo == 0 && row < rows;
         if (live) a.y[row] = val;
         const Best b = wave_best(Best{live ? val : -3.0e38f, live ? row : 0});
-        if (lane == 0) __hip_atomic_fetch_max(ws.am_key, best_key(b.v, b.i), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        if (lane == 0) {
+            // thousands of blocks hit this one word: an atomic costs its L2 channel several ns, a load almost nothing, and
+            // after the first few blocks hardly any candidate beats the word.  The maximum is the same in any order.
+            const unsigned long long key = best_key(b.v, b.i);
+            if (__hip_atomic_load(ws.am_key, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) < key)
+                __hip_atomic_fetch_max(ws.am_key, key, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
         return;
     }
     if (mo >= M || row >= rows) return;

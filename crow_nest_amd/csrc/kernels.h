@@ -19,9 +19,13 @@ using namespace crow;
 // The block's dynamic LDS (zeros, activation staging, wave hand-over: gemv.h); the launcher sizes it.
 extern __shared__ uint4 crow_dyn_lds[];
 #define LDS ((lds_p)crow_dyn_lds)
-// First statement of every GEMV entry point: the workspace descriptor and ALL kernel arguments are requested together and
-// waited for once - one scalar round trip between the start of a wave and its first weight load.  Left alone the compiler
-// fetches each argument where it is first used, behind whatever wait comes before: two or three dependent round trips.
+// After `geo` every entry point of the family takes the descriptor of the scratch memory its launch may use (per-slice partial
+// sums, arrival counters, the status word, the argmax key) BY VALUE too: the launcher appends the library's allocation, or -
+// crow_hip_launch_noalloc - the one it keeps in a static device array.
+//
+// First statement of every GEMV entry point: ALL kernel arguments are requested together and waited for once - one scalar
+// round trip between the start of a wave and its first weight load.  Left alone the compiler fetches each argument where it
+// is first used, behind whatever wait comes before: two or three dependent round trips.
 template <typename T>
 __device__ __forceinline__ void crow_need_one(T v) {
     asm volatile("" ::"s"(v));
@@ -32,9 +36,7 @@ __device__ __forceinline__ void crow_need_now(T v, R... rest) {
     crow_need_one(v);
     crow_need_now(rest...);
 }
-#define ENTER(...)                \
-    const Workspace ws = g_ws;    \
-    crow_need_now(ws.status, block_threads(), (int)gridDim.y, __VA_ARGS__)
+#define ENTER(...) crow_need_now(ws.status, block_threads(), (int)gridDim.y, __VA_ARGS__)
 // One-row kernels are compiled for at least this many resident waves per SIMD (it bounds their registers): six on bf16
 // activations, five on f32 ones (whose sixteen registers of activations in flight do not fit the tighter bound).  Blocks are
 // five waves per tensor at K = 5120, so five and six waves per SIMD hold the same four blocks per compute unit.
@@ -45,7 +47,7 @@ __device__ __forceinline__ void crow_need_now(T v, R... rest) {
 // reference: gemv_nvfp4_w, engine/src/kernels_p2.rs:355-368
 extern "C" __global__ void CROW_ONE_ROW_F32 __launch_bounds__(1024) gemv_nvfp4_w(const unsigned char* __restrict__ w, const float* __restrict__ x,
                                                                 const float* __restrict__ gs_ptr, float* __restrict__ y,
-                                                                const int* __restrict__ k_dim_p, const int* __restrict__ rows_p, int geo) {
+                                                                const int* __restrict__ k_dim_p, const int* __restrict__ rows_p, int geo, const Workspace ws) {
     ENTER(w, x, gs_ptr, y, k_dim_p, rows_p, geo);
     const int pairs = geo & 0xFFFFF;
     GemvArgs a = gemv_args(w, nullptr, gs_ptr, nullptr, x, 0, y, 0, pairs, k_dim_p, rows_p);
@@ -54,7 +56,7 @@ extern "C" __global__ void CROW_ONE_ROW_F32 __launch_bounds__(1024) gemv_nvfp4_w
 // the same product on bf16 activations (exact widening), for models that keep their activations in bf16
 extern "C" __global__ void CROW_ONE_ROW_BF16 __launch_bounds__(1024) gemv_nvfp4_w_bf16(const unsigned char* __restrict__ w, const unsigned short* __restrict__ x,
                                                                      const float* __restrict__ gs_ptr, float* __restrict__ y,
-                                                                     const int* __restrict__ k_dim_p, const int* __restrict__ rows_p, int geo) {
+                                                                     const int* __restrict__ k_dim_p, const int* __restrict__ rows_p, int geo, const Workspace ws) {
     ENTER(w, x, gs_ptr, y, k_dim_p, rows_p, geo);
     const int pairs = geo & 0xFFFFF;
     GemvArgs a = gemv_args(w, nullptr, gs_ptr, nullptr, x, 0, y, 0, pairs, k_dim_p, rows_p);
@@ -63,7 +65,7 @@ extern "C" __global__ void CROW_ONE_ROW_BF16 __launch_bounds__(1024) gemv_nvfp4_
 // reference: gemv_fp4, engine/src/kernels.rs:118-151 (+ rows_p: the reference's grid.x is the row count)
 extern "C" __global__ void CROW_ONE_ROW_F32 __launch_bounds__(1024) gemv_fp4(const unsigned char* __restrict__ w, const float* __restrict__ x,
                                                             const float* __restrict__ gs_ptr, float* __restrict__ y,
-                                                            const int* __restrict__ k_dim_p, const int* __restrict__ rows_p, int geo) {
+                                                            const int* __restrict__ k_dim_p, const int* __restrict__ rows_p, int geo, const Workspace ws) {
     ENTER(w, x, gs_ptr, y, k_dim_p, rows_p, geo);
     const int pairs = geo & 0xFFFFF;
     GemvArgs a = gemv_args(w, nullptr, gs_ptr, nullptr, x, 0, y, 0, pairs, k_dim_p, rows_p);
@@ -78,7 +80,7 @@ extern "C" __global__ void CROW_ONE_ROW_F32 __launch_bounds__(1024) gemv_fp4(con
 extern "C" __global__ void CROW_ONE_ROW_F32 __launch_bounds__(1024) gemv_nvfp4_w_argmax(const unsigned char* __restrict__ w, const float* __restrict__ x,
                                                                        const float* __restrict__ gs_ptr, float* __restrict__ y,
                                                                        const int* __restrict__ k_dim_p, const int* __restrict__ rows_p,
-                                                                       int* __restrict__ out_idx, int geo) {
+                                                                       int* __restrict__ out_idx, int geo, const Workspace ws) {
     ENTER(w, x, gs_ptr, y, k_dim_p, rows_p, out_idx, geo);
     const int pairs = geo & 0xFFFFF;
     GemvArgs a = gemv_args(w, nullptr, gs_ptr, nullptr, x, 0, y, 0, pairs, k_dim_p, rows_p);
@@ -91,7 +93,7 @@ extern "C" __global__ void CROW_ONE_ROW_F32 __launch_bounds__(1024) gemv_nvfp4_w
 extern "C" __global__ void CROW_ONE_ROW_F32 __launch_bounds__(1024) gemv_nvfp4_gu(const unsigned char* __restrict__ wg, const unsigned char* __restrict__ wu,
                                                                  const float* __restrict__ x, const float* __restrict__ gs_g,
                                                                  const float* __restrict__ gs_u, float* __restrict__ y,
-                                                                 const int* __restrict__ k_dim_p, const int* __restrict__ rows_p, int geo) {
+                                                                 const int* __restrict__ k_dim_p, const int* __restrict__ rows_p, int geo, const Workspace ws) {
     ENTER(wg, wu, x, gs_g, gs_u, y, k_dim_p, rows_p, geo);
     const int pairs = geo & 0xFFFFF;
     GemvArgs a = gemv_args(wg, wu, gs_g, gs_u, x, 0, y, 0, pairs, k_dim_p, rows_p);
@@ -102,7 +104,7 @@ extern "C" __global__ void CROW_ONE_ROW_F32 __launch_bounds__(1024) gemv_nvfp4_g
 extern "C" __global__ void CROW_ONE_ROW_BF16 __launch_bounds__(1024) gemv_nvfp4_gu_bf16(const unsigned char* __restrict__ wg, const unsigned char* __restrict__ wu,
                                                                       const unsigned short* __restrict__ x, const float* __restrict__ gs_g,
                                                                       const float* __restrict__ gs_u, float* __restrict__ y,
-                                                                      const int* __restrict__ k_dim_p, const int* __restrict__ rows_p, int geo) {
+                                                                      const int* __restrict__ k_dim_p, const int* __restrict__ rows_p, int geo, const Workspace ws) {
     ENTER(wg, wu, x, gs_g, gs_u, y, k_dim_p, rows_p, geo);
     const int pairs = geo & 0xFFFFF;
     GemvArgs a = gemv_args(wg, wu, gs_g, gs_u, x, 0, y, 0, pairs, k_dim_p, rows_p);
@@ -138,7 +140,7 @@ __device__ __forceinline__ int rows_of(GemvArgs& a, int geo, const int* m_p) {
 extern "C" __global__ void __launch_bounds__(512) gemv_nvfp4_wm(const unsigned char* __restrict__ w, const float* __restrict__ x,
                                                                  const float* __restrict__ gs_ptr, float* __restrict__ y,
                                                                  const int* __restrict__ k_dim_p, const int* __restrict__ rows_p,
-                                                                 const int* __restrict__ m_p, int geo) {
+                                                                 const int* __restrict__ m_p, int geo, const Workspace ws) {
     ENTER(w, x, gs_ptr, y, k_dim_p, rows_p, m_p, geo);
     const int pairs = geo & 0xFFFFF;
     GemvArgs a = gemv_args(w, nullptr, gs_ptr, nullptr, x, (size_t)pairs * CROW_PAIR_COLS, y, 0, pairs, k_dim_p, rows_p);
@@ -149,7 +151,7 @@ extern "C" __global__ void __launch_bounds__(512) gemv_nvfp4_gum(const unsigned 
                                                                    const float* __restrict__ x, const float* __restrict__ gs_g,
                                                                    const float* __restrict__ gs_u, float* __restrict__ y,
                                                                    const int* __restrict__ k_dim_p, const int* __restrict__ rows_p,
-                                                                   const int* __restrict__ m_p, int geo) {
+                                                                   const int* __restrict__ m_p, int geo, const Workspace ws) {
     ENTER(wg, wu, x, gs_g, gs_u, y, k_dim_p, rows_p, m_p, geo);
     const int pairs = geo & 0xFFFFF;
     GemvArgs a = gemv_args(wg, wu, gs_g, gs_u, x, (size_t)pairs * CROW_PAIR_COLS, y, 0, pairs, k_dim_p, rows_p);
@@ -159,7 +161,7 @@ extern "C" __global__ void __launch_bounds__(512) gemv_nvfp4_gum(const unsigned 
 extern "C" __global__ void __launch_bounds__(1024) gemv_nvfp4_wm_bf16(const unsigned char* __restrict__ w, const unsigned short* __restrict__ x,
                                                                       const float* __restrict__ gs_ptr, float* __restrict__ y,
                                                                       const int* __restrict__ k_dim_p, const int* __restrict__ rows_p,
-                                                                      const int* __restrict__ m_p, int geo) {
+                                                                      const int* __restrict__ m_p, int geo, const Workspace ws) {
     ENTER(w, x, gs_ptr, y, k_dim_p, rows_p, m_p, geo);
     const int pairs = geo & 0xFFFFF;
     GemvArgs a = gemv_args(w, nullptr, gs_ptr, nullptr, x, (size_t)pairs * CROW_PAIR_COLS, y, 0, pairs, k_dim_p, rows_p);
@@ -169,7 +171,7 @@ extern "C" __global__ void __launch_bounds__(1024) gemv_nvfp4_gum_bf16(const uns
                                                                        const unsigned short* __restrict__ x, const float* __restrict__ gs_g,
                                                                        const float* __restrict__ gs_u, float* __restrict__ y,
                                                                        const int* __restrict__ k_dim_p, const int* __restrict__ rows_p,
-                                                                       const int* __restrict__ m_p, int geo) {
+                                                                       const int* __restrict__ m_p, int geo, const Workspace ws) {
     ENTER(wg, wu, x, gs_g, gs_u, y, k_dim_p, rows_p, m_p, geo);
     const int pairs = geo & 0xFFFFF;
     GemvArgs a = gemv_args(wg, wu, gs_g, gs_u, x, (size_t)pairs * CROW_PAIR_COLS, y, 0, pairs, k_dim_p, rows_p);
@@ -203,21 +205,21 @@ __device__ __forceinline__ void gemv_tokens(const unsigned char* w, const float*
 extern "C" __global__ void __launch_bounds__(512) gemv_fp4_b(const unsigned char* __restrict__ w, const float* __restrict__ x,
                                                               const float* __restrict__ gs_ptr, float* __restrict__ y,
                                                               const int* __restrict__ k_dim_p, const int* __restrict__ rows_p,
-                                                              const int* __restrict__ t_p, int geo) {
+                                                              const int* __restrict__ t_p, int geo, const Workspace ws) {
     ENTER(w, x, gs_ptr, y, k_dim_p, rows_p, t_p, geo);
     gemv_tokens(w, x, gs_ptr, y, geo, k_dim_p, rows_p, t_p, 0, ws);
 }
 extern "C" __global__ void __launch_bounds__(512) gemv_fp4_b1k(const unsigned char* __restrict__ w, const float* __restrict__ x,
                                                                 const float* __restrict__ gs_ptr, float* __restrict__ y,
                                                                 const int* __restrict__ k_dim_p, const int* __restrict__ rows_p,
-                                                                const int* __restrict__ t_p, int geo) {
+                                                                const int* __restrict__ t_p, int geo, const Workspace ws) {
     ENTER(w, x, gs_ptr, y, k_dim_p, rows_p, t_p, geo);
     gemv_tokens(w, x, gs_ptr, y, geo, k_dim_p, rows_p, t_p, 0, ws);
 }
 extern "C" __global__ void __launch_bounds__(512) gemv_fp4_bs(const unsigned char* __restrict__ w, const float* __restrict__ x,
                                                                const float* __restrict__ gs_ptr, float* __restrict__ y,
                                                                const int* __restrict__ k_dim_p, const int* __restrict__ y_stride_p,
-                                                               const int* __restrict__ rows_p, const int* __restrict__ t_p, int geo) {
+                                                               const int* __restrict__ rows_p, const int* __restrict__ t_p, int geo, const Workspace ws) {
     ENTER(w, x, gs_ptr, y, k_dim_p, y_stride_p, rows_p, t_p, geo);
     const int y_stride = *y_stride_p;
     if (y_stride < *rows_p) {  // rows of y would overlap: refuse (uniform over the launch)
@@ -241,7 +243,7 @@ extern "C" __global__ void __launch_bounds__(512) gemv_fp4_bs(const unsigned cha
 extern "C" __global__ void CROW_ONE_ROW_F32 __launch_bounds__(1024) gemv_fp4_ptrb(const unsigned long long* __restrict__ ptrs, const float* __restrict__ x,
                                                                  const float* __restrict__ gs_ptr, float* __restrict__ y,
                                                                  const int* __restrict__ k_dim_p, const int* __restrict__ x_div_p,
-                                                                 const int* __restrict__ x_stride_p, const int* __restrict__ rows_p, int geo) {
+                                                                 const int* __restrict__ x_stride_p, const int* __restrict__ rows_p, int geo, const Workspace ws) {
     ENTER(ptrs, x, gs_ptr, y, k_dim_p, x_div_p, x_stride_p, rows_p, geo);
     const int pairs = geo & 0xFFFFF;
     const int combo = (int)blockIdx.z;
@@ -261,7 +263,7 @@ __device__ __forceinline__ size_t up_offset(int inter, int pairs) {
 extern "C" __global__ void CROW_ONE_ROW_F32 __launch_bounds__(1024) moe_gate_up_silu(const unsigned long long* __restrict__ ptrs, const float* __restrict__ x,
                                                                     const float* __restrict__ gs_ptr, float* __restrict__ h,
                                                                     const int* __restrict__ k_dim_p, const int* __restrict__ x_div_p,
-                                                                    const int* __restrict__ x_stride_p, const int* __restrict__ inter_p, int geo) {
+                                                                    const int* __restrict__ x_stride_p, const int* __restrict__ inter_p, int geo, const Workspace ws) {
     ENTER(ptrs, x, gs_ptr, h, k_dim_p, x_div_p, x_stride_p, inter_p, geo);
     const int pairs = geo & 0xFFFFF;
     const int combo = (int)blockIdx.z, inter = *inter_p;  // (arrives with ptrs[combo]: no round trip of its own)
@@ -283,7 +285,7 @@ extern "C" __global__ void CROW_ONE_ROW_F32 __launch_bounds__(1024) moe_gate_up_
 extern "C" __global__ void __launch_bounds__(1024) moe_down_combine(const unsigned long long* __restrict__ ptrs, const float* __restrict__ h,
                                                                     const float* __restrict__ gs_ptr, const float* __restrict__ rw,
                                                                     float* __restrict__ y, const int* __restrict__ k_dim_p,
-                                                                    const int* __restrict__ rows_p, int geo) {
+                                                                    const int* __restrict__ rows_p, int geo, const Workspace ws) {
     ENTER(ptrs, h, gs_ptr, rw, y, k_dim_p, rows_p, geo);
     const int pairs = geo & 0xFFFFF;
     constexpr int AREA = crow_gemv_lds_per_wave(1, false);
@@ -337,7 +339,7 @@ extern "C" __global__ void __launch_bounds__(512) moe_gate_up_silu_grouped(const
                                                                              const float* __restrict__ x, const float* __restrict__ gs_ptr,
                                                                              float* __restrict__ h, const int* __restrict__ k_dim_p,
                                                                              const int* __restrict__ x_div_p, const int* __restrict__ x_stride_p,
-                                                                             const int* __restrict__ inter_p, int geo) {
+                                                                             const int* __restrict__ inter_p, int geo, const Workspace ws) {
     ENTER(tiles, n_tiles_p, perm, table, x, gs_ptr, h, k_dim_p, x_div_p, x_stride_p, inter_p, geo);
     const int pairs = geo & 0xFFFFF;
     const int z = (int)blockIdx.z;
@@ -359,7 +361,7 @@ extern "C" __global__ void __launch_bounds__(512) moe_down_grouped(const int4* _
                                                                     const int* __restrict__ perm, const unsigned long long* __restrict__ table,
                                                                     const float* __restrict__ h, const float* __restrict__ gs_ptr,
                                                                     float* __restrict__ eo, const int* __restrict__ k_dim_p,
-                                                                    const int* __restrict__ rows_p, int geo) {
+                                                                    const int* __restrict__ rows_p, int geo, const Workspace ws) {
     ENTER(tiles, n_tiles_p, perm, table, h, gs_ptr, eo, k_dim_p, rows_p, geo);
     const int pairs = geo & 0xFFFFF;
     const int z = (int)blockIdx.z;

@@ -288,7 +288,7 @@ extern "C" __global__ void CROW_ONE_ROW_F32 __launch_bounds__(1024) moe_route_ga
                                                                           const float* __restrict__ x, const float* __restrict__ gs_ptr,
                                                                           float* __restrict__ h, int* __restrict__ ids, float* __restrict__ wts,
                                                                           unsigned long long* __restrict__ dn_ptrs, const int* __restrict__ k_dim_p,
-                                                                          const int* __restrict__ x_stride_p, const int* __restrict__ inter_p, int geo) {
+                                                                          const int* __restrict__ x_stride_p, const int* __restrict__ inter_p, int geo, const Workspace ws) {
     ENTER(logits, table, x, gs_ptr, h, ids, wts, dn_ptrs, k_dim_p, x_stride_p, inter_p, geo);
     const int pairs = geo & 0xFFFFF;
     __shared__ unsigned long long s_slab;
@@ -470,9 +470,9 @@ extern "C" __global__ void __launch_bounds__(1024) argmax_k(const float* __restr
 // Stage 2 of the fused head: the greedy token out of the key word gemv_nvfp4_w_argmax's blocks folded their candidates into
 // (device_common.h: same total order as argmax_k), and the word cleared for the next head.  grid (1), block 64.
 // (rows_p is unused: kept so that the call site's value list stays as it was.)
-extern "C" __global__ void __launch_bounds__(256) argmax_tiles(int* __restrict__ out, const int* __restrict__ rows_p) {
+extern "C" __global__ void __launch_bounds__(256) argmax_tiles(int* __restrict__ out, const int* __restrict__ rows_p, const Workspace ws) {
     if (threadIdx.x != 0) return;
-    unsigned long long* key = g_ws.am_key;
+    unsigned long long* key = ws.am_key;
     const unsigned long long k = __hip_atomic_load(key, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     out[0] = k != 0ull ? best_key_index(k) : 0;
     __hip_atomic_store(key, 0ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
