@@ -58,11 +58,20 @@ struct State {
     int cus = 256;
     hipStream_t stream = nullptr;
     crow::Workspace ws{};
+    crow::Workspace ws_static{};  // the same roles inside `scratch`, through the device address crow_hip_init asked for
     int* scalars = nullptr;  // two device words for the library's own launches (rows, k_dim)
     char name[256] = {0};
     int geo_topk = 0;  // host copy of the routed geometry (crow_hip_set_geo), for launch shapes
     size_t lds_cap = 64u * 1024u;  // most LDS one workgroup may take on this device
 } g;
+
+// Scratch memory of crow_hip_launch_noalloc: part of the code object, so it exists on a device from the moment the library
+// is loaded there until the process ends, and no call ever allocates it.  Words [0, NOALLOC_PARTIAL_FLOATS) hold the partial
+// sums of split launches, then NOALLOC_COUNTER_SLOTS arrival counters, the status word, one pad word, and the head's 64-bit key.
+const unsigned NOALLOC_PARTIAL_FLOATS = CROW_NOALLOC_MAX_PARTIAL_FLOATS;  // 4 MiB of split-K partial sums
+const unsigned NOALLOC_COUNTER_SLOTS = CROW_NOALLOC_MAX_STRIPS;
+const unsigned NOALLOC_WORDS = NOALLOC_PARTIAL_FLOATS + NOALLOC_COUNTER_SLOTS + 4;
+static __device__ __align__(256) unsigned scratch[NOALLOC_WORDS];
 
 const unsigned long long PARTIAL_FLOATS = 16ull << 20;  // 64 MiB of split-K partial sums
 const unsigned COUNTER_SLOTS = 1u << 16;
@@ -174,9 +183,22 @@ int crow_hip_init(int device) {
             (e = hipFuncSetAttribute(g_table[i].stub, hipFuncAttributeMaxDynamicSharedMemorySize, (int)most)) != hipSuccess)
             return fail(e);
     }
+    // `scratch` in host code is a stand-in, not a device address: ask for this device's copy once, and use only that
+    unsigned* sp = nullptr;
+    if ((e = hipGetSymbolAddress((void**)&sp, HIP_SYMBOL(scratch))) != hipSuccess || sp == nullptr) return fail(e != hipSuccess ? e : hipErrorInvalidSymbol);
+    crow::Workspace st{};
+    st.partials = (float*)sp;
+    st.partial_floats = NOALLOC_PARTIAL_FLOATS;
+    st.counters = sp + NOALLOC_PARTIAL_FLOATS;
+    st.counter_slots = NOALLOC_COUNTER_SLOTS;
+    st.status = st.counters + NOALLOC_COUNTER_SLOTS;
+    st.am_key = (unsigned long long*)(st.status + 2);
+    // counters, status and key start at zero (a process that shut the library down and initialises it again included)
+    if ((e = hipMemset(st.counters, 0, (NOALLOC_COUNTER_SLOTS + 4) * sizeof(unsigned))) != hipSuccess) return fail(e);
     if ((e = hipDeviceSynchronize()) != hipSuccess) return fail(e);
     g.scalars = scalars;
     g.ws = ws;
+    g.ws_static = st;
     g.device = device;
     g.stream = nullptr;
     g.ready = true;
@@ -264,6 +286,16 @@ int crow_hip_launch(crow_fn_t f, uint32_t gx, uint32_t gy, uint32_t gz, uint32_t
     const FnEntry* e = entry_of(f);
     if (!e) return CROW_ERR_KERNEL_MISSING;
     return launch_entry(e, dim3(gx, gy, gz), dim3(bx, 1, 1), vals, n_vals, stream ? (hipStream_t)stream : g.stream, g.ws);
+}
+
+int crow_hip_launch_noalloc(crow_fn_t f, uint32_t gx, uint32_t gy, uint32_t gz, uint32_t bx, const uint64_t* vals,
+                            uint32_t n_vals, void* stream) {
+    const FnEntry* e = entry_of(f);
+    if (!e) return CROW_ERR_KERNEL_MISSING;
+    // only kernels that are handed their scratch memory as an argument can be pointed at the static array
+    if (!e->takes_ws) return CROW_ERR_BAD_ARGUMENT;
+    // launch_entry refuses (CROW_ERR_WORKSPACE) a split whose partial sums or counters do not fit what it is given
+    return launch_entry(e, dim3(gx, gy, gz), dim3(bx, 1, 1), vals, n_vals, stream ? (hipStream_t)stream : g.stream, g.ws_static);
 }
 
 // Which GEMM entry point for m token rows on a [rows, *] tensor.  Up to 16 rows: the K-split body over blocks; up to 96:
@@ -400,13 +432,18 @@ int crow_hip_status(void) {
     // arrival counters are cleared below, or may still be about to raise a status bit
     hipError_t e = hipDeviceSynchronize();
     if (e != hipSuccess) return (int)e;
-    unsigned st = 0;
+    unsigned st = 0, st2 = 0;
     if ((e = hipMemcpy(&st, g.ws.status, sizeof st, hipMemcpyDeviceToHost)) != hipSuccess) return (int)e;
-    if (st == 0) return CROW_OK;
-    (void)hipMemset(g.ws.status, 0, sizeof st);
-    // a launch that bailed out may have left arrival counters behind
-    (void)hipMemset(g.ws.counters, 0, COUNTER_WORDS * sizeof(unsigned));
-    (void)hipMemset(g.ws.am_key, 0, sizeof(unsigned long long));  // ... or a head's candidates without their stage 2
+    if ((e = hipMemcpy(&st2, g.ws_static.status, sizeof st2, hipMemcpyDeviceToHost)) != hipSuccess) return (int)e;
+    if (st == 0 && st2 == 0) return CROW_OK;
+    if (st != 0) {
+        (void)hipMemset(g.ws.status, 0, sizeof st);
+        // a launch that bailed out may have left arrival counters behind
+        (void)hipMemset(g.ws.counters, 0, COUNTER_WORDS * sizeof(unsigned));
+        (void)hipMemset(g.ws.am_key, 0, sizeof(unsigned long long));  // ... or a head's candidates without their stage 2
+    }
+    if (st2 != 0) (void)hipMemset(g.ws_static.counters, 0, (NOALLOC_COUNTER_SLOTS + 4) * sizeof(unsigned));  // counters, status, key
+    st |= st2;
     if (st & CROW_STATUS_BAD_SCALE_BYTE) return CROW_ERR_SCALE_BYTE;
     if (st & crow::STATUS_WORKSPACE_TOO_SMALL) return CROW_ERR_WORKSPACE;
     if (st & crow::STATUS_BAD_GEO) return CROW_ERR_GEO;
@@ -418,6 +455,8 @@ int crow_hip_reset_workspace(void) {
     hipError_t e = hipDeviceSynchronize();
     if (e != hipSuccess) return (int)e;
     if ((e = hipMemset(g.ws.am_key, 0, sizeof(unsigned long long))) != hipSuccess) return (int)e;
+    if ((e = hipMemset(g.ws_static.counters, 0, NOALLOC_COUNTER_SLOTS * sizeof(unsigned))) != hipSuccess) return (int)e;
+    if ((e = hipMemset(g.ws_static.am_key, 0, sizeof(unsigned long long))) != hipSuccess) return (int)e;
     return hip_rc(hipMemset(g.ws.counters, 0, COUNTER_WORDS * sizeof(unsigned)));
 }
 

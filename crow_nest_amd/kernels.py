@@ -92,6 +92,14 @@ def launch_v(f: int, gx: int, gy: int, gz: int, bx: int, vals) -> None:
     _l.check(_l.lib().crow_hip_launch(f, gx, gy, gz, bx, arr, n, None), "launch_v")
 
 
+def launch_noalloc(f: int, gx: int, gy: int, gz: int, bx: int, vals) -> None:
+    """``launch_v`` for callers that may not allocate device memory: the kernels' scratch (split-K partial sums, arrival
+    counters, status, the head's key) is a fixed array inside the library; a split beyond its size raises."""
+    n = len(vals)
+    arr = (C.c_uint64 * n)(*[int(v) for v in vals])
+    _l.check(_l.lib().crow_hip_launch_noalloc(f, gx, gy, gz, bx, arr, n, None), "launch_noalloc")
+
+
 def sync() -> None:
     _l.check(_l.lib().crow_hip_sync(), "sync")
 

@@ -58,6 +58,7 @@ def lib():
         "crow_hip_function_arg_count": (C.c_int, [vp]),
         "crow_hip_set_geo": (C.c_int, [C.c_int] * 4),
         "crow_hip_launch": (C.c_int, [vp, u32, u32, u32, u32, u64p, u32, vp]),
+        "crow_hip_launch_noalloc": (C.c_int, [vp, u32, u32, u32, u32, u64p, u32, vp]),
         "crow_hip_launch_dims": (C.c_int, [C.c_char_p, u32, u32, u32, C.POINTER(Dims)]),
         "crow_hip_gemm_kernel": (C.c_char_p, [u32, u32]),
         "crow_hip_launch_dims_split": (C.c_int, [C.c_char_p, u32, u32, u32, u32, u32, C.POINTER(Dims)]),
@@ -102,7 +103,7 @@ def lib():
 EXPORTS = [
     "crow_hip_init", "crow_hip_shutdown", "crow_hip_error_string", "crow_hip_device_name", "crow_hip_module_load",
     "crow_hip_module_unload", "crow_hip_module_get", "crow_hip_get_function", "crow_hip_function_count",
-    "crow_hip_function_name", "crow_hip_function_arg_count", "crow_hip_set_geo", "crow_hip_launch",
+    "crow_hip_function_name", "crow_hip_function_arg_count", "crow_hip_set_geo", "crow_hip_launch", "crow_hip_launch_noalloc",
     "crow_hip_launch_dims", "crow_hip_launch_dims_split", "crow_hip_gemm_kernel", "crow_hip_status", "crow_hip_reset_workspace", "crow_hip_set_stream", "crow_hip_cur_stream",
     "crow_hip_sync", "crow_hip_event_create", "crow_hip_event_record", "crow_hip_event_elapsed_ms", "crow_hip_event_destroy", "crow_hip_time_launches", "crow_hip_time_sequence", "crow_hip_alloc", "crow_hip_free", "crow_hip_upload", "crow_hip_download",
     "crow_hip_stream_create", "crow_hip_stream_destroy", "crow_hip_begin_capture", "crow_hip_end_capture_instantiate",
