@@ -28,9 +28,27 @@ for p in (ROOT, os.path.join(ROOT, "tests")):
         sys.path.insert(0, p)
 
 PEAK_HBM_GBS = 8000.0
-# HBM bytes per launch of the dominant kernel, measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE and scaled by
-# a 256 MiB copy kernel in the same run (profiles/gemv_nvfp4_gu_bf16__config1_m1.md): 101,142,923 read + 818,176 written
-TRAFFIC_GATE_UP_M1 = 101961099
+REPS = 5  # timing repetitions per figure: the median is reported, the minimum beside it
+# HBM bytes per launch of the dominant kernel come from the committed rocprofv3 --pmc summary (FETCH_SIZE / WRITE_SIZE scaled by
+# a 256 MiB copy kernel of the same run), keyed by kernel and launch shape: a line
+#   TRAFFIC <kernel> grid=<gx>x<slices>x<gz> block=<bx> bytes=<n>
+# in this file.  A kernel launched with another shape than the one profiled reports traffic null.
+TRAFFIC_PROFILE = os.path.join(ROOT, "profiles", "gemv_nvfp4_gu_bf16__config1_m1.md")
+
+
+def traffic_from_profile(kernel: str, dims) -> int | None:
+    key = f"TRAFFIC {kernel} grid={dims[0]}x{max(1, dims[1] >> 24)}x{dims[2]} block={dims[3]} bytes="
+    try:
+        with open(TRAFFIC_PROFILE) as fh:
+            for line in fh:
+                line = line.strip().strip("`")
+                if line.startswith(key):
+                    return int(line[len(key):].replace(",", ""))
+    except OSError:
+        pass
+    return None
+
+
 N, K = 17408, 5120
 W_BYTES = N * K // 64 * 36  # 50,135,040: container encoding, 4.5 bits per weight
 
@@ -59,10 +77,16 @@ class Launch:
         if rc != 0:
             raise RuntimeError(f"crow_hip_launch failed: {rc}")
 
-    def us(self, iters=200, reps=3):
+    def us(self, iters=200, reps=REPS):
+        """(median, minimum) over `reps` repetitions of the mean microseconds per launch of `iters` back-to-back launches."""
         from crow_nest_amd.kernels import time_launches
         time_launches(self.f, *self.dims, self.raw, 20)
-        return min(time_launches(self.f, *self.dims, self.raw, iters) for _ in range(reps))
+        return med_min([time_launches(self.f, *self.dims, self.raw, iters) for _ in range(reps)])
+
+
+def med_min(ts):
+    ts = sorted(ts)
+    return ts[len(ts) // 2], ts[0]
 
 
 def main() -> int:
@@ -152,12 +176,23 @@ def main() -> int:
     # parity of what was just timed, against the CPU path (the checker, outside the timed region)
     ref_h = orc.silu_mul(orc.gemv(host["gate"][0], N, K, host["gate"][1], orc.bf16_bits_to_f32(xb_bits), threads=8),
                          orc.gemv(host["up"][0], N, K, host["up"][1], orc.bf16_bits_to_f32(xb_bits), threads=8))[0]
-    from gpu_common import rel_err
+    from gpu_common import FLOOR, FLOOR_CHAINED, gamma_rows, rel_err, rel_l2
     gu.go(lib, 0)
     dn.go(lib, 0)
     torch.cuda.synchronize()
-    parity_h = rel_err(h.cpu().numpy(), ref_h)
-    parity_y = rel_err(y.cpu().numpy(), orc.gemv(host["down"][0], K, N, host["down"][1], ref_h, threads=8)[0])
+    h_dev, y_dev = h.cpu().numpy(), y.cpu().numpy()
+    ref_y = orc.gemv(host["down"][0], K, N, host["down"][1], ref_h, threads=8)[0]
+    # the down projection alone, on the H the device wrote: one product, so the single-product floor applies to it
+    ref_y_dev_h = orc.gemv(host["down"][0], K, N, host["down"][1], h_dev, threads=8)[0]
+    r0, nr = 2048, 128  # 128 rows of each product against f64, to be inside the reference's own f32 bound
+    parity = {
+        "h_max_rel_err": float(f"{rel_err(h_dev, ref_h):.3g}"), "h_rel_l2": float(f"{rel_l2(h_dev, ref_h):.3g}"),
+        "y_on_device_h_max_rel_err": float(f"{rel_err(y_dev, ref_y_dev_h):.3g}"),
+        "y_on_device_h_gamma_ratio_128_rows": float(f"{gamma_rows(y_dev[r0:r0 + nr], host['down'][0], r0, nr, N, host['down'][1], h_dev):.3g}"),
+        "y_chained_max_rel_err": float(f"{rel_err(y_dev, ref_y, FLOOR_CHAINED):.3g}"), "y_chained_rel_l2": float(f"{rel_l2(y_dev, ref_y):.3g}"),
+        "denominator_floor": f"max(|ref|, {FLOOR} * rms(ref)) for one product, {FLOOR_CHAINED} * rms for the two products in a row "
+                             "(y_chained: H already differs by its own rounding); gamma ratio <= 1 = inside gamma(K/16 + 10) * sum|w x| around f64",
+    }
 
     # ---------------- the same step as a captured graph (10 steps, one per weight copy, in one graph)
     from crow_nest_amd.kernels import Graph
@@ -166,16 +201,34 @@ def main() -> int:
         for i in range(copies):
             step(i)
     gr.time(3)
-    graph_us_per_step = min(gr.time(40) for _ in range(3)) / copies
+    graph_med, graph_min = med_min([gr.time(40) / copies for _ in range(REPS)])
     gr.close()
 
     # ---------------- roofline of the dominant kernel (gate/up + SiLU), HIP events on the launch stream
-    gu_us = gu.us()
-    dn_us = dn.us()
+    gu_us, gu_us_min = gu.us()
+    dn_us, dn_us_min = dn.us()
     gu_bytes = alg_bytes_gate_up(1)
     roof = {"bound": "hbm", "kernel": "gemv_nvfp4_gu_bf16", "achieved": round(gu_bytes / gu_us / 1e3, 1), "peak": PEAK_HBM_GBS,
-            "unit": "GB/s", "frac": round(gu_bytes / gu_us / 1e3 / PEAK_HBM_GBS, 4), "traffic": TRAFFIC_GATE_UP_M1,
-            "us_per_launch": round(gu_us, 2), "algorithmic_bytes": gu_bytes, "grid": list(gu.dims)}
+            "unit": "GB/s", "frac": round(gu_bytes / gu_us / 1e3 / PEAK_HBM_GBS, 4), "traffic": traffic_from_profile("gemv_nvfp4_gu_bf16", gu.dims),
+            "traffic_source": "profiles/gemv_nvfp4_gu_bf16__config1_m1.md (rocprofv3 --pmc FETCH_SIZE + WRITE_SIZE, scaled by a 256 MiB copy), "
+                              "matched on kernel, grid and block; null when the launch shape differs from the profiled one",
+            "us_per_launch": round(gu_us, 2), "us_per_launch_min": round(gu_us_min, 2), "timing": f"median (and minimum) of {REPS} x 200 back-to-back launches, HIP events on the launch stream",
+            "algorithmic_bytes": gu_bytes, "grid": [gu.dims[0], max(1, gu.dims[1] >> 24), gu.dims[2]], "block": gu.dims[3]}
+
+    # config 0 (the reference's own CPU-runnable case): the plain GEMV y = W x on W_gate, f32 x, the same seeded weights
+    xk0 = torch.from_numpy(x32).to(dev)
+    y0 = torch.empty(N, dtype=torch.float32, device=dev)
+    l0 = Launch(eng, "gemv_nvfp4_w", N, K, 1, [[s_["gate"].data_ptr(), xk0.data_ptr(), base["gate"].gs_ptr, y0.data_ptr(), p.i32(K), p.i32(N)] for s_ in sets])
+    c0_us, c0_us_min = l0.us()
+    c0_bytes = W_BYTES + K * 4 + N * 4 + 4
+    torch.cuda.synchronize()
+    c0_ref = orc.gemv(host["gate"][0], N, K, host["gate"][1], x32, threads=8)[0]
+    c0_y = y0.cpu().numpy()
+    config0 = {"workload": "BASELINE config 0: y = W x, W [17408, 5120] NVFP4 (W_gate of config 1), x f32, batch 1",
+               "kernel": "gemv_nvfp4_w", "us_per_call": round(c0_us, 2), "us_per_call_min": round(c0_us_min, 2),
+               "GB/s": round(c0_bytes / c0_us / 1e3, 1), "pct_of_peak": round(c0_bytes / c0_us / 1e3 / 80, 1), "algorithmic_bytes": c0_bytes,
+               "parity_max_rel_err": float(f"{rel_err(c0_y, c0_ref):.3g}"), "parity_rel_l2": float(f"{rel_l2(c0_y, c0_ref):.3g}"),
+               "gamma_ratio_128_rows": float(f"{gamma_rows(c0_y[r0:r0 + nr], host['gate'][0], r0, nr, K, host['gate'][1], x32):.3g}")}
 
     out = {
         "metric": "NVFP4 GEMV achieved HBM GB/s (% of peak) and us/call at batch 1, 1 MI355X",
@@ -187,9 +240,11 @@ def main() -> int:
                    "algorithmic_bytes_per_step": step_bytes, "pct_of_peak": round(100 * value / PEAK_HBM_GBS, 1),
                    "arithmetic": "exact bf16 x bf16 products on the matrix cores (weights decode exactly, f32 activations split "
                                  "into three exact bf16 terms), f32 accumulation and scales",
-                   "graph_replay_us_per_step": round(graph_us_per_step, 2),
+                   "graph_replay_us_per_step": round(graph_med, 2), "graph_replay_us_per_step_min": round(graph_min, 2),
                    "us_per_call": {"gate_up_silu": round(gu_us, 2), "down": round(dn_us, 2)},
-                   "parity_max_rel_err": {"h": float(f"{parity_h:.3g}"), "y": float(f"{parity_y:.3g}")},
+                   "us_per_call_min": {"gate_up_silu": round(gu_us_min, 2), "down": round(dn_us_min, 2)},
+                   "parity": parity,
+                   "config0": config0,
                    "inputs": {"generator": "splitmix64 + Box-Muller, seed 0, one stream per tensor; W ~ N(0, 0.02^2) through the ceil encoder, "
                                            "x ~ N(0, 1) rounded to bf16", "sha256_16": input_sha256,
                               "global_scales": {nm: float(np.float32(host[nm][1])) for nm in host}},
@@ -210,12 +265,17 @@ def main() -> int:
         xkb = xk.to(torch.bfloat16)
         ybuf = torch.empty(4 * 151936, dtype=torch.float32, device=dev)
 
-        def entry(us, nbytes):
-            return {"us": round(us, 2), "GB/s": round(nbytes / us / 1e3, 1), "pct_peak": round(nbytes / us / 1e3 / 80, 1)}
+        others["note"] = ("timing only: microseconds per call are medians of %d repetitions (us_min beside them); weights of the shapes below "
+                          "that are not config 1's own tensors are random bytes (codes and scale bytes 0..63), activations N(0, 1)" % REPS)
 
-        # config 0: dense GEMV, f32 x
-        l0 = Launch(eng, "gemv_nvfp4_w", N, K, 1, [[s["gate"].data_ptr(), xk.data_ptr(), gs1.data_ptr(), ybuf.data_ptr(), p.i32(K), p.i32(N)] for s in sets])
-        others["config0_gemv_17408x5120_f32x"] = entry(l0.us(), W_BYTES + K * 4 + N * 4 + 4)
+        def entry(us, nbytes):
+            us, us_min = us
+            return {"us": round(us, 2), "us_min": round(us_min, 2), "GB/s": round(nbytes / us / 1e3, 1), "pct_peak": round(nbytes / us / 1e3 / 80, 1)}
+
+        def seq_us(seq, n_sets, iters):
+            time_sequence(seq, n_sets, max(n_sets, iters // 10))
+            return med_min([time_sequence(seq, n_sets, iters) for _ in range(REPS)])
+
         # config 1 at verify widths
         for m in (2, 4):
             lg = Launch(eng, "gemv_nvfp4_gum_bf16", N, K, m,
@@ -231,11 +291,11 @@ def main() -> int:
         idx = torch.zeros(1, dtype=torch.int32, device=dev)
         l3 = Launch(eng, "gemv_nvfp4_w_argmax", V, K, 1, [[hd.data_ptr(), xk.data_ptr(), gs1.data_ptr(), ybuf.data_ptr(), p.i32(K), p.i32(V), idx.data_ptr()] for hd in heads])
         from crow_nest_amd.kernels import time_sequence
-        seq3 = [(l3.f, l3.dims, l3.raw), (eng.k.f("argmax_tiles"), (1, 1, 1, 256), [[idx.data_ptr(), p.i32(V)]])]
         status()
-        time_sequence(seq3, 4, 10)
-        others["config3_lm_head_151936x5120_argmax"] = entry(min(time_sequence(seq3, 4, 100) for _ in range(3)), V * K // 64 * 36 + K * 4 + V * 4 + 4)
-        others["config3_lm_head_151936x5120_argmax"]["launches"] = 2
+        others["config3_lm_head_151936x5120_argmax"] = entry(l3.us(iters=100), V * K // 64 * 36 + K * 4 + V * 4 + 4)
+        others["config3_lm_head_151936x5120_argmax"]["launches"] = 1
+        lp = Launch(eng, "gemv_nvfp4_w", V, K, 1, [[hd.data_ptr(), xk.data_ptr(), gs1.data_ptr(), ybuf.data_ptr(), p.i32(K), p.i32(V)] for hd in heads])
+        others["config3_lm_head_151936x5120_logits_only"] = entry(lp.us(iters=100), V * K // 64 * 36 + K * 4 + V * 4)
         del heads
         # config 4: batched GEMM on the matrix cores
         for m in (16, 128, 512):
@@ -243,8 +303,9 @@ def main() -> int:
             ym = torch.empty(m, N, dtype=torch.float32, device=dev)
             nm = gemm_kernel_for(m, N)
             l4 = Launch(eng, nm, N, K, m, [[s["gate"].data_ptr(), xm.data_ptr(), gs1.data_ptr(), ym.data_ptr(), p.i32(K), p.i32(N), p.i32(m)] for s in sets])
-            us = l4.us(iters=50)
-            e = entry(us, W_BYTES + m * K * 2 + m * N * 4)
+            us2 = l4.us(iters=50)
+            us = us2[0]
+            e = entry(us2, W_BYTES + m * K * 2 + m * N * 4)
             e["TFLOP/s"] = round(2.0 * m * N * K / us / 1e6, 1)
             e["pct_mfma_peak_bf16"] = round(2.0 * m * N * K / us / 1e6 / 2500 * 100, 1)
             others[f"config4_gemm_M{m}"] = e
@@ -299,11 +360,20 @@ def main() -> int:
             nbytes = int(distinct * (2 * I * H // 64 * 36 + H * I // 64 * 36)) + t * H * 8 + t * E * 4  # every distinct expert once
             for tag, seq in (("", [lrg, ldn]), ("_router_apart", [lr, lgu, ldn])):
                 seq2 = [(l_.f, l_.dims, l_.raw) for l_ in seq]
-                time_sequence(seq2, len(lgs), 24)
-                us = min(time_sequence(seq2, len(lgs), 240) for _ in range(3))
-                others[f"config2_moe_layer_T{t}{tag}"] = entry(us, nbytes)
+                others[f"config2_moe_layer_T{t}{tag}"] = entry(seq_us(seq2, len(lgs), 240), nbytes)
                 others[f"config2_moe_layer_T{t}{tag}"]["launches"] = len(seq)
                 others[f"config2_moe_layer_T{t}{tag}"]["distinct_experts_mean"] = round(distinct, 2)
+            # the same layer inside a captured graph: 24 consecutive layers (one per routing decision) on one stream per replay
+            grm = Graph()
+            with grm.capture():
+                for i_ in range(len(lgs)):
+                    lrg.go(lib, i_)
+                    ldn.go(lib, i_)
+            grm.time(3)
+            g_med, g_min = med_min([grm.time(20) / len(lgs) for _ in range(REPS)])
+            grm.close()
+            others[f"config2_moe_layer_T{t}"]["graph_replay_24_layers_us_per_layer"] = round(g_med, 2)
+            others[f"config2_moe_layer_T{t}"]["graph_replay_24_layers_us_per_layer_min"] = round(g_min, 2)
         # the same layer for a batch in which experts repeat (64 tokens): per combo against grouped by expert
         t = 64
         combos = t * K8
@@ -336,9 +406,7 @@ def main() -> int:
         nbytes = int(distinct * (2 * I * H // 64 * 36 + H * I // 64 * 36)) + t * H * 8 + t * E * 4
         for tag, seq in (("per_combo", [lr, lgu, ldn]), ("grouped", [lr, lgr, lgg, ldg, lac])):
             sq = [(l_.f, l_.dims, l_.raw) for l_ in seq]
-            time_sequence(sq, len(lgs), 12)
-            us = min(time_sequence(sq, len(lgs), 120) for _ in range(3))
-            others[f"moe_layer_T64_{tag}"] = entry(us, nbytes)
+            others[f"moe_layer_T64_{tag}"] = entry(seq_us(sq, len(lgs), 120), nbytes)
             others[f"moe_layer_T64_{tag}"]["launches"] = len(seq)
         status()
         out["others"] = others
@@ -375,10 +443,44 @@ def main() -> int:
             tt.sort()
             by_threads[str(th)] = round(3 * W_BYTES / tt[len(tt) // 2] / 1e9, 2)
         by_threads[str(threads)] = round(3 * W_BYTES / med / 1e9, 2)
-        out["cpu_baseline"] = {"value": round(3 * W_BYTES / med / 1e9, 2), "unit": "GB/s", "cores": threads, "kind": "port",
-                               "ms_per_step": round(med * 1e3, 3), "GB/s_by_threads": by_threads,
+        # every hardware thread the host shows (the reference's own "all threads" leg, cpu_nvfp4.rs:729-777), whatever share of
+        # them this process may use: 48 calls
+        hw = os.cpu_count() or 1
+        best_med, best_threads = med, threads
+        if hw > threads:
+            th = min(hw, 512)
+            for u in units:
+                orc.ffn(u[0], gsv[0], u[1], gsv[1], u[2], gsv[2], K, N, xs, threads=th, path=1)
+            tt = []
+            for rep in range(48):
+                u = units[rep % 8]
+                c0 = time.perf_counter()
+                orc.ffn(u[0], gsv[0], u[1], gsv[1], u[2], gsv[2], K, N, xs, threads=th, path=1)
+                tt.append(time.perf_counter() - c0)
+            tt.sort()
+            by_threads[f"all({th})"] = round(3 * W_BYTES / tt[len(tt) // 2] / 1e9, 2)
+            if tt[len(tt) // 2] < best_med:
+                best_med, best_threads = tt[len(tt) // 2], th
+        cpu_model = "unknown"
+        try:
+            with open("/proc/cpuinfo") as fh:
+                for line in fh:
+                    if line.startswith("model name"):
+                        cpu_model = line.split(":", 1)[1].strip()
+                        break
+        except OSError:
+            pass
+        try:
+            usable = len(os.sched_getaffinity(0))
+        except (AttributeError, OSError):
+            usable = hw
+        out["cpu_baseline"] = {"value": round(3 * W_BYTES / best_med / 1e9, 2), "unit": "GB/s", "cores": best_threads, "kind": "port",
+                               "ms_per_step": round(best_med * 1e3, 3), "GB/s_by_threads": by_threads,
+                               "cpu_model": cpu_model, "hardware_concurrency": hw, "usable_cpus": usable,
                                "sample": "same step (gate/up + SiLU + down, one token, f32 x) on 8 rotating 150 MB weight units, median of 160 calls "
-                                         "after a warm-up pass (64 calls for each smaller thread count: about 15 core-seconds in all); AVX2 path of the C restatement of engine/src/cpu_nvfp4.rs (OpenMP row split)"}
+                                         f"at {threads} threads after a warm-up pass, 64 calls for each smaller thread count and 48 with every hardware "
+                                         "thread (about 20 core-seconds in all); value = the best of these legs, cores = its thread count; "
+                                         "AVX2 path of the C restatement of engine/src/cpu_nvfp4.rs (OpenMP row split)"}
     print(json.dumps(out))
     return 0
 

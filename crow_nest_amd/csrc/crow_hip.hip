@@ -22,7 +22,7 @@ struct FnEntry {
     int nr;
     int max_waves;  // per block (the kernel's launch bound)
     int lds_per_wave;
-    bool takes_ws;  // the launcher appends the scratch descriptor (every kernel of the GEMV family, and argmax_tiles)
+    bool takes_ws;  // the launcher appends the scratch descriptor (every kernel of the GEMV family)
 };
 
 #define CROW_FN(name, nargs) {#name, (const void*)&name, nargs, 0u, 0, 16, 0, false}
@@ -40,7 +40,7 @@ const FnEntry g_table[] = {
     CROW_GEMV(moe_route_gate_up_silu, 11, 2, 1, false), CROW_GEMV(moe_gate_up_silu_grouped, 11, 2, 4, false), CROW_GEMV(moe_down_grouped, 9, 1, 4, false),
     CROW_FN(moe_group, 6),
     CROW_FN(router_top10, 10),     CROW_FN(silu_mul_combo, 3),      CROW_FN(acc_combo, 3),
-    CROW_FN(argmax_k, 3),          {"argmax_tiles", (const void*)&argmax_tiles, 2, 0u, 0, 4, 0, true},        CROW_FN(dequant_fp4_flat, 4),    CROW_FN(repack_nvfp4, 4),
+    CROW_FN(argmax_k, 3),          CROW_FN(dequant_fp4_flat, 4),    CROW_FN(repack_nvfp4, 4),
     CROW_FN(unpack_nvfp4, 4),      CROW_FN(dequant_nvfp4_tiled, 5),
     // shared-X GEMM blocks: two staged X tiles of MT rows x 528 bytes
     {"gemm_nvfp4_bf16", (const void*)&gemm_nvfp4_bf16, 7, 2u * 128u * 528u, 0, 16, 0, false},
@@ -67,11 +67,15 @@ struct State {
 
 // Scratch memory of crow_hip_launch_noalloc: part of the code object, so it exists on a device from the moment the library
 // is loaded there until the process ends, and no call ever allocates it.  Words [0, NOALLOC_PARTIAL_FLOATS) hold the partial
-// sums of split launches, then NOALLOC_COUNTER_SLOTS arrival counters, the status word, one pad word, and the head's 64-bit key.
+// sums of split launches, then NOALLOC_COUNTER_SLOTS arrival counters, the status word (alone on 32 words), and the fused
+// head's key and counter words.
+const size_t HEAD_BYTES = (size_t)CROW_HEAD_WORDS * sizeof(unsigned long long);
 const unsigned NOALLOC_PARTIAL_FLOATS = CROW_NOALLOC_MAX_PARTIAL_FLOATS;  // 4 MiB of split-K partial sums
 const unsigned NOALLOC_COUNTER_SLOTS = CROW_NOALLOC_MAX_STRIPS;
-const unsigned NOALLOC_WORDS = NOALLOC_PARTIAL_FLOATS + NOALLOC_COUNTER_SLOTS + 4;
+const unsigned NOALLOC_TAIL_WORDS = 32 + 2 * CROW_HEAD_WORDS;  // status line, then the head's 8-byte words
+const unsigned NOALLOC_WORDS = NOALLOC_PARTIAL_FLOATS + NOALLOC_COUNTER_SLOTS + NOALLOC_TAIL_WORDS;
 static __device__ __align__(256) unsigned scratch[NOALLOC_WORDS];
+static_assert(sizeof(unsigned) * NOALLOC_WORDS == CROW_NOALLOC_SCRATCH_BYTES, "the header states the array's size");
 
 const unsigned long long PARTIAL_FLOATS = 16ull << 20;  // 64 MiB of split-K partial sums
 const unsigned COUNTER_SLOTS = 1u << 16;
@@ -158,14 +162,14 @@ int crow_hip_init(int device) {
     auto fail = [&](hipError_t why) {
         (void)hipFree(ws.partials);
         (void)hipFree(ws.counters);
-        (void)hipFree(ws.am_key);
+        (void)hipFree(ws.head);
         (void)hipFree(scalars);
         return (int)why;
     };
     if ((e = hipMalloc((void**)&ws.partials, PARTIAL_FLOATS * sizeof(float))) != hipSuccess) return fail(e);
     if ((e = hipMalloc((void**)&ws.counters, COUNTER_WORDS * sizeof(unsigned))) != hipSuccess) return fail(e);
-    if ((e = hipMalloc((void**)&ws.am_key, sizeof(unsigned long long))) != hipSuccess) return fail(e);
-    if ((e = hipMemset(ws.am_key, 0, sizeof(unsigned long long))) != hipSuccess) return fail(e);
+    if ((e = hipMalloc((void**)&ws.head, HEAD_BYTES)) != hipSuccess) return fail(e);
+    if ((e = hipMemset(ws.head, 0, HEAD_BYTES)) != hipSuccess) return fail(e);
     if ((e = hipMalloc((void**)&scalars, 16 * sizeof(int))) != hipSuccess) return fail(e);
     if ((e = hipMemset(ws.counters, 0, COUNTER_WORDS * sizeof(unsigned))) != hipSuccess) return fail(e);
     ws.status = ws.counters + COUNTER_SLOTS;
@@ -192,9 +196,9 @@ int crow_hip_init(int device) {
     st.counters = sp + NOALLOC_PARTIAL_FLOATS;
     st.counter_slots = NOALLOC_COUNTER_SLOTS;
     st.status = st.counters + NOALLOC_COUNTER_SLOTS;
-    st.am_key = (unsigned long long*)(st.status + 2);
+    st.head = (unsigned long long*)(st.status + 32);  // on a 128-byte line of its own
     // counters, status and key start at zero (a process that shut the library down and initialises it again included)
-    if ((e = hipMemset(st.counters, 0, (NOALLOC_COUNTER_SLOTS + 4) * sizeof(unsigned))) != hipSuccess) return fail(e);
+    if ((e = hipMemset(st.counters, 0, (NOALLOC_COUNTER_SLOTS + NOALLOC_TAIL_WORDS) * sizeof(unsigned))) != hipSuccess) return fail(e);
     if ((e = hipDeviceSynchronize()) != hipSuccess) return fail(e);
     g.scalars = scalars;
     g.ws = ws;
@@ -210,7 +214,7 @@ int crow_hip_shutdown(void) {
     (void)hipDeviceSynchronize();
     (void)hipFree(g.ws.partials);
     (void)hipFree(g.ws.counters);
-    (void)hipFree(g.ws.am_key);
+    (void)hipFree(g.ws.head);
     (void)hipFree(g.scalars);
     g = State{};
     return CROW_OK;
@@ -359,6 +363,8 @@ int crow_hip_launch_dims_split(const char* name, uint32_t rows, uint32_t k_dim, 
             return CROW_OK;
         }
         if (verify && z > 4) return CROW_ERR_SHAPE;
+        // the fused head counts at most 127 blocks into each of its scratch words
+        if (strcmp(name, "gemv_nvfp4_w_argmax") == 0 && strips > (uint32_t)CROW_HEAD_MAX_STRIPS) return CROW_ERR_SHAPE;
         const uint32_t wmax = (uint32_t)e->max_waves / (uint32_t)e->nr;  // waves per tensor in a block
         // A wave walks its run of groups with four of them (9 KB) in flight; few long walks beat many short ones (every wave
         // pays its start, its staging set-up and the block's meeting in LDS once), as long as the launch still has a few
@@ -413,7 +419,6 @@ int crow_hip_launch_dims_split(const char* name, uint32_t rows, uint32_t k_dim, 
     if (strcmp(name, "router_top10") == 0) { *out = crow_dims{z, 1, 1, 64}; return CROW_OK; }
     if (strcmp(name, "moe_group") == 0) { *out = crow_dims{1, 1, 1, 1024}; return CROW_OK; }
     if (strcmp(name, "argmax_k") == 0) { *out = crow_dims{1, 1, 1, 1024}; return CROW_OK; }
-    if (strcmp(name, "argmax_tiles") == 0) { *out = crow_dims{1, 1, 1, 64}; return CROW_OK; }
     if (strcmp(name, "acc_combo") == 0) { *out = crow_dims{(rows + 255) / 256, z, 1, 256}; return CROW_OK; }  // rows = hidden
     if (strcmp(name, "silu_mul_combo") == 0 || strcmp(name, "dequant_fp4_flat") == 0) {  // rows = element count
         *out = crow_dims{(rows + 255) / 256, 1, 1, 256};
@@ -440,9 +445,9 @@ int crow_hip_status(void) {
         (void)hipMemset(g.ws.status, 0, sizeof st);
         // a launch that bailed out may have left arrival counters behind
         (void)hipMemset(g.ws.counters, 0, COUNTER_WORDS * sizeof(unsigned));
-        (void)hipMemset(g.ws.am_key, 0, sizeof(unsigned long long));  // ... or a head's candidates without their stage 2
+        (void)hipMemset(g.ws.head, 0, HEAD_BYTES);  // ... or a head's candidates and counters
     }
-    if (st2 != 0) (void)hipMemset(g.ws_static.counters, 0, (NOALLOC_COUNTER_SLOTS + 4) * sizeof(unsigned));  // counters, status, key
+    if (st2 != 0) (void)hipMemset(g.ws_static.counters, 0, (NOALLOC_COUNTER_SLOTS + NOALLOC_TAIL_WORDS) * sizeof(unsigned));  // counters, status, key
     st |= st2;
     if (st & CROW_STATUS_BAD_SCALE_BYTE) return CROW_ERR_SCALE_BYTE;
     if (st & crow::STATUS_WORKSPACE_TOO_SMALL) return CROW_ERR_WORKSPACE;
@@ -454,9 +459,9 @@ int crow_hip_reset_workspace(void) {
     if (!g.ready) return CROW_ERR_NOT_INITIALIZED;
     hipError_t e = hipDeviceSynchronize();
     if (e != hipSuccess) return (int)e;
-    if ((e = hipMemset(g.ws.am_key, 0, sizeof(unsigned long long))) != hipSuccess) return (int)e;
+    if ((e = hipMemset(g.ws.head, 0, HEAD_BYTES)) != hipSuccess) return (int)e;
     if ((e = hipMemset(g.ws_static.counters, 0, NOALLOC_COUNTER_SLOTS * sizeof(unsigned))) != hipSuccess) return (int)e;
-    if ((e = hipMemset(g.ws_static.am_key, 0, sizeof(unsigned long long))) != hipSuccess) return (int)e;
+    if ((e = hipMemset(g.ws_static.head, 0, HEAD_BYTES)) != hipSuccess) return (int)e;
     return hip_rc(hipMemset(g.ws.counters, 0, COUNTER_WORDS * sizeof(unsigned)));
 }
 

@@ -40,13 +40,23 @@ __device__ __forceinline__ unsigned stream_load_u32(const unsigned* p) {
 
 // Library-owned scratch for kernels that split one output tile over several workgroups:
 // per-slice partial sums and one arrival counter per output tile.  Set once by crow_hip_init.
+// Scratch of the fused head (gemv_nvfp4_w_argmax): CROW_HEAD_SLOTS 64-bit words, each on a 128-byte line of its own (so that
+// the atomics of thousands of blocks spread over the L2 channels), all zero between launches.  Block b folds its candidate
+// into word b % CROW_HEAD_SLOTS with ONE compare-and-swap that also counts it: bits 63..7 = the best key so far (best_key),
+// bits 6..0 = blocks arrived.  Because key and count change together, a block that reads every word complete has read every
+// word's final key.  At most 127 blocks per word: 32,512 strips, 520,192 rows.
+#define CROW_HEAD_SLOTS 256
+#define CROW_HEAD_COUNT_BITS 7
+#define CROW_HEAD_MAX_STRIPS (127 * CROW_HEAD_SLOTS)
+#define CROW_HEAD_WORDS (16 * CROW_HEAD_SLOTS)
+
 struct Workspace {
     float* partials;
     unsigned* counters;
     unsigned long long partial_floats;  // capacity of `partials`
     unsigned counter_slots;             // capacity of `counters`
     unsigned* status;                   // device word: non-zero = a launch did not fit the workspace
-    unsigned long long* am_key;         // fused lm_head argmax: the best (value, index) so far as one ordered 64-bit key; 0 = none
+    unsigned long long* head;           // fused lm_head argmax: CROW_HEAD_WORDS 8-byte words, all zero between launches (layout below)
 };
 __device__ Workspace g_ws;
 
@@ -97,18 +107,20 @@ __device__ __forceinline__ bool better(float v, int i, float bv, int bi) {
     const unsigned ki = __brev((unsigned)i & 1023u), kb = __brev((unsigned)bi & 1023u);
     return v > bv || (v == bv && (ki < kb || (ki == kb && i < bi)));
 }
-// The same order as ONE unsigned 64-bit key, larger = better: the value's bits made monotonic (sign flipped for positive
-// floats, all bits for negative ones) above the complement of (bit-reversed (i mod 1024), i / 1024).  A 64-bit atomic maximum
-// over such keys is the tournament, whatever the arrival order.  No key of a real candidate is 0.
+// The same order as ONE unsigned 57-bit key, larger = better: the value's bits made monotonic (sign flipped for positive
+// floats, all bits for negative ones; -0 counts as +0 and a NaN as the start value, as under the comparisons above) above
+// the 25-bit complement of (bit-reversed (i mod 1024), i / 1024), i < 2^25.  A maximum over such keys is the tournament,
+// whatever the arrival order.  No key of a real candidate is 0.
 __device__ __forceinline__ unsigned long long best_key(float v, int i) {
+    v = v == v ? v + 0.0f : -3.0e38f;
     const unsigned u = __float_as_uint(v);
     const unsigned hi = (u & 0x80000000u) ? ~u : (u | 0x80000000u);
-    const unsigned tie = ((__brev((unsigned)i & 1023u) >> 22) << 22) | ((unsigned)i >> 10);
-    return ((unsigned long long)hi << 32) | (unsigned long long)(0xFFFFFFFFu - tie);
+    const unsigned tie = ((__brev((unsigned)i & 1023u) >> 22) << 15) | (((unsigned)i >> 10) & 0x7FFFu);
+    return ((unsigned long long)hi << 25) | (unsigned long long)(0x1FFFFFFu - tie);
 }
 __device__ __forceinline__ int best_key_index(unsigned long long key) {
-    const unsigned tie = 0xFFFFFFFFu - (unsigned)(key & 0xFFFFFFFFull);
-    return (int)(((tie & 0x3FFFFFu) << 10) | (__brev(tie >> 22) >> 22));
+    const unsigned tie = 0x1FFFFFFu - (unsigned)(key & 0x1FFFFFFull);
+    return (int)(((tie & 0x7FFFu) << 10) | (__brev(tie >> 15) >> 22));
 }
 __device__ __forceinline__ Best wave_best(Best b) {
     for (int o = 32; o > 0; o >>= 1) {

@@ -467,17 +467,6 @@ extern "C" __global__ void __launch_bounds__(1024) argmax_k(const float* __restr
     }
 }
 
-// Stage 2 of the fused head: the greedy token out of the key word gemv_nvfp4_w_argmax's blocks folded their candidates into
-// (device_common.h: same total order as argmax_k), and the word cleared for the next head.  grid (1), block 64.
-// (rows_p is unused: kept so that the call site's value list stays as it was.)
-extern "C" __global__ void __launch_bounds__(256) argmax_tiles(int* __restrict__ out, const int* __restrict__ rows_p, const Workspace ws) {
-    if (threadIdx.x != 0) return;
-    unsigned long long* key = ws.am_key;
-    const unsigned long long k = __hip_atomic_load(key, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    out[0] = k != 0ull ? best_key_index(k) : 0;
-    __hip_atomic_store(key, 0ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-}
-
 // ------------------------------------------------------------------ BF16 and F32 keeps
 // The tensors the container keeps unquantised (router, q/k, MTP head): y[t][row] = sum_k w[row][k] * x[t][k], f32
 // activations, f32 accumulation.  16-byte non-temporal weight loads (8 bf16 or 4 f32 per lane per step: 1024 contiguous

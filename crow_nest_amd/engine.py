@@ -119,8 +119,8 @@ class Engine:
 
     # ------------------------------------------------------------------ head
     def lm_head_row(self, w: Fp4, x: torch.Tensor, fused: bool = True):
-        """logits[V] and the greedy token.  fused: the GEMV leaves one candidate per 64-row tile and argmax_tiles
-        picks among those; else gemv_nvfp4_w + argmax_k over all logits, as the reference."""
+        """logits[V] and the greedy token.  fused: one launch writes both (the last block to finish picks the token);
+        else gemv_nvfp4_w + argmax_k over all logits, as the reference."""
         rows, k = w.rows, w.cols
         logits = torch.empty(rows, dtype=torch.float32, device=self.dev)
         idx = torch.zeros(1, dtype=torch.int32, device=self.dev)
@@ -129,7 +129,6 @@ class Engine:
             gx, gy, gz, bx = launch_dims("gemv_nvfp4_w_argmax", rows, k)
             launch_v(self.k.f("gemv_nvfp4_w_argmax"), gx, gy, gz, bx,
                      [w.w_ptr, x.data_ptr(), w.gs_ptr, logits.data_ptr(), p.i32(k), p.i32(rows), idx.data_ptr()])
-            launch_v(self.k.f("argmax_tiles"), 1, 1, 1, 256, [idx.data_ptr(), p.i32(rows)])
         else:
             self.dense_proj(w, 1, x, logits.view(1, rows))
             self.argmax(logits, idx)

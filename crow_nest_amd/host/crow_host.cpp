@@ -225,7 +225,6 @@ int Engine::lm_head_row(const Fp4& w, uint64_t x, uint64_t logits) {
     DevBuf idx(sizeof(int));
     launch_v(k.f("gemv_nvfp4_w_argmax"), launch_dims("gemv_nvfp4_w_argmax", (uint32_t)w.rows, (uint32_t)w.cols),
              {w.w.ptr(), x, w.gs.ptr(), logits, p.i32(w.cols), p.i32(w.rows), idx.ptr()});
-    launch_v(k.f("argmax_tiles"), 1, 1, 1, 256, {idx.ptr(), p.i32(w.rows)});
     int out = -1;
     idx.download(&out, sizeof out);
     return out;

@@ -31,11 +31,10 @@ CROW_KERNEL(gemv_nvfp4_w_bf16, 6) /* the same on bf16 x */
 /* w, x, gs, y, k_dim_p, rows_p.  gemv_fp4 of engine/src/kernels.rs:118-152 (the older one-block-per-row entry point the
  * engine still calls for some tensors); same arithmetic as gemv_nvfp4_w here. */
 CROW_KERNEL(gemv_fp4, 6)
-/* w, x, gs, y(logits), k_dim_p, rows_p, out_idx.  lm_head_row (engine/src/gen.rs:4766-4784) with the first stage of
- * argmax_k (engine/src/kernels.rs:4238-4260) fused: leaves one (value, index) candidate per 64-row tile in the library's
- * workspace; argmax_tiles then writes the winner to out_idx[0].  Same tie order as argmax_k. */
+/* w, x, gs, y(logits), k_dim_p, rows_p, out_idx.  lm_head_row (engine/src/gen.rs:4766-4784) and argmax_k
+ * (engine/src/kernels.rs:4238-4260) in one launch: logits[rows] and out_idx[0] = the greedy token, same tie order as
+ * argmax_k.  The blocks' candidates meet in the library's scratch memory; the last block to finish writes the token. */
 CROW_KERNEL(gemv_nvfp4_w_argmax, 7)
-CROW_KERNEL(argmax_tiles, 2) /* out_idx, rows_p */
 CROW_KERNEL(argmax_k, 3)     /* logits, out_idx, n_p.  engine/src/kernels.rs:4238-4260 */
 
 /* ---- fused gate / up + SiLU ----------------------------------------------------------------------------------------- */

@@ -35,7 +35,7 @@ def test_kernel_table_names_without_a_device():
     for want in ["gemv_nvfp4_w", "gemv_nvfp4_gu", "gemv_nvfp4_gu_bf16", "gemv_nvfp4_wm", "gemv_nvfp4_gum", "gemv_fp4", "gemv_fp4_b", "gemv_fp4_bs",
                  "gemv_fp4_b1k", "gemv_fp4_ptrb", "router_top10", "silu_mul_combo", "acc_combo", "argmax_k",
                  "dequant_fp4_flat", "gemv_nvfp4_w_argmax", "moe_gate_up_silu", "moe_down_combine", "moe_route_gate_up_silu", "moe_group", "moe_gate_up_silu_grouped", "moe_down_grouped", "gemm_nvfp4_bf16",
-                 "gemm_nvfp4_bf16_m16", "gemm_nvfp4_bf16_m32", "gemm_nvfp4_bf16_m64", "argmax_tiles", "gemv_bf16_w", "gemv_bf16", "gemv_bf16_b", "gemv_b", "gemv_bf16_ws", "gemv_bf16_bs"]:
+                 "gemm_nvfp4_bf16_m16", "gemm_nvfp4_bf16_m32", "gemm_nvfp4_bf16_m64", "gemv_bf16_w", "gemv_bf16", "gemv_bf16_b", "gemv_b", "gemv_bf16_ws", "gemv_bf16_bs"]:
         assert want in names, want
     import ctypes as C
     out = C.c_void_p()

@@ -769,7 +769,7 @@ def test_container_tensors_load_dequantise_and_multiply(eng):
 # ---------------------------------------------------------------- captured launch sequences
 
 def test_captured_sequence_replays_match_eager_launches(eng):
-    """The decode sequence gate/up+SiLU -> down -> lm_head + argmax stage 1 -> argmax stage 2, captured once and replayed
+    """The decode sequence gate/up+SiLU -> down -> lm_head with its argmax, captured once and replayed
     with new inputs, eager work and synchronisations in between: every replay equals the eager result bit for bit."""
     from crow_nest_amd.kernels import Graph, launch_dims, launch_v, sync
     H, I, V = 1024, 2816, 4000
@@ -783,8 +783,7 @@ def test_captured_sequence_replays_match_eager_launches(eng):
     tok = torch.zeros(1, dtype=torch.int32, device="cuda")
     seq = [("gemv_nvfp4_gu", launch_dims("gemv_nvfp4_gu", I, H), [g_.w_ptr, u_.w_ptr, x.data_ptr(), g_.gs_ptr, u_.gs_ptr, hbuf.data_ptr(), p.i32(H), p.i32(I)]),
            ("gemv_nvfp4_w", launch_dims("gemv_nvfp4_w", H, I), [d_.w_ptr, hbuf.data_ptr(), d_.gs_ptr, y.data_ptr(), p.i32(I), p.i32(H)]),
-           ("gemv_nvfp4_w_argmax", launch_dims("gemv_nvfp4_w_argmax", V, H), [h_.w_ptr, y.data_ptr(), h_.gs_ptr, logits.data_ptr(), p.i32(H), p.i32(V), tok.data_ptr()]),
-           ("argmax_tiles", launch_dims("argmax_tiles", V, H), [tok.data_ptr(), p.i32(V)])]
+           ("gemv_nvfp4_w_argmax", launch_dims("gemv_nvfp4_w_argmax", V, H), [h_.w_ptr, y.data_ptr(), h_.gs_ptr, logits.data_ptr(), p.i32(H), p.i32(V), tok.data_ptr()])]
 
     def eager():
         for name, dims, vals in seq:

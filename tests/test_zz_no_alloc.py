@@ -1,7 +1,7 @@
 """crow_hip_launch_noalloc (scratch memory in a fixed array inside the library, nothing allocated per call) against
 crow_hip_launch (scratch memory from the workspace crow_hip_init allocated): same kernels, same launch dimensions, so the
-same bits.  Two calls in a row share the one array, the second with a smaller input; then the fused head, whose key word
-lives in the same array; then the size limit."""
+same bits.  Two calls in a row share the one array, the second with a smaller input; then the fused head, whose key and counter
+words live in the same array; then the size limit."""
 import numpy as np
 import pytest
 import torch
@@ -78,11 +78,11 @@ def test_several_activation_rows_through_the_static_scratch(eng):
         assert gamma_ratio(b[t], w, rows, cols, gs, x[t]) <= 1.0
 
 
-def test_fused_head_keeps_its_key_in_the_static_scratch(eng):
+def test_fused_head_keeps_its_keys_in_the_static_scratch(eng):
     from crow_nest_amd.kernels import launch_dims, launch_noalloc, launch_v
     p = eng.p
     toks = []
-    # twice in a row: the second head (fewer rows) must find the key word cleared by the first one's stage 2
+    # twice in a row: the second head (fewer rows) must find the key and counter words cleared by the first one's last block
     for seed, rows, cols in [(31, 4000, 1024), (32, 1000, 512)]:
         w = random_nvfp4(seed, rows, cols)
         gs = 5.0e-4
@@ -96,7 +96,6 @@ def test_fused_head_keeps_its_key_in_the_static_scratch(eng):
             tok = torch.full((1,), -1, dtype=torch.int32, device="cuda")
             launch(eng.k.f("gemv_nvfp4_w_argmax"), *dims,
                    [f.w_ptr, xd.data_ptr(), f.gs_ptr, logits.data_ptr(), p.i32(cols), p.i32(rows), tok.data_ptr()])
-            launch(eng.k.f("argmax_tiles"), *launch_dims("argmax_tiles", rows, cols), [tok.data_ptr(), p.i32(rows)])
             res.append((logits.cpu().numpy(), int(tok.item())))
         eng.check()
         (la, ta), (lb, tb) = res
