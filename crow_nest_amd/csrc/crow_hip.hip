@@ -22,14 +22,15 @@ struct FnEntry {
     int nr;
     int max_waves;  // per block (the kernel's launch bound)
     int lds_per_wave;
+    int ns;  // adjacent 16-row strips per block (kernels for several activation rows: CROW_MULTI_STRIPS), else 1
     bool takes_ws;  // the launcher appends the scratch descriptor (every kernel of the GEMV family)
 };
 
-#define CROW_FN(name, nargs) {#name, (const void*)&name, nargs, 0u, 0, 16, 0, false}
+#define CROW_FN(name, nargs) {#name, (const void*)&name, nargs, 0u, 0, 16, 0, 1, false}
 // NR tensors per block, bodies for 1 .. MMAX activation rows, bf16 or f32 activations
-// (the bodies for several f32 rows need more registers than a block of sixteen waves leaves each: they run in blocks of eight)
+// (the bodies for several rows need more registers than a block of sixteen waves leaves each: they run in blocks of eight)
 #define CROW_GEMV(name, nargs, NR, MMAX, XBF16) \
-    {#name, (const void*)&name, nargs, 0u, NR, (MMAX > 1 && !XBF16) ? 8 : 16, crow::crow_gemv_lds_per_wave(MMAX, XBF16), true}
+    {#name, (const void*)&name, nargs, 0u, NR, MMAX > 1 ? 8 : 16, crow::crow_gemv_lds_per_wave(MMAX, XBF16), MMAX > 1 ? CROW_MULTI_STRIPS : 1, true}
 const FnEntry g_table[] = {
     CROW_GEMV(gemv_nvfp4_w, 6, 1, 1, false),       CROW_GEMV(gemv_nvfp4_w_bf16, 6, 1, 1, true),  CROW_GEMV(gemv_nvfp4_w_argmax, 7, 1, 1, false),
     CROW_GEMV(gemv_nvfp4_gu, 8, 2, 1, false),      CROW_GEMV(gemv_nvfp4_gu_bf16, 8, 2, 1, true),
@@ -43,10 +44,10 @@ const FnEntry g_table[] = {
     CROW_FN(argmax_k, 3),          CROW_FN(dequant_fp4_flat, 4),    CROW_FN(repack_nvfp4, 4),
     CROW_FN(unpack_nvfp4, 4),      CROW_FN(dequant_nvfp4_tiled, 5),
     // shared-X GEMM blocks: two staged X tiles of MT rows x 528 bytes
-    {"gemm_nvfp4_bf16", (const void*)&gemm_nvfp4_bf16, 7, 2u * 128u * 528u, 0, 16, 0, false},
-    {"gemm_nvfp4_bf16_m64", (const void*)&gemm_nvfp4_bf16_m64, 7, 2u * 64u * 528u, 0, 16, 0, false},
-    {"gemm_nvfp4_bf16_m48", (const void*)&gemm_nvfp4_bf16_m48, 7, 2u * 48u * 528u, 0, 16, 0, false},
-    {"gemm_nvfp4_bf16_m96", (const void*)&gemm_nvfp4_bf16_m96, 7, 2u * 96u * 528u, 0, 16, 0, false},
+    {"gemm_nvfp4_bf16", (const void*)&gemm_nvfp4_bf16, 7, 2u * 128u * 528u, 0, 16, 0, 1, false},
+    {"gemm_nvfp4_bf16_m64", (const void*)&gemm_nvfp4_bf16_m64, 7, 2u * 64u * 528u, 0, 16, 0, 1, false},
+    {"gemm_nvfp4_bf16_m48", (const void*)&gemm_nvfp4_bf16_m48, 7, 2u * 48u * 528u, 0, 16, 0, 1, false},
+    {"gemm_nvfp4_bf16_m96", (const void*)&gemm_nvfp4_bf16_m96, 7, 2u * 96u * 528u, 0, 16, 0, 1, false},
     CROW_FN(gemm_nvfp4_bf16_m32, 7), CROW_FN(gemm_nvfp4_bf16_m16, 7), CROW_FN(gemv_bf16_w, 5),
     CROW_FN(gemv_bf16, 5), CROW_FN(gemv_bf16_b, 5), CROW_FN(gemv_b, 5), CROW_FN(gemv_bf16_ws, 5), CROW_FN(gemv_bf16_bs, 6),
 };
@@ -124,7 +125,7 @@ int launch_entry(const FnEntry* e, dim3 grid, dim3 block, const uint64_t* vals, 
         lds = (size_t)CROW_GEMV_ZERO_BYTES + (size_t)waves * (size_t)e->lds_per_wave;
         if (lds > g.lds_cap) return CROW_ERR_SHAPE;
         // a split launch must fit the scratch memory it is given (the kernels check again and report through the status word)
-        if (slices > 1 && ((unsigned long long)grid.x * grid.z * (unsigned)slices * (unsigned)e->nr * 64ull > ws.partial_floats ||
+        if (slices > 1 && ((unsigned long long)grid.x * grid.z * (unsigned)slices * (unsigned)(e->nr * e->ns) * 64ull > ws.partial_floats ||
                            (unsigned long long)grid.x * grid.z > ws.counter_slots))
             return CROW_ERR_WORKSPACE;
         geo = (int)(word & 0xFFFFFFu);
@@ -390,8 +391,9 @@ int crow_hip_launch_dims_split(const char* name, uint32_t rows, uint32_t k_dim, 
         }
         const uint32_t gz = routed ? z : (tokens ? (z + 3) / 4 : 1);
         const uint32_t hint = verify ? z : (tokens ? (z - 1) % 4 + 1 : 0);
-        *out = crow_dims{strips, pairs | (hint << 20) | (s << 24), gz, 64u * w * (uint32_t)e->nr};
-        if (s > 1 && ((unsigned long long)strips * gz * s * 2 * 64 > PARTIAL_FLOATS || (unsigned long long)strips * gz > COUNTER_SLOTS)) return CROW_ERR_WORKSPACE;
+        const uint32_t gx = (strips + (uint32_t)e->ns - 1) / (uint32_t)e->ns;
+        *out = crow_dims{gx, pairs | (hint << 20) | (s << 24), gz, 64u * w * (uint32_t)e->nr};
+        if (s > 1 && ((unsigned long long)gx * gz * s * (unsigned)(e->nr * e->ns) * 64 > PARTIAL_FLOATS || (unsigned long long)gx * gz > COUNTER_SLOTS)) return CROW_ERR_WORKSPACE;
         return CROW_OK;
     }
     if (strncmp(name, "gemm_nvfp4_bf16", 15) == 0) {  // z = M token rows

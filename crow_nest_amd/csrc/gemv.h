@@ -134,11 +134,12 @@ __device__ __forceinline__ void split3(float f, unsigned& hi, unsigned& mid, uns
     lo = __float_as_uint(r2) & 0xffff0000u;
 }
 
-// One 256-column group: four pairs.  `a1[q]`, `a2[q]` are this lane's LDS addresses of its A1 / A2 operand for pair 0 of the
-// group's staging slot, set q (or of the zero area).
-template <int M, bool XBF16>
-__device__ __forceinline__ void group_multiply(unsigned sc, const u32x4 (&cd)[2], const lds_p (&a1)[XBF16 ? 1 : (3 * M + 3) / 4],
-                                               const lds_p (&a2)[XBF16 ? 1 : (3 * M + 3) / 4], float (&acc)[M]) {
+// One 256-column group of NS strips: four pairs.  `a1[q]`, `a2[q]` are this lane's LDS addresses of its A1 / A2 operand for pair
+// 0 of the group's staging slot, set q (or of the zero area).  The activation operands of a pair are read once and serve all
+// NS strips; per strip the operation sequence is that of a one-strip walk.
+template <int M, bool XBF16, int NS>
+__device__ __forceinline__ void group_multiply(const unsigned (&sc)[NS], const u32x4 (&cd)[NS][2], const lds_p (&a1)[XBF16 ? 1 : (3 * M + 3) / 4],
+                                               const lds_p (&a2)[XBF16 ? 1 : (3 * M + 3) / 4], float (&acc)[NS][M]) {
     constexpr int NSET = XBF16 ? 1 : (3 * M + 3) / 4;
     typedef __attribute__((address_space(3))) const u32x4* lds_v4;
 #pragma unroll
@@ -149,23 +150,26 @@ __device__ __forceinline__ void group_multiply(unsigned sc, const u32x4 (&cd)[2]
             A1[q] = __builtin_bit_cast(bf16x8, *(lds_v4)(a1[q] + 128 * jj));
             A2[q] = __builtin_bit_cast(bf16x8, *(lds_v4)(a2[q] + 128 * jj));
         }
-        const u32x4 c = cd[jj >> 1];
-        const bf16x8 B0 = decode8((jj & 1) ? c.z : c.x), B1 = decode8((jj & 1) ? c.w : c.y);
-        const float sv = jj == 0 ? e4m3_to_f32<0>(sc) : (jj == 1 ? e4m3_to_f32<1>(sc) : (jj == 2 ? e4m3_to_f32<2>(sc) : e4m3_to_f32<3>(sc)));
-        f32x4 D[NSET];
 #pragma unroll
-        for (int q = 0; q < NSET; q++) {
-            const f32x4 z = {0.f, 0.f, 0.f, 0.f};
-            D[q] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(A1[q], B0, z, 0, 0, 0);
-            D[q] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(A2[q], B1, D[q], 0, 0, 0);
-        }
+        for (int s = 0; s < NS; s++) {
+            const u32x4 c = cd[s][jj >> 1];
+            const bf16x8 B0 = decode8((jj & 1) ? c.z : c.x), B1 = decode8((jj & 1) ? c.w : c.y);
+            const float sv = jj == 0 ? e4m3_to_f32<0>(sc[s]) : (jj == 1 ? e4m3_to_f32<1>(sc[s]) : (jj == 2 ? e4m3_to_f32<2>(sc[s]) : e4m3_to_f32<3>(sc[s])));
+            f32x4 D[NSET];
 #pragma unroll
-        for (int m = 0; m < M; m++) {
-            if (XBF16) {
-                acc[m] = __builtin_fmaf(D[0][m], sv, acc[m]);
-            } else {
-                const float hi = D[(3 * m) / 4][(3 * m) % 4], mid = D[(3 * m + 1) / 4][(3 * m + 1) % 4], lo = D[(3 * m + 2) / 4][(3 * m + 2) % 4];
-                acc[m] = __builtin_fmaf(__fadd_rn(__fadd_rn(hi, mid), lo), sv, acc[m]);
+            for (int q = 0; q < NSET; q++) {
+                const f32x4 z = {0.f, 0.f, 0.f, 0.f};
+                D[q] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(A1[q], B0, z, 0, 0, 0);
+                D[q] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(A2[q], B1, D[q], 0, 0, 0);
+            }
+#pragma unroll
+            for (int m = 0; m < M; m++) {
+                if (XBF16) {
+                    acc[s][m] = __builtin_fmaf(D[0][m], sv, acc[s][m]);
+                } else {
+                    const float hi = D[(3 * m) / 4][(3 * m) % 4], mid = D[(3 * m + 1) / 4][(3 * m + 1) % 4], lo = D[(3 * m + 2) / 4][(3 * m + 2) % 4];
+                    acc[s][m] = __builtin_fmaf(__fadd_rn(__fadd_rn(hi, mid), lo), sv, acc[s][m]);
+                }
             }
         }
     }
@@ -188,8 +192,8 @@ struct StripWalk {
     typedef Staging<M, XBF16> St;
     static constexpr int NSET = XBF16 ? 1 : (3 * M + 3) / 4;
     typedef typename std::conditional<XBF16, u32x2, f32x4>::type XV;  // plain vector types: they live in registers
-    unsigned sc[CROW_GEMV_RING];
-    u32x4 cd[CROW_GEMV_RING][2];
+    unsigned sc[CROW_GEMV_RING][1];
+    u32x4 cd[CROW_GEMV_RING][1][2];
     XV xv[CROW_GEMV_RING][M];
     lds_p a1[2][NSET], a2[2][NSET];  // this lane's operand addresses in the two staging slots (or in the zero area)
     lds_p xw;
@@ -197,7 +201,7 @@ struct StripWalk {
     const unsigned char* xl;  // the lane's view of the wave's first column of activation row 0
     size_t xoff[M];           // byte offsets of the activation rows
     int col_lane, k_dim, lane;
-    float acc[M];
+    float acc[1][M];
 
     __device__ __forceinline__ void init(const unsigned char* strip, int first, int k_dim_, const void* x, const size_t (&xoff_elems)[M], lds_p xw_,
                                          lds_p zero) {
@@ -210,7 +214,7 @@ struct StripWalk {
 #pragma unroll
         for (int m = 0; m < M; m++) {
             xoff[m] = xoff_elems[m] * (XBF16 ? 2 : 4);
-            acc[m] = 0.0f;
+            acc[0][m] = 0.0f;
         }
         // this lane as a holder of A operand row i = lane % 16, K group g = lane / 16 (K indices 8 g .. 8 g + 7)
         const int g = lane >> 4, i = lane & 15, r4 = i & 3;
@@ -239,9 +243,9 @@ struct StripWalk {
     template <int J>
     __device__ __forceinline__ void issue_w(int g) {
         const unsigned char* p = wl + (size_t)g * CROW_GROUP_BYTES;
-        sc[J] = stream_load_u32((const unsigned*)p + lane);
-        cd[J][0] = stream_load_v((const uint4*)(p + CROW_GROUP_SCALE_BYTES) + lane);
-        cd[J][1] = stream_load_v((const uint4*)(p + CROW_GROUP_SCALE_BYTES + 1024) + lane);
+        sc[J][0] = stream_load_u32((const unsigned*)p + lane);
+        cd[J][0][0] = stream_load_v((const uint4*)(p + CROW_GROUP_SCALE_BYTES) + lane);
+        cd[J][0][1] = stream_load_v((const uint4*)(p + CROW_GROUP_SCALE_BYTES + 1024) + lane);
     }
     template <int J>
     __device__ __forceinline__ void stage(int g) {
@@ -268,7 +272,7 @@ struct StripWalk {
     }
     template <int J>
     __device__ __forceinline__ void multiply() {
-        group_multiply<M, XBF16>(sc[J], cd[J], a1[J & 1], a2[J & 1], acc);
+        group_multiply<M, XBF16, 1>(sc[J], cd[J], a1[J & 1], a2[J & 1], acc);
         __builtin_amdgcn_wave_barrier();
         // a group is one scheduling region: without the fence the scheduler pulls the decodes of several groups forward in the
         // long straight-line tails of the walk and runs out of registers there
@@ -373,12 +377,169 @@ struct StripWalk {
     __device__ __forceinline__ void finish(float (&out)[M]) const {
 #pragma unroll
         for (int m = 0; m < M; m++) {
-            const unsigned a = __float_as_uint(acc[m]);
+            const unsigned a = __float_as_uint(acc[0][m]);
             const u32x2 sw = __builtin_amdgcn_permlane32_swap(a, a, false, false);  // .x = lanes 0..31's value, .y = lanes 32..63's
             const unsigned b = __float_as_uint(__fadd_rn(__uint_as_float(sw.x), __uint_as_float(sw.y)));
             const u32x2 sq = __builtin_amdgcn_permlane16_swap(b, b, false, false);  // .x = the even 16-lane group's value, .y = the odd one's
             out[m] = __fadd_rn(__uint_as_float(sq.x), __uint_as_float(sq.y));
         }
+    }
+};
+
+// The walk of a wave that takes NS adjacent strips at once (the kernels for several activation rows): per group the staged
+// activations and the operand reads from LDS serve NS x 16 weight rows, which is what bounds those kernels - at four f32 rows a
+// group's operand reads are ten times its weight bytes.  Two groups (NS x 2304 bytes each) in flight; per strip and
+// activation row the operation sequence is StripWalk's, so the sums are the same bits.
+//   wl[s]   the lane's view of the wave's first group of strip s (a strip beyond the tensor: any strip that exists; its
+//           sums are never stored)
+template <int M, bool XBF16, int NS>
+struct MultiWalk {
+    typedef Staging<M, XBF16> St;
+    static constexpr int NSET = XBF16 ? 1 : (3 * M + 3) / 4;
+    typedef typename std::conditional<XBF16, u32x2, f32x4>::type XV;
+    unsigned sc[2][NS];
+    u32x4 cd[2][NS][2];
+    XV xv[2][M];
+    lds_p a1[2][NSET], a2[2][NSET];
+    lds_p xw;
+    const unsigned char* wl[NS];
+    const unsigned char* xl;
+    size_t xoff[M];
+    int col_lane, k_dim, lane;
+    float acc[NS][M];
+
+    __device__ __forceinline__ void init(const unsigned char* const (&strip)[NS], int first, int k_dim_, const void* x, const size_t (&xoff_elems)[M],
+                                         lds_p xw_, lds_p zero) {
+        lane = lane_id();
+        xw = xw_;
+        k_dim = k_dim_;
+#pragma unroll
+        for (int s = 0; s < NS; s++) wl[s] = strip[s] + (size_t)first * CROW_GROUP_BYTES;
+        col_lane = first * CROW_GROUP_COLS + 4 * lane;
+        xl = (const unsigned char*)x;
+#pragma unroll
+        for (int m = 0; m < M; m++) {
+            xoff[m] = xoff_elems[m] * (XBF16 ? 2 : 4);
+#pragma unroll
+            for (int s = 0; s < NS; s++) acc[s][m] = 0.0f;
+        }
+        const int g = lane >> 4, i = lane & 15, r4 = i & 3;
+        const bool half_ok = (g >> 1) == (i >> 3);
+        const bool second = ((i >> 2) & 1) != 0;
+#pragma unroll
+        for (int sl = 0; sl < 2; sl++)
+#pragma unroll
+            for (int q = 0; q < NSET; q++) {
+                const int row = 4 * q + r4;
+                const bool live = half_ok && row < St::XR;
+                lds_p data = xw + sl * St::SLOT + row * CROW_GEMV_XROW_BYTES + 16 * g;
+                a1[sl][q] = (live && !second) ? data : zero + 16 * g;
+                a2[sl][q] = (live && second) ? data + 64 : zero + 16 * g;
+            }
+    }
+    template <int J>
+    __device__ __forceinline__ void issue_x(int g) {
+        const int col = col_lane + g * CROW_GROUP_COLS;
+        const size_t o = (size_t)(col < k_dim ? col : k_dim - 4) * (XBF16 ? 2 : 4);
+#pragma unroll
+        for (int t = 0; t < M; t++) xv[J][t] = *(const __attribute__((address_space(1))) XV*)(xl + xoff[t] + o);
+    }
+    template <int J>
+    __device__ __forceinline__ void issue_w(int g) {
+#pragma unroll
+        for (int s = 0; s < NS; s++) {
+            const unsigned char* p = wl[s] + (size_t)g * CROW_GROUP_BYTES;
+            sc[J][s] = stream_load_u32((const unsigned*)p + lane);
+            cd[J][s][0] = stream_load_v((const uint4*)(p + CROW_GROUP_SCALE_BYTES) + lane);
+            cd[J][s][1] = stream_load_v((const uint4*)(p + CROW_GROUP_SCALE_BYTES + 1024) + lane);
+        }
+    }
+    template <int J>
+    __device__ __forceinline__ void stage(int g) {
+        const bool in = col_lane + g * CROW_GROUP_COLS < k_dim;
+        lds_p slot = xw + J * St::SLOT + 8 * lane;
+#pragma unroll
+        for (int t = 0; t < M; t++) {
+            if constexpr (XBF16) {
+                lds_store8(slot + t * CROW_GEMV_XROW_BYTES, in ? xv[J][t].x : 0u, in ? xv[J][t].y : 0u);
+            } else {
+                unsigned h[4], m[4], l[4];
+                split3(in ? xv[J][t].x : 0.f, h[0], m[0], l[0]);
+                split3(in ? xv[J][t].y : 0.f, h[1], m[1], l[1]);
+                split3(in ? xv[J][t].z : 0.f, h[2], m[2], l[2]);
+                split3(in ? xv[J][t].w : 0.f, h[3], m[3], l[3]);
+                lds_p row = slot + (3 * t) * CROW_GEMV_XROW_BYTES;
+                lds_store8(row, __builtin_amdgcn_perm(h[1], h[0], 0x07060302u), __builtin_amdgcn_perm(h[3], h[2], 0x07060302u));
+                lds_store8(row + CROW_GEMV_XROW_BYTES, __builtin_amdgcn_perm(m[1], m[0], 0x07060302u), __builtin_amdgcn_perm(m[3], m[2], 0x07060302u));
+                lds_store8(row + 2 * CROW_GEMV_XROW_BYTES, __builtin_amdgcn_perm(l[1], l[0], 0x07060302u), __builtin_amdgcn_perm(l[3], l[2], 0x07060302u));
+            }
+        }
+        __builtin_amdgcn_wave_barrier();
+    }
+    template <int J>
+    __device__ __forceinline__ void multiply() {
+        group_multiply<M, XBF16, NS>(sc[J], cd[J], a1[J], a2[J], acc);
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_sched_barrier(0);
+    }
+    // On entry: the weights of groups g0, g0 + 1 are in (or on their way to) slots 0, 1; group g0 is staged; the activations of
+    // g0 + 1 and g0 + 2 are in (or on their way to) x slots 1 and 0.  Requests for groups beyond the wave's run read columns
+    // that exist (or the row's last four) and are never used.  On return, if REFILL, the same holds for g0 + 2.
+    template <bool REFILL>
+    __device__ __forceinline__ void duo(int g0) {
+        stage<1>(g0 + 1);
+        issue_x<1>(g0 + 3);
+        multiply<0>();
+        if (REFILL) {
+            issue_w<0>(g0 + 2);
+            stage<0>(g0 + 2);
+            issue_x<0>(g0 + 4);
+        }
+        multiply<1>();
+        if (REFILL) issue_w<1>(g0 + 3);
+    }
+    // (one copy of each body, and no branch whose two sides begin alike: see StripWalk::go)
+    template <class Mid>
+    __device__ __forceinline__ void go(int count, Mid mid) {
+        const int even = count & ~1;
+        if (even > 0) {
+            issue_x<0>(0);
+            issue_x<1>(1);
+            issue_w<0>(0);
+            issue_w<1>(1);
+            mid();
+            stage<0>(0);
+            issue_x<0>(2);
+            int g = 0;
+            for (; g + 2 < even; g += 2) duo<true>(g);
+            duo<false>(g);
+            if (count & 1) {
+                issue_x<0>(even);
+                issue_w<0>(even);
+                stage<0>(even);
+                multiply<0>();
+            }
+        } else if (count == 1) {
+            issue_x<0>(0);
+            issue_w<0>(0);
+            mid();
+            stage<0>(0);
+            multiply<0>();
+        } else {
+            mid();
+        }
+    }
+    __device__ __forceinline__ void finish(float (&out)[NS][M]) const {
+#pragma unroll
+        for (int s = 0; s < NS; s++)
+#pragma unroll
+            for (int m = 0; m < M; m++) {
+                const unsigned a = __float_as_uint(acc[s][m]);
+                const u32x2 sw = __builtin_amdgcn_permlane32_swap(a, a, false, false);
+                const unsigned b = __float_as_uint(__fadd_rn(__uint_as_float(sw.x), __uint_as_float(sw.y)));
+                const u32x2 sq = __builtin_amdgcn_permlane16_swap(b, b, false, false);
+                out[s][m] = __fadd_rn(__uint_as_float(sq.x), __uint_as_float(sq.y));
+            }
     }
 };
 
@@ -445,13 +606,16 @@ typedef __attribute__((address_space(3))) float* lds_f;
 // The body every GEMV entry point runs.  The caller has already offset the pointers in `a` for its token group / combo `z`,
 // which only indexes the workspace here.  `lds` is the block's dynamic LDS, laid out as described at the top of the file and
 // sized by the launcher for M_ALLOC rows: entry points that dispatch over M size it for their widest body.
-template <int NR, int M, bool XBF16, int EPI, int M_ALLOC = M>
+// NS = strips per block: 1 for the one-row kernels (StripWalk); the kernels for several activation rows take NS adjacent strips
+// per block, every wave all NS of them over its run of columns (MultiWalk), blockIdx.x = strip / NS.
+template <int NR, int M, bool XBF16, int EPI, int M_ALLOC = M, int NS = 1>
 __device__ __forceinline__ void gemv_body(const GemvArgs& a, unsigned z, lds_p lds, const Workspace& ws) {
     static_assert(M <= M_ALLOC, "the allocation covers this body");
     constexpr int AREA = crow_gemv_lds_per_wave(M_ALLOC, XBF16);
+    static_assert(NS * M * 64 <= AREA, "a wave's sums fit its staging area");
     const int lane = lane_id();
     const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6)), waves = block_threads() >> 6;  // wave-uniform on purpose
-    const int strip = (int)blockIdx.x, strips = (int)gridDim.x;
+    const int strip = (int)blockIdx.x * NS, strips = (int)gridDim.x * NS;
     const int slice = (int)blockIdx.y, slices = (int)gridDim.y;
     const int k_dim = a.pairs * CROW_PAIR_COLS;
     const int groups = (a.pairs + CROW_GROUP_PAIRS - 1) / CROW_GROUP_PAIRS;
@@ -465,7 +629,6 @@ __device__ __forceinline__ void gemv_body(const GemvArgs& a, unsigned z, lds_p l
     const bool extra_wave = NR == 2 && wave - r_own * wpt >= wpt;
     const int count = extra_wave ? 0 : base + (unit < rem ? 1 : 0), first = unit * base + (unit < rem ? unit : rem);
     const unsigned char* wsel = r_own != 0 ? a.w[1] : a.w[0];  // a select, never an indexed read
-    const unsigned char* strip_p = wsel + (size_t)strip * groups * CROW_GROUP_BYTES;
     // element offsets of this launch's activation rows, and which output row each of them writes
     size_t xoff[M];
     int yrow[M];
@@ -482,43 +645,68 @@ __device__ __forceinline__ void gemv_body(const GemvArgs& a, unsigned z, lds_p l
     }
     lds_p zero = lds;
     lds_p areas = lds + CROW_GEMV_ZERO_BYTES;
-    StripWalk<M, XBF16> walk;
-    walk.init(strip_p, first, k_dim, a.x, xoff, areas + wave * AREA, zero);
-    walk.go(count, [&]() {  // (the wave's first loads have left by now)
+    auto mid = [&]() {  // (the wave's first loads have left by now)
         for (int o = 16 * (int)threadIdx.x; o < CROW_GEMV_ZERO_BYTES; o += 16 * (waves << 6)) lds_store16(zero + o, 0, 0, 0, 0);
         if (waves > 1) __syncthreads();
         else __builtin_amdgcn_wave_barrier();
-    });
-    float part[M];
-    walk.finish(part);
-
-    // waves of the block -> wave 0: lane l of wave 0 takes output (m = l / 16, n = l % 16) and adds the waves' sums in wave order
-    float v[NR];
+    };
+    float part[NS][M];
+    if constexpr (NS == 1) {
+        StripWalk<M, XBF16> walk;
+        walk.init(wsel + (size_t)strip * groups * CROW_GROUP_BYTES, first, k_dim, a.x, xoff, areas + wave * AREA, zero);
+        walk.go(count, mid);
+        walk.finish(part[0]);
+    } else {
+        // Only the launch's last block can reach past the tensor's last strip: it alone reads the row count before its first
+        // weight load, and reads an existing strip instead (the sums of a strip beyond the tensor are never stored).
+        int have = NS;
+        if (blockIdx.x + 1 == gridDim.x) {
+            const int left = (*a.rows_p + CROW_STRIP_ROWS - 1) / CROW_STRIP_ROWS - strip;
+            have = left < 1 ? 1 : (left < NS ? left : NS);
+        }
+        const unsigned char* sp[NS];
 #pragma unroll
-    for (int r = 0; r < NR; r++) v[r] = 0.0f;
+        for (int s = 0; s < NS; s++) sp[s] = wsel + (size_t)(strip + (s < have ? s : 0)) * groups * CROW_GROUP_BYTES;
+        MultiWalk<M, XBF16, NS> walk;
+        walk.init(sp, first, k_dim, a.x, xoff, areas + wave * AREA, zero);
+        walk.go(count, mid);
+        walk.finish(part);
+    }
+
+    // waves of the block -> wave 0: lane l of wave 0 takes output (m = l / 16, n = l % 16) of every strip and adds the waves'
+    // sums in wave order
+    float v[NR * NS];
+#pragma unroll
+    for (int r = 0; r < NR * NS; r++) v[r] = 0.0f;
     const int mo = lane >> 4, n = lane & 15;
     if (waves > 1) {
         if (lane < 16) {
 #pragma unroll
-            for (int m = 0; m < M; m++) ((lds_f)(areas + wave * AREA))[m * 16 + lane] = part[m];
+            for (int s = 0; s < NS; s++)
+#pragma unroll
+                for (int m = 0; m < M; m++) ((lds_f)(areas + wave * AREA))[(s * M + m) * 16 + lane] = part[s][m];
         }
         __syncthreads();
         if (wave > 0) return;
         if (mo < M) {
 #pragma unroll
-            for (int r = 0; r < NR; r++) {
-                v[r] = ((lds_f)(areas + (r * wpt) * AREA))[lane];
-                for (int w = 1; w < wpt; w++) v[r] += ((lds_f)(areas + (r * wpt + w) * AREA))[lane];
-            }
+            for (int r = 0; r < NR; r++)
+#pragma unroll
+                for (int s = 0; s < NS; s++) {
+                    v[r * NS + s] = ((lds_f)(areas + (r * wpt) * AREA))[s * M * 16 + lane];
+                    for (int w = 1; w < wpt; w++) v[r * NS + s] += ((lds_f)(areas + (r * wpt + w) * AREA))[s * M * 16 + lane];
+                }
         }
     } else {
 #pragma unroll
-        for (int m = 0; m < M; m++)
-            if (mo == m) v[0] = part[m];
+        for (int s = 0; s < NS; s++)
+#pragma unroll
+            for (int m = 0; m < M; m++)
+                if (mo == m) v[s] = part[s][m];
     }
 
-    // slices of the strip -> the last one to arrive, in slice order
-    if (slices > 1 && !slice_hand_over<NR>(v, z * (unsigned)strips + (unsigned)strip, slice, slices, ws, lane)) return;
+    // slices of the block's strips -> the last one to arrive, in slice order
+    if (slices > 1 && !slice_hand_over<NR * NS>(v, z * gridDim.x + blockIdx.x, slice, slices, ws, lane)) return;
 
     const int rows = *a.rows_p;
     // the launch geometry was made for another problem, or the two tensors cannot share the block's waves evenly: nothing is stored
@@ -527,69 +715,76 @@ __device__ __forceinline__ void gemv_body(const GemvArgs& a, unsigned z, lds_p l
         if (lane == 0) atomicOr(ws.status, STATUS_BAD_SHAPE);
         return;
     }
-    const int row = strip * CROW_STRIP_ROWS + n;
-    if (EPI == EPI_SCALE && a.argmax_out != nullptr) {
-        // fused head: logits out, and the greedy token of the whole launch from its last block (device_common.h: the head's
-        // scratch).  Same total order as argmax_k, whatever order the blocks finish in.
-        typedef __attribute__((address_space(1))) unsigned long long* gk_p;
-        const float val = v[0] * a.gs[0][0];
-        const bool live = mo == 0 && row < rows;
-        if (live) a.y[row] = val;
-        const Best b = wave_best(Best{live ? val : -3.0e38f, live ? row : 0});
-        gk_p words = (gk_p)ws.head;
-        const unsigned slot = (unsigned)strip % CROW_HEAD_SLOTS, n_strips = (unsigned)strips;
-        constexpr unsigned long long COUNT = (1ull << CROW_HEAD_COUNT_BITS) - 1;
-        unsigned last = 0;
-        if (lane == 0) {
-            // candidate in and block counted in one step; a failed swap means another block of the slot got in, so at most
-            // (blocks of the slot - 1) retries
-            const unsigned in_slot = (n_strips - slot + CROW_HEAD_SLOTS - 1) / CROW_HEAD_SLOTS;
-            const unsigned long long mine = best_key(b.v, b.i);
-            unsigned long long w = __hip_atomic_load(words + 16 * slot, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT), nw;
-            do {
-                const unsigned long long cur = w >> CROW_HEAD_COUNT_BITS;
-                nw = ((cur > mine ? cur : mine) << CROW_HEAD_COUNT_BITS) | ((w & COUNT) + 1);
-            } while (!__hip_atomic_compare_exchange_strong(words + 16 * slot, &w, nw, __ATOMIC_RELAXED, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT));
-            last = (nw & COUNT) == in_slot ? 1u : 0u;
-        }
-        if (__builtin_amdgcn_readfirstlane(last) == 0) return;
-        // This block completed its slot.  If it now reads every slot complete it has every slot's final key: it writes the
-        // token and zeroes the words.  (The block that completed the last slot always does; should another one read all
-        // slots complete as well, it computes the same token; one that reads a word already zeroed stands back.)
-        device_order();
-        unsigned long long best = 0;
-        bool complete = true;
-#pragma unroll
-        for (int j = 0; j < CROW_HEAD_SLOTS / 64; j++) {
-            const unsigned s = (unsigned)lane + 64u * j;
-            if (s < n_strips) {
-                const unsigned long long w = __hip_atomic_load(words + 16 * s, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-                complete = complete && (w & COUNT) == (n_strips - s + CROW_HEAD_SLOTS - 1) / CROW_HEAD_SLOTS;
-                best = (w >> CROW_HEAD_COUNT_BITS) > best ? (w >> CROW_HEAD_COUNT_BITS) : best;
+    if constexpr (NS == 1 && EPI == EPI_SCALE) {
+        const int row = strip * CROW_STRIP_ROWS + n;
+        if (a.argmax_out != nullptr) {
+            // fused head: logits out, and the greedy token of the whole launch from its last block (device_common.h: the head's
+            // scratch).  Same total order as argmax_k, whatever order the blocks finish in.
+            typedef __attribute__((address_space(1))) unsigned long long* gk_p;
+            const float val = v[0] * a.gs[0][0];
+            const bool live = mo == 0 && row < rows;
+            if (live) a.y[row] = val;
+            const Best b = wave_best(Best{live ? val : -3.0e38f, live ? row : 0});
+            gk_p words = (gk_p)ws.head;
+            const unsigned slot = (unsigned)strip % CROW_HEAD_SLOTS, n_strips = (unsigned)strips;
+            constexpr unsigned long long COUNT = (1ull << CROW_HEAD_COUNT_BITS) - 1;
+            unsigned last = 0;
+            if (lane == 0) {
+                // candidate in and block counted in one step; a failed swap means another block of the slot got in, so at most
+                // (blocks of the slot - 1) retries
+                const unsigned in_slot = (n_strips - slot + CROW_HEAD_SLOTS - 1) / CROW_HEAD_SLOTS;
+                const unsigned long long mine = best_key(b.v, b.i);
+                unsigned long long w = __hip_atomic_load(words + 16 * slot, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT), nw;
+                do {
+                    const unsigned long long cur = w >> CROW_HEAD_COUNT_BITS;
+                    nw = ((cur > mine ? cur : mine) << CROW_HEAD_COUNT_BITS) | ((w & COUNT) + 1);
+                } while (!__hip_atomic_compare_exchange_strong(words + 16 * slot, &w, nw, __ATOMIC_RELAXED, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT));
+                last = (nw & COUNT) == in_slot ? 1u : 0u;
             }
-        }
-        if (__builtin_amdgcn_ballot_w64(!complete) != 0ull) return;
+            if (__builtin_amdgcn_readfirstlane(last) == 0) return;
+            // This block completed its slot.  If it now reads every slot complete it has every slot's final key: it writes the
+            // token and zeroes the words.  (The block that completed the last slot always does; should another one read all
+            // slots complete as well, it computes the same token; one that reads a word already zeroed stands back.)
+            device_order();
+            unsigned long long best = 0;
+            bool complete = true;
 #pragma unroll
-        for (int j = 0; j < CROW_HEAD_SLOTS / 64; j++)
-            if ((unsigned)lane + 64u * j < n_strips)
-                __hip_atomic_store(words + 16 * (lane + 64 * j), 0ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        for (int o = 32; o > 0; o >>= 1) {
-            const unsigned long long other = ((unsigned long long)__shfl_xor((unsigned)(best >> 32), o) << 32) | __shfl_xor((unsigned)best, o);
-            best = other > best ? other : best;
+            for (int j = 0; j < CROW_HEAD_SLOTS / 64; j++) {
+                const unsigned s = (unsigned)lane + 64u * j;
+                if (s < n_strips) {
+                    const unsigned long long w = __hip_atomic_load(words + 16 * s, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                    complete = complete && (w & COUNT) == (n_strips - s + CROW_HEAD_SLOTS - 1) / CROW_HEAD_SLOTS;
+                    best = (w >> CROW_HEAD_COUNT_BITS) > best ? (w >> CROW_HEAD_COUNT_BITS) : best;
+                }
+            }
+            if (__builtin_amdgcn_ballot_w64(!complete) != 0ull) return;
+#pragma unroll
+            for (int j = 0; j < CROW_HEAD_SLOTS / 64; j++)
+                if ((unsigned)lane + 64u * j < n_strips)
+                    __hip_atomic_store(words + 16 * (lane + 64 * j), 0ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            for (int o = 32; o > 0; o >>= 1) {
+                const unsigned long long other = ((unsigned long long)__shfl_xor((unsigned)(best >> 32), o) << 32) | __shfl_xor((unsigned)best, o);
+                best = other > best ? other : best;
+            }
+            if (lane == 0) a.argmax_out[0] = best != 0ull ? best_key_index(best) : 0;
+            return;
         }
-        if (lane == 0) a.argmax_out[0] = best != 0ull ? best_key_index(best) : 0;
-        return;
     }
-    if (mo >= M || row >= rows) return;
+    if (mo >= M) return;
     int yr = yrow[0];
 #pragma unroll
     for (int m = 1; m < M; m++)
         if (mo == m) yr = yrow[m];
     const size_t yo = (size_t)yr * (a.y_stride != 0 ? a.y_stride : (size_t)rows);
-    if (EPI == EPI_SCALE) {
-        a.y[yo + row] = v[0] * a.gs[0][0];
-    } else {
-        a.y[yo + row] = silu_mul(v[0] * a.gs[0][0], v[NR - 1] * a.gs[NR - 1][0]);
+#pragma unroll
+    for (int s = 0; s < NS; s++) {
+        const int row = (strip + s) * CROW_STRIP_ROWS + n;
+        if (row >= rows) continue;
+        if (EPI == EPI_SCALE) {
+            a.y[yo + row] = v[s] * a.gs[0][0];
+        } else {
+            a.y[yo + row] = silu_mul(v[s] * a.gs[0][0], v[(NR - 1) * NS + s] * a.gs[NR - 1][0]);
+        }
     }
 }
 

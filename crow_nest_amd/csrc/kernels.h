@@ -111,6 +111,11 @@ extern "C" __global__ void CROW_ONE_ROW_BF16 __launch_bounds__(1024) gemv_nvfp4_
 }
 
 // ------------------------------------------------------------------ M <= 4 rows (MTP verify)
+// Every kernel that multiplies several activation rows at once takes this many adjacent 16-row strips per block (gemv.h:
+// MultiWalk); crow_hip_launch_dims sizes grid.x accordingly.
+#ifndef CROW_MULTI_STRIPS
+#define CROW_MULTI_STRIPS 2
+#endif
 template <int NR, bool XBF16, int EPI>
 __device__ __forceinline__ void gemv_m_dispatch(const GemvArgs& a, int m, unsigned z, lds_p lds, const Workspace& ws) {
     if (m < 1 || m > 4) {  // the reference's NVFP4_MMAX (engine/src/kernels_p2.rs:397-400); uniform over the launch
@@ -119,10 +124,10 @@ __device__ __forceinline__ void gemv_m_dispatch(const GemvArgs& a, int m, unsign
     }
     // one body per M keeps each row's operation sequence identical to the one-row kernel
     switch (m) {
-        case 1: gemv_body<NR, 1, XBF16, EPI, 4>(a, z, lds, ws); break;
-        case 2: gemv_body<NR, 2, XBF16, EPI, 4>(a, z, lds, ws); break;
-        case 3: gemv_body<NR, 3, XBF16, EPI, 4>(a, z, lds, ws); break;
-        default: gemv_body<NR, 4, XBF16, EPI, 4>(a, z, lds, ws); break;
+        case 1: gemv_body<NR, 1, XBF16, EPI, 4, CROW_MULTI_STRIPS>(a, z, lds, ws); break;
+        case 2: gemv_body<NR, 2, XBF16, EPI, 4, CROW_MULTI_STRIPS>(a, z, lds, ws); break;
+        case 3: gemv_body<NR, 3, XBF16, EPI, 4, CROW_MULTI_STRIPS>(a, z, lds, ws); break;
+        default: gemv_body<NR, 4, XBF16, EPI, 4, CROW_MULTI_STRIPS>(a, z, lds, ws); break;
     }
 }
 // The activation row count of a verify launch: from the geometry word when the launcher put it there (then the word behind
@@ -157,7 +162,7 @@ extern "C" __global__ void __launch_bounds__(512) gemv_nvfp4_gum(const unsigned 
     gemv_m_dispatch<2, false, EPI_SILU_GU>(a, rows_of(a, geo, m_p), 0, LDS, ws);
 }
 // bf16-activation twins of the two verify kernels (X [M][k_dim] bf16, outputs f32)
-extern "C" __global__ void __launch_bounds__(1024) gemv_nvfp4_wm_bf16(const unsigned char* __restrict__ w, const unsigned short* __restrict__ x,
+extern "C" __global__ void __launch_bounds__(512) gemv_nvfp4_wm_bf16(const unsigned char* __restrict__ w, const unsigned short* __restrict__ x,
                                                                       const float* __restrict__ gs_ptr, float* __restrict__ y,
                                                                       const int* __restrict__ k_dim_p, const int* __restrict__ rows_p,
                                                                       const int* __restrict__ m_p, int geo, const Workspace ws) {
@@ -166,7 +171,7 @@ extern "C" __global__ void __launch_bounds__(1024) gemv_nvfp4_wm_bf16(const unsi
     GemvArgs a = gemv_args(w, nullptr, gs_ptr, nullptr, x, (size_t)pairs * CROW_PAIR_COLS, y, 0, pairs, k_dim_p, rows_p);
     gemv_m_dispatch<1, true, EPI_SCALE>(a, rows_of(a, geo, m_p), 0, LDS, ws);
 }
-extern "C" __global__ void __launch_bounds__(1024) gemv_nvfp4_gum_bf16(const unsigned char* __restrict__ wg, const unsigned char* __restrict__ wu,
+extern "C" __global__ void __launch_bounds__(512) gemv_nvfp4_gum_bf16(const unsigned char* __restrict__ wg, const unsigned char* __restrict__ wu,
                                                                        const unsigned short* __restrict__ x, const float* __restrict__ gs_g,
                                                                        const float* __restrict__ gs_u, float* __restrict__ y,
                                                                        const int* __restrict__ k_dim_p, const int* __restrict__ rows_p,

@@ -78,8 +78,9 @@ def test_launch_dims_depend_on_the_matrix_only():
     d1, d4 = L.Dims(), L.Dims()
     assert lib.crow_hip_launch_dims(b"gemv_nvfp4_w", 17408, 5120, 1, C.byref(d1)) == 0
     assert lib.crow_hip_launch_dims(b"gemv_nvfp4_wm", 17408, 5120, 1, C.byref(d4)) == 0
-    # verify rows == decode row, bit for bit: same grid, same block, same K word and slice count; only the row hint differs
-    assert (d1.gx, d1.gy & 0xFF0FFFFF, d1.gz, d1.bx) == (d4.gx, d4.gy & 0xFF0FFFFF, d4.gz, d4.bx)
+    # verify rows == decode row, bit for bit: same split of K over waves and slices (it fixes the order of the sums); the verify
+    # kernel's blocks take two strips each, and the row hint differs
+    assert (d1.gy & 0xFF0FFFFF, d1.gz, d1.bx) == (d4.gy & 0xFF0FFFFF, d4.gz, d4.bx) and d4.gx == (d1.gx + 1) // 2
     assert d1.gx == 17408 // 16 and d1.bx == 3 * 64 and d1.gy == (5120 // 64) | (1 << 24)  # one block per strip, whole K inside it
     assert (d4.gy >> 20) & 0xF == 1
     assert lib.crow_hip_launch_dims(b"gemv_nvfp4_w", 5120, 17408, 1, C.byref(d1)) == 0
