@@ -6,6 +6,7 @@
 #include <cstring>
 
 #include "../../include/crow_hip.h"
+#include "../../include/crow_hip_bench.h"
 #include "kernels.h"
 #include "misc_kernels.h"
 #include "gemm.h"

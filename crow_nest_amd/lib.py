@@ -100,14 +100,17 @@ def lib():
     return L
 
 
+# include/crow_hip_bench.h: timing loops and the forced GEMV split, for bench.py and the tests (not part of the drop-in ABI)
+BENCH_EXPORTS = ["crow_hip_launch_dims_split", "crow_hip_time_launches", "crow_hip_time_sequence", "crow_hip_time_graph"]
+
 EXPORTS = [
     "crow_hip_init", "crow_hip_shutdown", "crow_hip_error_string", "crow_hip_device_name", "crow_hip_module_load",
     "crow_hip_module_unload", "crow_hip_module_get", "crow_hip_get_function", "crow_hip_function_count",
     "crow_hip_function_name", "crow_hip_function_arg_count", "crow_hip_set_geo", "crow_hip_launch", "crow_hip_launch_noalloc",
-    "crow_hip_launch_dims", "crow_hip_launch_dims_split", "crow_hip_gemm_kernel", "crow_hip_status", "crow_hip_reset_workspace", "crow_hip_set_stream", "crow_hip_cur_stream",
-    "crow_hip_sync", "crow_hip_event_create", "crow_hip_event_record", "crow_hip_event_elapsed_ms", "crow_hip_event_destroy", "crow_hip_time_launches", "crow_hip_time_sequence", "crow_hip_alloc", "crow_hip_free", "crow_hip_upload", "crow_hip_download",
+    "crow_hip_launch_dims", "crow_hip_gemm_kernel", "crow_hip_status", "crow_hip_reset_workspace", "crow_hip_set_stream", "crow_hip_cur_stream",
+    "crow_hip_sync", "crow_hip_event_create", "crow_hip_event_record", "crow_hip_event_elapsed_ms", "crow_hip_event_destroy", "crow_hip_alloc", "crow_hip_free", "crow_hip_upload", "crow_hip_download",
     "crow_hip_stream_create", "crow_hip_stream_destroy", "crow_hip_begin_capture", "crow_hip_end_capture_instantiate",
-    "crow_hip_launch_graph", "crow_hip_graph_exec_destroy", "crow_hip_time_graph",
+    "crow_hip_launch_graph", "crow_hip_graph_exec_destroy",
     "crow_hip_container_bytes", "crow_hip_tiled_bytes", "crow_hip_tile_code_offset", "crow_hip_tile_scale_offset", "crow_hip_repack_nvfp4", "crow_hip_unpack_nvfp4",
     "crow_hip_dequant_tiled",
 ]

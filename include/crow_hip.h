@@ -93,10 +93,6 @@ int crow_hip_launch_noalloc(crow_fn_t f, uint32_t gx, uint32_t gy, uint32_t gz, 
 /* grid/block for `name` on a [rows, k_dim] tensor with `z` token rows (batched and verify kernels: the value *t_p / *m_p
  * will hold) or combos (routed kernels); 1 otherwise.  The split of the work depends on (rows, k_dim) only, never on z. */
 int crow_hip_launch_dims(const char* name, uint32_t rows, uint32_t k_dim, uint32_t z, crow_dims* out);
-/* the same with the GEMV split forced: `s` column slices per 16-row strip (blocks that hand their partial sums over through
- * the workspace) and `w` waves per block and tensor; 0 = the library's choice.  Every GEMV kernel is correct for every split:
- * this is for tuning and for tests.  Other kernels ignore s and w. */
-int crow_hip_launch_dims_split(const char* name, uint32_t rows, uint32_t k_dim, uint32_t z, uint32_t s, uint32_t w, crow_dims* out);
 /* the GEMM entry point (a name of the kernel table) that serves `m` token rows fastest on a tensor of `rows` rows: the
  * choice depends on how the blocks of each tiling fall on this device's compute units */
 const char* crow_hip_gemm_kernel(uint32_t rows, uint32_t m);
@@ -119,16 +115,6 @@ int crow_hip_event_create(void** out);
 int crow_hip_event_record(void* ev);                              /* on the current stream */
 int crow_hip_event_elapsed_ms(void* start, void* stop, float* ms); /* waits for `stop` */
 int crow_hip_event_destroy(void* ev);
-/* `iters` back-to-back launches of `f` on the current stream between two events, launch i taking
- * the argument set vals[(i % n_sets) * n_vals ...] (rotating weight copies keep the working set
- * larger than the 256 MB memory-side cache).  Returns the mean microseconds per launch. */
-int crow_hip_time_launches(crow_fn_t f, uint32_t gx, uint32_t gy, uint32_t gz, uint32_t bx, const uint64_t* vals,
-                           uint32_t n_vals, uint32_t n_sets, uint32_t iters, float* us_per_launch);
-/* the same for a SEQUENCE of n_kernels launches per iteration (e.g. router -> gate|up -> down): dims[k] and
- * n_vals[k] per kernel; argument set s of iteration i = vals + (i % n_sets) * sum(n_vals), kernels back to back
- * inside it.  Returns the mean microseconds per iteration (per sequence). */
-int crow_hip_time_sequence(uint32_t n_kernels, const crow_fn_t* fns, const crow_dims* dims, const uint32_t* n_vals,
-                           const uint64_t* vals, uint32_t n_sets, uint32_t iters, float* us_per_iteration);
 
 /* ---- graph capture: cuda::stream_create_non_blocking / begin_capture / end_capture_instantiate / launch_graph /
  * graph_exec_destroy / stream_destroy, engine/src/cuda.rs:113-203.  A launch sequence issued with crow_hip_launch
@@ -141,8 +127,6 @@ int crow_hip_begin_capture(void* stream);       /* also makes `stream` the curre
 int crow_hip_end_capture_instantiate(void* stream, void** graph_exec_out); /* the template graph is destroyed */
 int crow_hip_launch_graph(void* graph_exec, void* stream);
 int crow_hip_graph_exec_destroy(void* graph_exec);
-/* `iters` back-to-back replays on `stream` between two events; mean microseconds per replay */
-int crow_hip_time_graph(void* graph_exec, void* stream, uint32_t iters, float* us_per_replay);
 
 /* ---- load-time repack (the one call the reference does not have) ---- */
 size_t crow_hip_container_bytes(uint32_t rows, uint32_t cols);

@@ -12,8 +12,8 @@ from crow_nest_amd import lib as L
 from crow_nest_amd.weights import Nvfp4Matrix
 
 
-def _declared():
-    text = open(os.path.join(ROOT, "include", "crow_hip.h")).read()
+def _declared(header="crow_hip.h"):
+    text = open(os.path.join(ROOT, "include", header)).read()
     text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
     return sorted(set(re.findall(r"\b(crow_hip_[a-z0-9_]+)\s*\(", text)))
 
@@ -26,6 +26,11 @@ def test_library_exports_every_declared_symbol():
     for name in declared:
         assert hasattr(lib, name), f"{name} is declared in include/crow_hip.h but not exported"
     assert sorted(L.EXPORTS) == declared
+    # the timing and tuning helpers of the benchmark and the tests live in a header of their own, outside the product ABI
+    bench = _declared("crow_hip_bench.h")
+    assert bench == sorted(L.BENCH_EXPORTS) and not set(bench) & set(declared)
+    for name in bench:
+        assert hasattr(lib, name), f"{name} is declared in include/crow_hip_bench.h but not exported"
 
 
 def test_kernel_table_names_without_a_device():

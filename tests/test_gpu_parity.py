@@ -191,6 +191,59 @@ def test_split_launches_back_to_back_with_changing_inputs(eng):
             assert rel_err(got[i], ref[i]) <= TOL, (s, wv, i)
 
 
+def test_five_thousand_hand_overs_in_a_row_give_the_same_bits(eng):
+    """The cross-block hand-over under sustained load: 5,000 launches back to back of the split GEMV at the benchmark's down
+    projection size (5 column slices per strip through the workspace) and as many of the K-split 16-token GEMM at full size,
+    rotating over 8 inputs; every result is compared bit for bit with the first result for its input (on the device, after
+    every round of 8), and the first results with the CPU path."""
+    from crow_nest_amd.kernels import launch_dims, launch_v
+    p = eng.p
+    rounds = 625
+    # --- the split GEMV [5120, 17408]
+    rows, cols = 5120, 17408
+    w = random_nvfp4(501, rows, cols)
+    gs = 2.0e-4
+    f = _load(w, rows, cols, gs)
+    xs = np.stack([normal_f32(502, i, cols) for i in range(8)])
+    xd = _dev(xs)
+    dims = launch_dims("gemv_nvfp4_w", rows, cols)
+    assert dims[1] >> 24 > 1
+    y = torch.empty((8, rows), dtype=torch.float32, device="cuda")
+    first = None
+    for r in range(rounds):
+        for i in range(8):
+            launch_v(eng.k.f("gemv_nvfp4_w"), *dims, [f.w_ptr, xd[i].data_ptr(), f.gs_ptr, y[i].data_ptr(), p.i32(cols), p.i32(rows)])
+        if first is None:
+            first = y.clone()
+        else:
+            assert torch.equal(y.view(torch.int32), first.view(torch.int32)), f"GEMV round {r}"
+        y.fill_(-1.0)
+    eng.check()
+    got = first.cpu().numpy()
+    for i in (0, 7):
+        assert gamma_rows(got[i][:256], w, 0, 256, cols, gs, xs[i]) <= 1.0
+    # --- the K-split GEMM for 16 tokens on [17408, 5120]
+    rows, cols, m = 17408, 5120, 16
+    w = random_nvfp4(503, rows, cols)
+    f = _load(w, rows, cols, gs)
+    xb = [_bf16_dev(normal_f32(504, i, m * cols).reshape(m, cols)) for i in range(8)]
+    dims = launch_dims("gemm_nvfp4_bf16_m16", rows, cols, m)
+    assert dims[2] > 1  # the panels are dealt over several blocks per row tile
+    y = torch.empty((8, m, rows), dtype=torch.float32, device="cuda")
+    first = None
+    for r in range(rounds):
+        for i in range(8):
+            launch_v(eng.k.f("gemm_nvfp4_bf16_m16"), *dims, [f.w_ptr, xb[i][0].data_ptr(), f.gs_ptr, y[i].data_ptr(), p.i32(cols), p.i32(rows), p.i32(m)])
+        if first is None:
+            first = y.clone()
+        else:
+            assert torch.equal(y.view(torch.int32), first.view(torch.int32)), f"GEMM round {r}"
+        y.fill_(-1.0)
+    eng.check()
+    got = first.cpu().numpy()
+    assert gamma_rows(got[3][:, :128], w, 0, 128, cols, gs, xb[3][1]) <= 1.0
+
+
 def test_verify_rows_are_bit_identical_to_one_row_decode(eng):
     """kernels_p2.rs:391-396: row m of an M-row launch == a one-row launch on x row m."""
     rows, cols = 700, 5120
