@@ -115,7 +115,7 @@ def status() -> None:
 
 
 def launch_dims(name: str, rows: int, k_dim: int, z: int = 1, split: tuple[int, int] = (0, 0)) -> tuple[int, int, int, int]:
-    """Grid and block the library chooses; `split` = (column slices per row tile, waves per block) forces a GEMV split."""
+    """Grid and block the library chooses; `split` = (column slices per strip, waves per block and tensor) forces a GEMV split."""
     d = _l.Dims()
     rc = _l.lib().crow_hip_launch_dims_split(name.encode(), rows, k_dim, z, split[0], split[1], C.byref(d))
     if rc == -2:
