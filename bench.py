@@ -276,6 +276,19 @@ def main() -> int:
             time_sequence(seq, n_sets, max(n_sets, iters // 10))
             return med_min([time_sequence(seq, n_sets, iters) for _ in range(REPS)])
 
+        # config 0 the reference's way: lanes across the columns, f32 multiply-adds, no matrix instructions, container layout
+        # (measurement only: the A/B behind running one activation row on the matrix cores)
+        raw = [torch.from_numpy(host["gate"][0]).to(dev) for _ in range(copies)]
+        best = None
+        for nm in ("gemv_nvfp4_w_valu1", "gemv_nvfp4_w_valu2", "gemv_nvfp4_w_valu4"):
+            lv = Launch(eng, nm, N, K, 1, [[r_.data_ptr(), xk0.data_ptr(), base["gate"].gs_ptr, ybuf.data_ptr(), p.i32(K), p.i32(N)] for r_ in raw])
+            t_ = lv.us()
+            if best is None or t_[0] < best[1][0]:
+                best = (nm, t_)
+        others["config0_without_matrix_instructions"] = entry(best[1], c0_bytes)
+        others["config0_without_matrix_instructions"]["kernel"] = best[0]
+        others["config0_without_matrix_instructions"]["vs_matrix_core_kernel"] = round(best[1][0] / c0_us, 2)
+        del raw
         # config 1 at verify widths
         for m in (2, 4):
             lg = Launch(eng, "gemv_nvfp4_gum_bf16", N, K, m,

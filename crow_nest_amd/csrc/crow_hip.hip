@@ -51,6 +51,7 @@ const FnEntry g_table[] = {
     {"gemm_nvfp4_bf16_m96", (const void*)&gemm_nvfp4_bf16_m96, 7, 2u * 96u * 528u, 0, 16, 0, 1, false},
     CROW_FN(gemm_nvfp4_bf16_m32, 7), CROW_FN(gemm_nvfp4_bf16_m16, 7), CROW_FN(gemv_bf16_w, 5),
     CROW_FN(gemv_bf16, 5), CROW_FN(gemv_bf16_b, 5), CROW_FN(gemv_b, 5), CROW_FN(gemv_bf16_ws, 5), CROW_FN(gemv_bf16_bs, 6),
+    CROW_FN(gemv_nvfp4_w_valu1, 6), CROW_FN(gemv_nvfp4_w_valu2, 6), CROW_FN(gemv_nvfp4_w_valu4, 6),  // measurement only
 };
 const int g_table_n = (int)(sizeof(g_table) / sizeof(g_table[0]));
 
@@ -395,6 +396,12 @@ int crow_hip_launch_dims_split(const char* name, uint32_t rows, uint32_t k_dim, 
         const uint32_t gx = (strips + (uint32_t)e->ns - 1) / (uint32_t)e->ns;
         *out = crow_dims{gx, pairs | (hint << 20) | (s << 24), gz, 64u * w * (uint32_t)e->nr};
         if (s > 1 && ((unsigned long long)gx * gz * s * (unsigned)(e->nr * e->ns) * 64 > PARTIAL_FLOATS || (unsigned long long)gx * gz > COUNTER_SLOTS)) return CROW_ERR_WORKSPACE;
+        return CROW_OK;
+    }
+    if (strncmp(name, "gemv_nvfp4_w_valu", 17) == 0) {  // a 16-lane group per RG rows, four groups per wave, four waves per block
+        if (k_dim == 0 || k_dim % CROW_BLOCK_VALUES != 0) return CROW_ERR_SHAPE;
+        const uint32_t per_block = 16u * (uint32_t)(name[17] - '0');
+        *out = crow_dims{(rows + per_block - 1) / per_block, 1, 1, 256};
         return CROW_OK;
     }
     if (strncmp(name, "gemm_nvfp4_bf16", 15) == 0) {  // z = M token rows

@@ -573,3 +573,78 @@ extern "C" __global__ void __launch_bounds__(256) gemv_bf16_bs(const unsigned sh
     }
     keep_gemv_body<true>(w, x, y, *k_dim_p, *rows_p, (size_t)*y_stride_p);
 }
+
+// ------------------------------------------------------------------ measurement only: the one-row GEMV without matrix instructions
+// The reference's own shape for this product (kernels_p2.rs:304-368: a warp per few rows, lanes across the columns, f32
+// multiply-adds on decoded weights, a shuffle tree) written for 64-wide waves, on the CONTAINER layout as it stands (no repack),
+// so that the choice of the matrix cores for one activation row rests on a measured number.  Not part of the drop-in set:
+// the engine never asks for it.  Each 16-lane group of a wave owns RG adjacent rows and its lanes take every 16th 64-value
+// block of them: per block and row one scale dword + eight code dwords, 32 conversions, 64 multiply-adds against the 64
+// activations the lane holds for all its rows, one scale multiply-add per 16 values.  grid (ceil(rows / (16 RG))), block 256.
+template <int RG>
+__device__ __forceinline__ void gemv_valu_body(const unsigned char* __restrict__ w, const float* __restrict__ x, const float* __restrict__ gs_ptr,
+                                               float* __restrict__ y, int k_dim, int rows) {
+    const int lane = lane_id(), wave = (int)(threadIdx.x >> 6);
+    const int nb = k_dim / CROW_BLOCK_VALUES;
+    const int row0 = (((int)blockIdx.x * 4 + wave) * 4 + (lane >> 4)) * RG, j = lane & 15;
+    float acc[RG];
+#pragma unroll
+    for (int r = 0; r < RG; r++) acc[r] = 0.0f;
+    for (int b = j; b < nb; b += 16) {
+        f32x4 xv[16];
+#pragma unroll
+        for (int i = 0; i < 16; i++) xv[i] = *(const f32x4*)(x + (size_t)b * 64 + 4 * i);
+#pragma unroll
+        for (int r = 0; r < RG; r++) {
+            const int row = row0 + r < rows ? row0 + r : rows - 1;
+            const unsigned* blk = (const unsigned*)(w + ((size_t)row * nb + b) * CROW_BLOCK_BYTES);
+            // the scale rule on four bytes at once: bit 7 cleared, 0x7F -> 0x7E
+            unsigned sc = stream_load_u32(blk) & 0x7F7F7F7Fu;
+            sc -= ((sc + 0x01010101u) & 0x80808080u) >> 7;
+            unsigned c[8];
+#pragma unroll
+            for (int i = 0; i < 8; i++) c[i] = stream_load_u32(blk + 1 + i);
+#pragma unroll
+            for (int sb = 0; sb < 4; sb++) {
+                float part = 0.0f;
+#pragma unroll
+                for (int h = 0; h < 2; h++) {
+                    const unsigned cw = c[2 * sb + h];
+                    const f32x2 v0 = fp4x2_to_f32<0>(cw), v1 = fp4x2_to_f32<1>(cw), v2 = fp4x2_to_f32<2>(cw), v3 = fp4x2_to_f32<3>(cw);
+                    const f32x4 xa = xv[4 * sb + 2 * h], xb = xv[4 * sb + 2 * h + 1];
+                    part = __builtin_fmaf(v0.x, xa.x, part);
+                    part = __builtin_fmaf(v0.y, xa.y, part);
+                    part = __builtin_fmaf(v1.x, xa.z, part);
+                    part = __builtin_fmaf(v1.y, xa.w, part);
+                    part = __builtin_fmaf(v2.x, xb.x, part);
+                    part = __builtin_fmaf(v2.y, xb.y, part);
+                    part = __builtin_fmaf(v3.x, xb.z, part);
+                    part = __builtin_fmaf(v3.y, xb.w, part);
+                }
+                const float sv = sb == 0 ? e4m3_to_f32<0>(sc) : (sb == 1 ? e4m3_to_f32<1>(sc) : (sb == 2 ? e4m3_to_f32<2>(sc) : e4m3_to_f32<3>(sc)));
+                acc[r] = __builtin_fmaf(part, sv, acc[r]);
+            }
+        }
+    }
+    const float gs = gs_ptr[0];
+#pragma unroll
+    for (int r = 0; r < RG; r++) {
+        float v = acc[r];
+        for (int o = 8; o > 0; o >>= 1) v += __shfl_xor(v, o);
+        if (j == 0 && row0 + r < rows) y[row0 + r] = v * gs;
+    }
+}
+#define CROW_VALU_ENTRY(NAME, RG)                                                                                                          \
+    extern "C" __global__ void __launch_bounds__(256) NAME(const unsigned char* __restrict__ w, const float* __restrict__ x,              \
+                                                           const float* __restrict__ gs_ptr, float* __restrict__ y,                       \
+                                                           const int* __restrict__ k_dim_p, const int* __restrict__ rows_p) {             \
+        const int k = *k_dim_p;                                                                                                            \
+        if (block_threads() != 256 || k <= 0 || k % CROW_BLOCK_VALUES != 0) {                                                              \
+            if (threadIdx.x == 0) atomicOr(g_ws.status, STATUS_BAD_SHAPE);                                                                 \
+            return;                                                                                                                        \
+        }                                                                                                                                  \
+        gemv_valu_body<RG>(w, x, gs_ptr, y, k, *rows_p);                                                                                   \
+    }
+CROW_VALU_ENTRY(gemv_nvfp4_w_valu1, 1)
+CROW_VALU_ENTRY(gemv_nvfp4_w_valu2, 2)
+CROW_VALU_ENTRY(gemv_nvfp4_w_valu4, 4)

@@ -125,6 +125,14 @@ CROW_KERNEL(unpack_nvfp4, 4)        /* src(tiled), dst(container bytes), rows_p,
 CROW_KERNEL(dequant_nvfp4_tiled, 5) /* w, gs, out(f32 [rows][k_dim]), rows_p, k_dim_p: bit-exact decode (cnq.rs:1298-1308) */
 CROW_KERNEL(dequant_fp4_flat, 4)    /* w(raw container bytes), gs, out, n_p.  dequant_fp4_flat of kernels.rs:1460, same list */
 
+/* ---- measurement only (not part of the drop-in set: the engine never asks for these) --------------------------------- */
+/* w(raw container bytes), x, gs, y, k_dim_p, rows_p.  The one-row GEMV written the reference's way (kernels_p2.rs:304-368: lanes
+ * across the columns, f32 multiply-adds on decoded weights, no matrix instructions), 1 / 2 / 4 rows per 16-lane group: the A/B
+ * behind the choice of the matrix cores for one activation row (bench.py reports it). */
+CROW_KERNEL(gemv_nvfp4_w_valu1, 6)
+CROW_KERNEL(gemv_nvfp4_w_valu2, 6)
+CROW_KERNEL(gemv_nvfp4_w_valu4, 6)
+
 #ifdef CROW_KERNEL_DEFAULTED_
 #undef CROW_KERNEL
 #undef CROW_KERNEL_DEFAULTED_

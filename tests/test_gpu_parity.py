@@ -244,6 +244,28 @@ def test_five_thousand_hand_overs_in_a_row_give_the_same_bits(eng):
     assert gamma_rows(got[3][:, :128], w, 0, 128, cols, gs, xb[3][1]) <= 1.0
 
 
+@pytest.mark.parametrize("name", ["gemv_nvfp4_w_valu1", "gemv_nvfp4_w_valu2", "gemv_nvfp4_w_valu4"])
+def test_the_measurement_only_gemv_without_matrix_instructions(eng, name):
+    """The A/B kernels (container layout, f32 multiply-adds): same product, within the same bounds."""
+    from crow_nest_amd.kernels import launch_dims, launch_v
+    p = eng.p
+    for rows, cols in [(37, 256), (130, 320), (1000, 5120), (64, 17408)]:
+        w = random_nvfp4(700 + rows, rows, cols, scale_lo=0, scale_hi=0x100, p7f=1 / 16)
+        w = w.copy().reshape(-1, 36)
+        w[:, :4][w[:, :4] == 0xFF] = 0x7F  # (the tiled path refuses 0xFF; keep the comparison on common ground)
+        w = w.reshape(-1)
+        gs = 7.0e-4
+        x = normal_f32(701, rows, cols)
+        wd, xd = _dev(w), _dev(x)
+        gsd = torch.tensor([gs], dtype=torch.float32, device="cuda")
+        y = torch.full((rows,), -7.0, dtype=torch.float32, device="cuda")
+        launch_v(eng.k.f(name), *launch_dims(name, rows, cols), [wd.data_ptr(), xd.data_ptr(), gsd.data_ptr(), y.data_ptr(), p.i32(cols), p.i32(rows)])
+        eng.check()
+        got = y.cpu().numpy()
+        assert rel_err(got, orc.gemv(w, rows, cols, gs, x)[0]) <= TOL, (rows, cols)
+        assert gamma_ratio(got, w, rows, cols, gs, x) <= 1.0, (rows, cols)
+
+
 def test_verify_rows_are_bit_identical_to_one_row_decode(eng):
     """kernels_p2.rs:391-396: row m of an M-row launch == a one-row launch on x row m."""
     rows, cols = 700, 5120
