@@ -306,7 +306,7 @@ def main() -> int:
         from crow_nest_amd.kernels import time_sequence
         status()
         others["config3_lm_head_151936x5120_argmax"] = entry(l3.us(iters=100), V * K // 64 * 36 + K * 4 + V * 4 + 4)
-        others["config3_lm_head_151936x5120_argmax"]["launches"] = 1
+        others["config3_lm_head_151936x5120_argmax"]["launches"] = "1 call of crow_hip_launch = the GEMV + a one-block finishing kernel"
         lp = Launch(eng, "gemv_nvfp4_w", V, K, 1, [[hd.data_ptr(), xk.data_ptr(), gs1.data_ptr(), ybuf.data_ptr(), p.i32(K), p.i32(V)] for hd in heads])
         others["config3_lm_head_151936x5120_logits_only"] = entry(lp.us(iters=100), V * K // 64 * 36 + K * 4 + V * 4)
         del heads

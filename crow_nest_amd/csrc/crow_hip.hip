@@ -71,11 +71,12 @@ struct State {
 // Scratch memory of crow_hip_launch_noalloc: part of the code object, so it exists on a device from the moment the library
 // is loaded there until the process ends, and no call ever allocates it.  Words [0, NOALLOC_PARTIAL_FLOATS) hold the partial
 // sums of split launches, then NOALLOC_COUNTER_SLOTS arrival counters, the status word (alone on 32 words), and the fused
-// head's key and counter words.
-const size_t HEAD_BYTES = (size_t)CROW_HEAD_WORDS * sizeof(unsigned long long);
+// head's keys (8 bytes per strip).
+const unsigned HEAD_WORDS = 65536;  // the allocated workspace: heads of up to 1,048,576 rows
+const unsigned NOALLOC_HEAD_WORDS = CROW_NOALLOC_MAX_HEAD_STRIPS;
 const unsigned NOALLOC_PARTIAL_FLOATS = CROW_NOALLOC_MAX_PARTIAL_FLOATS;  // 4 MiB of split-K partial sums
 const unsigned NOALLOC_COUNTER_SLOTS = CROW_NOALLOC_MAX_STRIPS;
-const unsigned NOALLOC_TAIL_WORDS = 32 + 2 * CROW_HEAD_WORDS;  // status line, then the head's 8-byte words
+const unsigned NOALLOC_TAIL_WORDS = 32 + 2 * NOALLOC_HEAD_WORDS;  // status line, then the head's 8-byte words
 const unsigned NOALLOC_WORDS = NOALLOC_PARTIAL_FLOATS + NOALLOC_COUNTER_SLOTS + NOALLOC_TAIL_WORDS;
 static __device__ __align__(256) unsigned scratch[NOALLOC_WORDS];
 static_assert(sizeof(unsigned) * NOALLOC_WORDS == CROW_NOALLOC_SCRATCH_BYTES, "the header states the array's size");
@@ -135,7 +136,15 @@ int launch_entry(const FnEntry* e, dim3 grid, dim3 block, const uint64_t* vals, 
         args[na++] = (void*)&geo;
     }
     if (e->takes_ws) args[na++] = (void*)&ws_arg;
-    const hipError_t rc = hipLaunchKernel(e->stub, grid, block, args, lds, s);
+    const bool head = e->stub == (const void*)&gemv_nvfp4_w_argmax;
+    // the fused head keeps one key per strip (the kernel checks again and reports through the status word)
+    if (head && grid.x > ws.head_words) return CROW_ERR_WORKSPACE;
+    hipError_t rc = hipLaunchKernel(e->stub, grid, block, args, lds, s);
+    if (rc == hipSuccess && head) {  // ... and its finishing kernel right behind it: the token out of the strips' keys
+        unsigned strips = grid.x;
+        void* fargs[3] = {(void*)&vals[6], (void*)&strips, (void*)&ws_arg};
+        rc = hipLaunchKernel((const void*)&argmax_finish, dim3(1), dim3(1024), fargs, 0, s);
+    }
     if (rc != hipSuccess) (void)hipGetLastError();  // reported here: not left behind for an unrelated later call to find
     return hip_rc(rc);
 }
@@ -171,8 +180,9 @@ int crow_hip_init(int device) {
     };
     if ((e = hipMalloc((void**)&ws.partials, PARTIAL_FLOATS * sizeof(float))) != hipSuccess) return fail(e);
     if ((e = hipMalloc((void**)&ws.counters, COUNTER_WORDS * sizeof(unsigned))) != hipSuccess) return fail(e);
-    if ((e = hipMalloc((void**)&ws.head, HEAD_BYTES)) != hipSuccess) return fail(e);
-    if ((e = hipMemset(ws.head, 0, HEAD_BYTES)) != hipSuccess) return fail(e);
+    if ((e = hipMalloc((void**)&ws.head, HEAD_WORDS * sizeof(unsigned long long))) != hipSuccess) return fail(e);
+    if ((e = hipMemset(ws.head, 0, HEAD_WORDS * sizeof(unsigned long long))) != hipSuccess) return fail(e);
+    ws.head_words = HEAD_WORDS;
     if ((e = hipMalloc((void**)&scalars, 16 * sizeof(int))) != hipSuccess) return fail(e);
     if ((e = hipMemset(ws.counters, 0, COUNTER_WORDS * sizeof(unsigned))) != hipSuccess) return fail(e);
     ws.status = ws.counters + COUNTER_SLOTS;
@@ -199,7 +209,8 @@ int crow_hip_init(int device) {
     st.counters = sp + NOALLOC_PARTIAL_FLOATS;
     st.counter_slots = NOALLOC_COUNTER_SLOTS;
     st.status = st.counters + NOALLOC_COUNTER_SLOTS;
-    st.head = (unsigned long long*)(st.status + 32);  // on a 128-byte line of its own
+    st.head = (unsigned long long*)(st.status + 32);
+    st.head_words = NOALLOC_HEAD_WORDS;
     // counters, status and key start at zero (a process that shut the library down and initialises it again included)
     if ((e = hipMemset(st.counters, 0, (NOALLOC_COUNTER_SLOTS + NOALLOC_TAIL_WORDS) * sizeof(unsigned))) != hipSuccess) return fail(e);
     if ((e = hipDeviceSynchronize()) != hipSuccess) return fail(e);
@@ -366,8 +377,8 @@ int crow_hip_launch_dims_split(const char* name, uint32_t rows, uint32_t k_dim, 
             return CROW_OK;
         }
         if (verify && z > 4) return CROW_ERR_SHAPE;
-        // the fused head counts at most 127 blocks into each of its scratch words
-        if (strcmp(name, "gemv_nvfp4_w_argmax") == 0 && strips > (uint32_t)CROW_HEAD_MAX_STRIPS) return CROW_ERR_SHAPE;
+        // the fused head keeps one key per strip in the workspace
+        if (strcmp(name, "gemv_nvfp4_w_argmax") == 0 && strips > HEAD_WORDS) return CROW_ERR_SHAPE;
         const uint32_t wmax = (uint32_t)e->max_waves / (uint32_t)e->nr;  // waves per tensor in a block
         // A wave walks its run of groups with four of them (9 KB) in flight; few long walks beat many short ones (every wave
         // pays its start, its staging set-up and the block's meeting in LDS once), as long as the launch still has a few
@@ -455,7 +466,6 @@ int crow_hip_status(void) {
         (void)hipMemset(g.ws.status, 0, sizeof st);
         // a launch that bailed out may have left arrival counters behind
         (void)hipMemset(g.ws.counters, 0, COUNTER_WORDS * sizeof(unsigned));
-        (void)hipMemset(g.ws.head, 0, HEAD_BYTES);  // ... or a head's candidates and counters
     }
     if (st2 != 0) (void)hipMemset(g.ws_static.counters, 0, (NOALLOC_COUNTER_SLOTS + NOALLOC_TAIL_WORDS) * sizeof(unsigned));  // counters, status, key
     st |= st2;
@@ -469,9 +479,7 @@ int crow_hip_reset_workspace(void) {
     if (!g.ready) return CROW_ERR_NOT_INITIALIZED;
     hipError_t e = hipDeviceSynchronize();
     if (e != hipSuccess) return (int)e;
-    if ((e = hipMemset(g.ws.head, 0, HEAD_BYTES)) != hipSuccess) return (int)e;
     if ((e = hipMemset(g.ws_static.counters, 0, NOALLOC_COUNTER_SLOTS * sizeof(unsigned))) != hipSuccess) return (int)e;
-    if ((e = hipMemset(g.ws_static.head, 0, HEAD_BYTES)) != hipSuccess) return (int)e;
     return hip_rc(hipMemset(g.ws.counters, 0, COUNTER_WORDS * sizeof(unsigned)));
 }
 

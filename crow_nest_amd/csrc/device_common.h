@@ -40,23 +40,17 @@ __device__ __forceinline__ unsigned stream_load_u32(const unsigned* p) {
 
 // Library-owned scratch for kernels that split one output tile over several workgroups:
 // per-slice partial sums and one arrival counter per output tile.  Set once by crow_hip_init.
-// Scratch of the fused head (gemv_nvfp4_w_argmax): CROW_HEAD_SLOTS 64-bit words, each on a 128-byte line of its own (so that
-// the atomics of thousands of blocks spread over the L2 channels), all zero between launches.  Block b folds its candidate
-// into word b % CROW_HEAD_SLOTS with ONE compare-and-swap that also counts it: bits 63..7 = the best key so far (best_key),
-// bits 6..0 = blocks arrived.  Because key and count change together, a block that reads every word complete has read every
-// word's final key.  At most 127 blocks per word: 32,512 strips, 520,192 rows.
-#define CROW_HEAD_SLOTS 256
-#define CROW_HEAD_COUNT_BITS 7
-#define CROW_HEAD_MAX_STRIPS (127 * CROW_HEAD_SLOTS)
-#define CROW_HEAD_WORDS (16 * CROW_HEAD_SLOTS)
-
+// Scratch of the fused head (gemv_nvfp4_w_argmax): one 64-bit key per 16-row strip.  Every block stores the best_key of its
+// strip (a plain store: nobody reads it inside the launch), and the one-block kernel that the launcher starts right behind
+// it (argmax_finish) takes the maximum.  Every launch overwrites the words it reads, so nothing is ever cleared.
 struct Workspace {
     float* partials;
     unsigned* counters;
     unsigned long long partial_floats;  // capacity of `partials`
     unsigned counter_slots;             // capacity of `counters`
     unsigned* status;                   // device word: non-zero = a launch did not fit the workspace
-    unsigned long long* head;           // fused lm_head argmax: CROW_HEAD_WORDS 8-byte words, all zero between launches (layout below)
+    unsigned long long* head;           // fused lm_head argmax: one key per strip
+    unsigned head_words;                // how many strips the head's scratch takes
 };
 __device__ Workspace g_ws;
 

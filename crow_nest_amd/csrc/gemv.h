@@ -711,62 +711,20 @@ __device__ __forceinline__ void gemv_body(const GemvArgs& a, unsigned z, lds_p l
     const int rows = *a.rows_p;
     // the launch geometry was made for another problem, or the two tensors cannot share the block's waves evenly: nothing is stored
     if (*a.k_dim_p != k_dim || (a.count_p != nullptr && *a.count_p != a.count_expect) || (NR == 2 && (waves & 1)) ||
-        (EPI == EPI_SCALE && a.argmax_out != nullptr && strips > CROW_HEAD_MAX_STRIPS)) {
+        (EPI == EPI_SCALE && a.argmax_out != nullptr && (unsigned)strips > ws.head_words)) {
         if (lane == 0) atomicOr(ws.status, STATUS_BAD_SHAPE);
         return;
     }
     if constexpr (NS == 1 && EPI == EPI_SCALE) {
         const int row = strip * CROW_STRIP_ROWS + n;
         if (a.argmax_out != nullptr) {
-            // fused head: logits out, and the greedy token of the whole launch from its last block (device_common.h: the head's
-            // scratch).  Same total order as argmax_k, whatever order the blocks finish in.
-            typedef __attribute__((address_space(1))) unsigned long long* gk_p;
+            // fused head: logits out, and this strip's best (value, index) as one ordered key for the finishing kernel that the
+            // launcher starts behind this one (misc_kernels.h: argmax_finish).  Same total order as argmax_k.
             const float val = v[0] * a.gs[0][0];
             const bool live = mo == 0 && row < rows;
             if (live) a.y[row] = val;
             const Best b = wave_best(Best{live ? val : -3.0e38f, live ? row : 0});
-            gk_p words = (gk_p)ws.head;
-            const unsigned slot = (unsigned)strip % CROW_HEAD_SLOTS, n_strips = (unsigned)strips;
-            constexpr unsigned long long COUNT = (1ull << CROW_HEAD_COUNT_BITS) - 1;
-            unsigned last = 0;
-            if (lane == 0) {
-                // candidate in and block counted in one step; a failed swap means another block of the slot got in, so at most
-                // (blocks of the slot - 1) retries
-                const unsigned in_slot = (n_strips - slot + CROW_HEAD_SLOTS - 1) / CROW_HEAD_SLOTS;
-                const unsigned long long mine = best_key(b.v, b.i);
-                unsigned long long w = __hip_atomic_load(words + 16 * slot, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT), nw;
-                do {
-                    const unsigned long long cur = w >> CROW_HEAD_COUNT_BITS;
-                    nw = ((cur > mine ? cur : mine) << CROW_HEAD_COUNT_BITS) | ((w & COUNT) + 1);
-                } while (!__hip_atomic_compare_exchange_strong(words + 16 * slot, &w, nw, __ATOMIC_RELAXED, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT));
-                last = (nw & COUNT) == in_slot ? 1u : 0u;
-            }
-            if (__builtin_amdgcn_readfirstlane(last) == 0) return;
-            // This block completed its slot.  If it now reads every slot complete it has every slot's final key: it writes the
-            // token and zeroes the words.  (The block that completed the last slot always does; should another one read all
-            // slots complete as well, it computes the same token; one that reads a word already zeroed stands back.)
-            device_order();
-            unsigned long long best = 0;
-            bool complete = true;
-#pragma unroll
-            for (int j = 0; j < CROW_HEAD_SLOTS / 64; j++) {
-                const unsigned s = (unsigned)lane + 64u * j;
-                if (s < n_strips) {
-                    const unsigned long long w = __hip_atomic_load(words + 16 * s, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-                    complete = complete && (w & COUNT) == (n_strips - s + CROW_HEAD_SLOTS - 1) / CROW_HEAD_SLOTS;
-                    best = (w >> CROW_HEAD_COUNT_BITS) > best ? (w >> CROW_HEAD_COUNT_BITS) : best;
-                }
-            }
-            if (__builtin_amdgcn_ballot_w64(!complete) != 0ull) return;
-#pragma unroll
-            for (int j = 0; j < CROW_HEAD_SLOTS / 64; j++)
-                if ((unsigned)lane + 64u * j < n_strips)
-                    __hip_atomic_store(words + 16 * (lane + 64 * j), 0ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-            for (int o = 32; o > 0; o >>= 1) {
-                const unsigned long long other = ((unsigned long long)__shfl_xor((unsigned)(best >> 32), o) << 32) | __shfl_xor((unsigned)best, o);
-                best = other > best ? other : best;
-            }
-            if (lane == 0) a.argmax_out[0] = best != 0ull ? best_key_index(best) : 0;
+            if (lane == 0) ws.head[strip] = best_key(b.v, b.i);
             return;
         }
     }

@@ -72,10 +72,10 @@ extern "C" __global__ void CROW_ONE_ROW_F32 __launch_bounds__(1024) gemv_fp4(con
     gemv_body<1, 1, false, EPI_SCALE>(a, 0, LDS, ws);
 }
 
-// lm_head with the greedy argmax fused in: logits[rows] and out_idx[0] = the greedy token, in ONE launch.  Every block folds
-// the best of its 16-row strip into the head's scratch words; the block that finishes last picks the winner, writes it and
-// leaves the scratch zeroed for the next head (gemv.h).  Replaces lm_head_row + argmax_k (engine/src/gen.rs:4766-4784,
-// engine/src/kernels.rs:4238-4260), which re-read all logits in a second launch; same tie rule.
+// lm_head with the greedy argmax fused in: logits[rows] and out_idx[0] = the greedy token from ONE call of the launcher.  Every
+// block leaves the best of its 16-row strip as an ordered key in the head's scratch; the launcher starts argmax_finish (one
+// block, misc_kernels.h) right behind this kernel, which takes the maximum of ceil(rows / 16) keys instead of re-reading all
+// logits.  Replaces lm_head_row + argmax_k (engine/src/gen.rs:4766-4784, engine/src/kernels.rs:4238-4260); same tie rule.
 extern "C" __global__ void CROW_ONE_ROW_F32 __launch_bounds__(1024) gemv_nvfp4_w_argmax(const unsigned char* __restrict__ w, const float* __restrict__ x,
                                                                        const float* __restrict__ gs_ptr, float* __restrict__ y,
                                                                        const int* __restrict__ k_dim_p, const int* __restrict__ rows_p,

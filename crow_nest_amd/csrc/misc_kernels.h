@@ -467,6 +467,34 @@ extern "C" __global__ void __launch_bounds__(1024) argmax_k(const float* __restr
     }
 }
 
+// The fused head's second kernel, started by the launcher right behind gemv_nvfp4_w_argmax (callers launch ONE kernel): the
+// maximum of the `strips` keys the GEMV's blocks left in the head's scratch, decoded into the greedy token.  One block of 1024
+// threads, every thread's loads in flight at once; the order is a total order on keys, so the reduction shape is free.
+extern "C" __global__ void __launch_bounds__(1024) argmax_finish(int* __restrict__ out, unsigned strips, const Workspace ws) {
+    __shared__ unsigned long long wave_max[16];
+    const int lane = lane_id(), wave = (int)(threadIdx.x >> 6);
+    unsigned long long best = 0;
+    for (unsigned base = threadIdx.x; base < strips; base += 16 * 1024) {  // sixteen loads in flight per thread: one round trip
+        unsigned long long k[16];
+#pragma unroll
+        for (int j = 0; j < 16; j++) {
+            const unsigned i = base + 1024u * j;
+            k[j] = ws.head[i < strips ? i : base];
+        }
+#pragma unroll
+        for (int j = 0; j < 16; j++) best = k[j] > best ? k[j] : best;
+    }
+    for (int o = 32; o > 0; o >>= 1) {
+        const unsigned long long other = ((unsigned long long)__shfl_xor((unsigned)(best >> 32), o) << 32) | __shfl_xor((unsigned)best, o);
+        best = other > best ? other : best;
+    }
+    if (lane == 0) wave_max[wave] = best;
+    __syncthreads();
+    if (threadIdx.x != 0) return;
+    for (int w = 1; w < 16; w++) best = wave_max[w] > best ? wave_max[w] : best;
+    out[0] = best != 0ull ? best_key_index(best) : 0;
+}
+
 // ------------------------------------------------------------------ BF16 and F32 keeps
 // The tensors the container keeps unquantised (router, q/k, MTP head): y[t][row] = sum_k w[row][k] * x[t][k], f32
 // activations, f32 accumulation.  16-byte non-temporal weight loads (8 bf16 or 4 f32 per lane per step: 1024 contiguous

@@ -119,7 +119,7 @@ class Engine:
 
     # ------------------------------------------------------------------ head
     def lm_head_row(self, w: Fp4, x: torch.Tensor, fused: bool = True):
-        """logits[V] and the greedy token.  fused: one launch writes both (the last block to finish picks the token);
+        """logits[V] and the greedy token.  fused: one call writes both (the library runs a one-block finishing kernel behind the GEMV);
         else gemv_nvfp4_w + argmax_k over all logits, as the reference."""
         rows, k = w.rows, w.cols
         logits = torch.empty(rows, dtype=torch.float32, device=self.dev)

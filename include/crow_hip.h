@@ -78,16 +78,18 @@ int crow_hip_launch(crow_fn_t f, uint32_t gx, uint32_t gy, uint32_t gz, uint32_t
 /* crow_hip_launch for callers that cannot allocate device memory (code under HIP graph capture, tight serving loops,
  * harnesses that forbid hipMalloc).  It has no counterpart in the reference.  Same arguments and results as crow_hip_launch,
  * for the kernels that use scratch memory (the NVFP4 GEMV family; any other kernel: CROW_ERR_BAD_ARGUMENT),
- * but their scratch - split-K partial sums, arrival counters, the status word, the fused head's keys and counters - is a fixed array
+ * but their scratch - split-K partial sums, arrival counters, the status word, the fused head's keys - is a fixed array
  * inside the library's code object (CROW_NOALLOC_SCRATCH_BYTES per device, held until the process ends) instead of the
  * workspace crow_hip_init allocates; the call itself allocates and frees nothing.  A split launch (column slices S > 1 in
  * `gy`) with more than CROW_NOALLOC_MAX_PARTIAL_FLOATS partial sums (gx * gz * S * tensors * 64) or more than
- * CROW_NOALLOC_MAX_STRIPS strips (gx * gz) is refused with CROW_ERR_WORKSPACE before anything runs.  Every call on a device
+ * CROW_NOALLOC_MAX_STRIPS strips (gx * gz), and a fused head (gemv_nvfp4_w_argmax) of more than CROW_NOALLOC_MAX_HEAD_STRIPS
+ * strips, is refused with CROW_ERR_WORKSPACE before anything runs.  Every call on a device
  * shares the one array: calls that overlap on the device (two streams, two threads) race; order them on one stream.  crow_hip_status
  * reports both scratch areas. */
 #define CROW_NOALLOC_MAX_PARTIAL_FLOATS (1u << 20)
 #define CROW_NOALLOC_MAX_STRIPS 4096u
-#define CROW_NOALLOC_SCRATCH_BYTES (4u * (CROW_NOALLOC_MAX_PARTIAL_FLOATS + CROW_NOALLOC_MAX_STRIPS + 32u + 8192u))
+#define CROW_NOALLOC_MAX_HEAD_STRIPS 16384u /* the fused head through this entry point: at most 262,144 rows */
+#define CROW_NOALLOC_SCRATCH_BYTES (4u * (CROW_NOALLOC_MAX_PARTIAL_FLOATS + CROW_NOALLOC_MAX_STRIPS + 32u + 2u * CROW_NOALLOC_MAX_HEAD_STRIPS))
 int crow_hip_launch_noalloc(crow_fn_t f, uint32_t gx, uint32_t gy, uint32_t gz, uint32_t bx, const uint64_t* vals,
                             uint32_t n_vals, void* stream);
 /* grid/block for `name` on a [rows, k_dim] tensor with `z` token rows (batched and verify kernels: the value *t_p / *m_p

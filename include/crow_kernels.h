@@ -32,8 +32,9 @@ CROW_KERNEL(gemv_nvfp4_w_bf16, 6) /* the same on bf16 x */
  * engine still calls for some tensors); same arithmetic as gemv_nvfp4_w here. */
 CROW_KERNEL(gemv_fp4, 6)
 /* w, x, gs, y(logits), k_dim_p, rows_p, out_idx.  lm_head_row (engine/src/gen.rs:4766-4784) and argmax_k
- * (engine/src/kernels.rs:4238-4260) in one launch: logits[rows] and out_idx[0] = the greedy token, same tie order as
- * argmax_k.  The blocks' candidates meet in the library's scratch memory; the last block to finish writes the token. */
+ * (engine/src/kernels.rs:4238-4260) in one call: logits[rows] and out_idx[0] = the greedy token, same tie order as
+ * argmax_k.  Each block leaves its strip's candidate in the library's scratch memory; crow_hip_launch starts a one-block
+ * finishing kernel right behind the GEMV (on the same stream, also under capture) that writes the token. */
 CROW_KERNEL(gemv_nvfp4_w_argmax, 7)
 CROW_KERNEL(argmax_k, 3)     /* logits, out_idx, n_p.  engine/src/kernels.rs:4238-4260 */
 

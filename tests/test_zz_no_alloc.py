@@ -1,7 +1,7 @@
 """crow_hip_launch_noalloc (scratch memory in a fixed array inside the library, nothing allocated per call) against
 crow_hip_launch (scratch memory from the workspace crow_hip_init allocated): same kernels, same launch dimensions, so the
-same bits.  Two calls in a row share the one array, the second with a smaller input; then the fused head, whose key and counter
-words live in the same array; then the size limit."""
+same bits.  Two calls in a row share the one array, the second with a smaller input; then the fused head, whose keys
+live in the same array; then the size limit."""
 import numpy as np
 import pytest
 import torch
@@ -82,7 +82,7 @@ def test_fused_head_keeps_its_keys_in_the_static_scratch(eng):
     from crow_nest_amd.kernels import launch_dims, launch_noalloc, launch_v
     p = eng.p
     toks = []
-    # twice in a row: the second head (fewer rows) must find the key and counter words cleared by the first one's last block
+    # twice in a row: the second head (fewer rows) must not see the first one's keys
     for seed, rows, cols in [(31, 4000, 1024), (32, 1000, 512)]:
         w = random_nvfp4(seed, rows, cols)
         gs = 5.0e-4
