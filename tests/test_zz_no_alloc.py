@@ -123,6 +123,12 @@ def test_sizes_beyond_the_static_scratch_and_other_kernels_are_refused(eng):
     with pytest.raises(CrowHipError) as ei:
         launch_noalloc(eng.k.f("gemv_nvfp4_w"), *dims, [dummy.data_ptr()] * 4 + [p.i32(cols), p.i32(rows)])
     assert ei.value.code == -5
+    # a fused head of more strips than the static scratch holds keys for (the allocated workspace takes four times as many)
+    rows = (16384 + 1) * 16
+    dims = launch_dims("gemv_nvfp4_w_argmax", rows, 64)
+    with pytest.raises(CrowHipError) as ei:
+        launch_noalloc(eng.k.f("gemv_nvfp4_w_argmax"), *dims, [dummy.data_ptr()] * 4 + [p.i32(64), p.i32(rows), dummy.data_ptr()])
+    assert ei.value.code == -5
     with pytest.raises(CrowHipError) as ei:  # a kernel that takes no scratch descriptor
         launch_noalloc(eng.k.f("argmax_k"), 1, 1, 1, 1024, [dummy.data_ptr(), dummy.data_ptr(), p.i32(16)])
     assert ei.value.code == -3
