@@ -37,15 +37,10 @@ __device__ __forceinline__ void crow_need_now(T v, R... rest) {
     crow_need_now(rest...);
 }
 #define ENTER(...) crow_need_now(ws.status, block_threads(), (int)gridDim.y, __VA_ARGS__)
-// One-row kernels are compiled for at least this many resident waves per SIMD (it bounds their registers): six on bf16
-// activations, five on f32 ones (whose sixteen registers of activations in flight do not fit the tighter bound).  Blocks are
-// five waves per tensor at K = 5120, so five and six waves per SIMD hold the same four blocks per compute unit.
-#define CROW_ONE_ROW_BF16
-#define CROW_ONE_ROW_F32
 
 // ------------------------------------------------------------------ dense GEMV (decode, one row)
 // reference: gemv_nvfp4_w, engine/src/kernels_p2.rs:355-368
-extern "C" __global__ void CROW_ONE_ROW_F32 __launch_bounds__(1024) gemv_nvfp4_w(const unsigned char* __restrict__ w, const float* __restrict__ x,
+extern "C" __global__ void __launch_bounds__(1024) gemv_nvfp4_w(const unsigned char* __restrict__ w, const float* __restrict__ x,
                                                                 const float* __restrict__ gs_ptr, float* __restrict__ y,
                                                                 const int* __restrict__ k_dim_p, const int* __restrict__ rows_p, int geo, const Workspace ws) {
     ENTER(w, x, gs_ptr, y, k_dim_p, rows_p, geo);
@@ -54,7 +49,7 @@ extern "C" __global__ void CROW_ONE_ROW_F32 __launch_bounds__(1024) gemv_nvfp4_w
     gemv_body<1, 1, false, EPI_SCALE>(a, 0, LDS, ws);
 }
 // the same product on bf16 activations (exact widening), for models that keep their activations in bf16
-extern "C" __global__ void CROW_ONE_ROW_BF16 __launch_bounds__(1024) gemv_nvfp4_w_bf16(const unsigned char* __restrict__ w, const unsigned short* __restrict__ x,
+extern "C" __global__ void __launch_bounds__(1024) gemv_nvfp4_w_bf16(const unsigned char* __restrict__ w, const unsigned short* __restrict__ x,
                                                                      const float* __restrict__ gs_ptr, float* __restrict__ y,
                                                                      const int* __restrict__ k_dim_p, const int* __restrict__ rows_p, int geo, const Workspace ws) {
     ENTER(w, x, gs_ptr, y, k_dim_p, rows_p, geo);
@@ -63,7 +58,7 @@ extern "C" __global__ void CROW_ONE_ROW_BF16 __launch_bounds__(1024) gemv_nvfp4_
     gemv_body<1, 1, true, EPI_SCALE>(a, 0, LDS, ws);
 }
 // reference: gemv_fp4, engine/src/kernels.rs:118-151 (+ rows_p: the reference's grid.x is the row count)
-extern "C" __global__ void CROW_ONE_ROW_F32 __launch_bounds__(1024) gemv_fp4(const unsigned char* __restrict__ w, const float* __restrict__ x,
+extern "C" __global__ void __launch_bounds__(1024) gemv_fp4(const unsigned char* __restrict__ w, const float* __restrict__ x,
                                                             const float* __restrict__ gs_ptr, float* __restrict__ y,
                                                             const int* __restrict__ k_dim_p, const int* __restrict__ rows_p, int geo, const Workspace ws) {
     ENTER(w, x, gs_ptr, y, k_dim_p, rows_p, geo);
@@ -76,7 +71,7 @@ extern "C" __global__ void CROW_ONE_ROW_F32 __launch_bounds__(1024) gemv_fp4(con
 // block leaves the best of its 16-row strip as an ordered key in the head's scratch; the launcher starts argmax_finish (one
 // block, misc_kernels.h) right behind this kernel, which takes the maximum of ceil(rows / 16) keys instead of re-reading all
 // logits.  Replaces lm_head_row + argmax_k (engine/src/gen.rs:4766-4784, engine/src/kernels.rs:4238-4260); same tie rule.
-extern "C" __global__ void CROW_ONE_ROW_F32 __launch_bounds__(1024) gemv_nvfp4_w_argmax(const unsigned char* __restrict__ w, const float* __restrict__ x,
+extern "C" __global__ void __launch_bounds__(1024) gemv_nvfp4_w_argmax(const unsigned char* __restrict__ w, const float* __restrict__ x,
                                                                        const float* __restrict__ gs_ptr, float* __restrict__ y,
                                                                        const int* __restrict__ k_dim_p, const int* __restrict__ rows_p,
                                                                        int* __restrict__ out_idx, int geo, const Workspace ws) {
@@ -89,7 +84,7 @@ extern "C" __global__ void CROW_ONE_ROW_F32 __launch_bounds__(1024) gemv_nvfp4_w
 
 // ------------------------------------------------------------------ fused gate/up + SiLU (decode)
 // reference: gemv_nvfp4_gu, engine/src/kernels_p2.rs:372-389
-extern "C" __global__ void CROW_ONE_ROW_F32 __launch_bounds__(1024) gemv_nvfp4_gu(const unsigned char* __restrict__ wg, const unsigned char* __restrict__ wu,
+extern "C" __global__ void __launch_bounds__(1024) gemv_nvfp4_gu(const unsigned char* __restrict__ wg, const unsigned char* __restrict__ wu,
                                                                  const float* __restrict__ x, const float* __restrict__ gs_g,
                                                                  const float* __restrict__ gs_u, float* __restrict__ y,
                                                                  const int* __restrict__ k_dim_p, const int* __restrict__ rows_p, int geo, const Workspace ws) {
@@ -100,7 +95,7 @@ extern "C" __global__ void CROW_ONE_ROW_F32 __launch_bounds__(1024) gemv_nvfp4_g
 }
 
 // the same on bf16 activations (exact widening)
-extern "C" __global__ void CROW_ONE_ROW_BF16 __launch_bounds__(1024) gemv_nvfp4_gu_bf16(const unsigned char* __restrict__ wg, const unsigned char* __restrict__ wu,
+extern "C" __global__ void __launch_bounds__(1024) gemv_nvfp4_gu_bf16(const unsigned char* __restrict__ wg, const unsigned char* __restrict__ wu,
                                                                       const unsigned short* __restrict__ x, const float* __restrict__ gs_g,
                                                                       const float* __restrict__ gs_u, float* __restrict__ y,
                                                                       const int* __restrict__ k_dim_p, const int* __restrict__ rows_p, int geo, const Workspace ws) {
@@ -244,7 +239,7 @@ extern "C" __global__ void __launch_bounds__(512) gemv_fp4_bs(const unsigned cha
     }
 // reference: gemv_fp4_ptrb, engine/src/kernels.rs:195-233.  grid.z = combo; ptrs[combo] is the
 // device address of that combo's expert matrix in the tiled layout; x row = combo / x_div.
-extern "C" __global__ void CROW_ONE_ROW_F32 __launch_bounds__(1024) gemv_fp4_ptrb(const unsigned long long* __restrict__ ptrs, const float* __restrict__ x,
+extern "C" __global__ void __launch_bounds__(1024) gemv_fp4_ptrb(const unsigned long long* __restrict__ ptrs, const float* __restrict__ x,
                                                                  const float* __restrict__ gs_ptr, float* __restrict__ y,
                                                                  const int* __restrict__ k_dim_p, const int* __restrict__ x_div_p,
                                                                  const int* __restrict__ x_stride_p, const int* __restrict__ rows_p, int geo, const Workspace ws) {
@@ -264,7 +259,7 @@ extern "C" __global__ void CROW_ONE_ROW_F32 __launch_bounds__(1024) gemv_fp4_ptr
 __device__ __forceinline__ size_t up_offset(int inter, int pairs) {
     return (size_t)(inter / CROW_STRIP_ROWS) * ((pairs + CROW_GROUP_PAIRS - 1) / CROW_GROUP_PAIRS) * CROW_GROUP_BYTES;
 }
-extern "C" __global__ void CROW_ONE_ROW_F32 __launch_bounds__(1024) moe_gate_up_silu(const unsigned long long* __restrict__ ptrs, const float* __restrict__ x,
+extern "C" __global__ void __launch_bounds__(1024) moe_gate_up_silu(const unsigned long long* __restrict__ ptrs, const float* __restrict__ x,
                                                                     const float* __restrict__ gs_ptr, float* __restrict__ h,
                                                                     const int* __restrict__ k_dim_p, const int* __restrict__ x_div_p,
                                                                     const int* __restrict__ x_stride_p, const int* __restrict__ inter_p, int geo, const Workspace ws) {

@@ -284,7 +284,7 @@ extern "C" __global__ void __launch_bounds__(64) router_top10(const float* __res
 // logits row is 1 KB) instead of reading pointers a router launch left behind, which takes a launch (4 us back to back) off
 // the layer.  grid (inter / 16, 1, T K), block as moe_gate_up_silu.  Block (strip 0, pick 0) of each token writes
 // ids, wts and dn_ptrs for moe_down_combine.  table[2 e] / table[2 e + 1] = gate|up / down slab of expert e.
-extern "C" __global__ void CROW_ONE_ROW_F32 __launch_bounds__(1024) moe_route_gate_up_silu(const float* __restrict__ logits, const unsigned long long* __restrict__ table,
+extern "C" __global__ void __launch_bounds__(1024) moe_route_gate_up_silu(const float* __restrict__ logits, const unsigned long long* __restrict__ table,
                                                                           const float* __restrict__ x, const float* __restrict__ gs_ptr,
                                                                           float* __restrict__ h, int* __restrict__ ids, float* __restrict__ wts,
                                                                           unsigned long long* __restrict__ dn_ptrs, const int* __restrict__ k_dim_p,
