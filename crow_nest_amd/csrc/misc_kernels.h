@@ -299,10 +299,29 @@ extern "C" __global__ void __launch_bounds__(1024) moe_route_gate_up_silu(const 
     }
     const int combo = (int)blockIdx.z, t = combo / K, j = combo % K;
     if (threadIdx.x < 64) {  // wave 0
+        // Up to 256 experts the whole pointer table (16 bytes per expert) is requested together with the logits, four entries
+        // per lane, and the picked expert's entry is taken from registers: read after the routing it would be one more
+        // dependent round trip between the logits and the block's first weight load.
+        const int lane = (int)threadIdx.x;
+        u32x4 entry[4];
+        if (E <= 256) {
+#pragma unroll
+            for (int q = 0; q < 4; q++) {
+                const int i = lane + 64 * q;
+                entry[q] = *(const __attribute__((address_space(1))) u32x4*)((const unsigned char*)table + 16 * (size_t)(i < E ? i : 0));
+            }
+        }
         int picked;
         router_dispatch(E, logits, nullptr, ids, wts, nullptr, dn_ptrs, table, nullptr, nullptr, nullptr, K, t, blockIdx.x == 0 && j == 0, picked);
         const int e = __builtin_amdgcn_readlane(picked, j);
-        if (threadIdx.x == 0) s_slab = table[2 * e];
+        if (E <= 256) {
+            const int q = e >> 6;  // uniform
+            const u32x4 mine = q == 0 ? entry[0] : (q == 1 ? entry[1] : (q == 2 ? entry[2] : entry[3]));
+            const unsigned lo = (unsigned)__builtin_amdgcn_readlane((int)mine.x, e & 63), hi = (unsigned)__builtin_amdgcn_readlane((int)mine.y, e & 63);
+            if (threadIdx.x == 0) s_slab = ((unsigned long long)hi << 32) | lo;
+        } else if (threadIdx.x == 0) {
+            s_slab = table[2 * e];
+        }
     }
     __syncthreads();
     const int inter = *inter_p;
