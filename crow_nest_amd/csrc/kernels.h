@@ -300,6 +300,15 @@ extern "C" __global__ void __launch_bounds__(1024) moe_down_combine(const unsign
     // activations were
     lds_p zero = LDS, areas = LDS + CROW_GEMV_ZERO_BYTES;
     const unsigned char* w = (const unsigned char*)ptrs[combo];
+    // everything the epilogue needs is requested in the same round trip as the slab pointer: at one wave per SIMD nothing
+    // hides a dependent load between the last product and the store (the row count, the caller's K, the routing weight, the
+    // scale, and the old value of y that the result is added to)
+    const int rows = *rows_p, k_word = *k_dim_p;
+    const float gs = gs_ptr[0], weight = rw[combo];
+    const int row = strip * CROW_STRIP_ROWS + lane;
+    const bool writer = j == 0 && lane < 16 && row < rows;
+    float y_old = 0.0f;
+    if (writer) y_old = y[(size_t)t * rows + row];
     const size_t xoff[1] = {0};
     StripWalk<1, false> walk;
     // a routing launch that refused its geometry left zeros behind: no weights to read; the wave still joins the barriers below
@@ -312,17 +321,16 @@ extern "C" __global__ void __launch_bounds__(1024) moe_down_combine(const unsign
     float acc[1];
     walk.finish(acc);
     if (w == nullptr && lane == 0) atomicOr(ws.status, STATUS_BAD_GEO);
-    if (lane < 16) ((lds_f)(areas + j * AREA))[lane] = rw[combo] * (acc[0] * gs_ptr[0]);
+    if (lane < 16) ((lds_f)(areas + j * AREA))[lane] = weight * (acc[0] * gs);
     __syncthreads();
-    const int rows = *rows_p, row = strip * CROW_STRIP_ROWS + lane;
-    if (j != 0 || lane >= 16 || row >= rows) return;
-    if (*k_dim_p != k) {
+    if (!writer) return;
+    if (k_word != k) {
         if (lane == 0) atomicOr(ws.status, STATUS_BAD_SHAPE);
         return;
     }
     float sum = 0.0f;
     for (int q = 0; q < topk; q++) sum = __fadd_rn(sum, ((lds_f)(areas + q * AREA))[lane]);
-    y[(size_t)t * rows + row] += sum;
+    y[(size_t)t * rows + row] = y_old + sum;
 }
 
 // ------------------------------------------------------------------ routed experts, grouped by expert (batches of many tokens)
