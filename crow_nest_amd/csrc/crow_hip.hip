@@ -49,6 +49,10 @@ const FnEntry g_table[] = {
     {"gemm_nvfp4_bf16_m64", (const void*)&gemm_nvfp4_bf16_m64, 7, 2u * 64u * 528u, 0, 16, 0, 1, false},
     {"gemm_nvfp4_bf16_m48", (const void*)&gemm_nvfp4_bf16_m48, 7, 2u * 48u * 528u, 0, 16, 0, 1, false},
     {"gemm_nvfp4_bf16_m96", (const void*)&gemm_nvfp4_bf16_m96, 7, 2u * 96u * 528u, 0, 16, 0, 1, false},
+    {"gemm_nvfp4_bf16_w48", (const void*)&gemm_nvfp4_bf16_w48, 7, 2u * 48u * 528u, 0, 8, 0, 1, false},
+    {"gemm_nvfp4_bf16_w64", (const void*)&gemm_nvfp4_bf16_w64, 7, 2u * 64u * 528u, 0, 8, 0, 1, false},
+    {"gemm_nvfp4_bf16_w80", (const void*)&gemm_nvfp4_bf16_w80, 7, 2u * 80u * 528u, 0, 8, 0, 1, false},
+    {"gemm_nvfp4_bf16_w96", (const void*)&gemm_nvfp4_bf16_w96, 7, 2u * 96u * 528u, 0, 8, 0, 1, false},
     CROW_FN(gemm_nvfp4_bf16_m32, 7), CROW_FN(gemm_nvfp4_bf16_m16, 7), CROW_FN(gemv_bf16_w, 5),
     CROW_FN(gemv_bf16, 5), CROW_FN(gemv_bf16_b, 5), CROW_FN(gemv_b, 5), CROW_FN(gemv_bf16_ws, 5), CROW_FN(gemv_bf16_bs, 6),
     CROW_FN(gemv_nvfp4_w_valu1, 6), CROW_FN(gemv_nvfp4_w_valu2, 6), CROW_FN(gemv_nvfp4_w_valu4, 6),  // measurement only
@@ -323,14 +327,20 @@ int crow_hip_launch_noalloc(crow_fn_t f, uint32_t gx, uint32_t gy, uint32_t gz, 
 const char* crow_hip_gemm_kernel(uint32_t rows, uint32_t m) {
     if (m <= 16) return "gemm_nvfp4_bf16_m16";
     if (m <= 96) return "gemm_nvfp4_bf16_m32";
-    static const struct { const char* name; uint32_t mt; double alone, shared; } cand[] = {
-        {"gemm_nvfp4_bf16_m48", 48, 58.0, 45.0}, {"gemm_nvfp4_bf16_m64", 64, 63.0, 48.5}, {"gemm_nvfp4_bf16_m96", 96, 78.0, 78.0}};
-    const unsigned long long quads = (rows + 4 * CROW_TILE_ROWS - 1) / (4 * CROW_TILE_ROWS);
+    // Measured on MI355X at K = 5120 (microseconds): a block of the four-wave kernels alone on a compute unit / each of several
+    // sharing one; a block of the eight-wave kernels (one per compute unit: two waves per SIMD) per round of the launch.  The
+    // launch lasts as long as the fullest compute unit.
+    static const struct { const char* name; uint32_t mt, tiles_per_block; double alone, shared; } cand[] = {
+        {"gemm_nvfp4_bf16_m48", 48, 4, 58.0, 45.0},  {"gemm_nvfp4_bf16_m64", 64, 4, 63.0, 48.5},  {"gemm_nvfp4_bf16_m96", 96, 4, 78.0, 78.0},
+        {"gemm_nvfp4_bf16_w48", 48, 8, 82.0, 82.0},  {"gemm_nvfp4_bf16_w64", 64, 8, 93.0, 93.0},  {"gemm_nvfp4_bf16_w80", 80, 8, 110.0, 110.0},
+        {"gemm_nvfp4_bf16_w96", 96, 8, 118.0, 118.0}};
+    const unsigned long long row_tiles = (rows + CROW_TILE_ROWS - 1) / CROW_TILE_ROWS;
     const unsigned long long cus = g.cus > 0 ? (unsigned long long)g.cus : 256ull;
     const char* best = cand[1].name;
     double best_t = 0.0;
     for (const auto& c : cand) {
-        const unsigned long long blocks = quads * ((m + c.mt - 1) / c.mt), per_cu = (blocks + cus - 1) / cus;
+        const unsigned long long blocks = ((row_tiles + c.tiles_per_block - 1) / c.tiles_per_block) * ((m + c.mt - 1) / c.mt);
+        const unsigned long long per_cu = (blocks + cus - 1) / cus;
         const double t = per_cu <= 1 ? c.alone : (double)per_cu * c.shared;
         if (best_t == 0.0 || t < best_t) {
             best_t = t;
@@ -423,6 +433,11 @@ int crow_hip_launch_dims_split(const char* name, uint32_t rows, uint32_t k_dim, 
             if (s > 16) s = 16;
             while (s > 1 && ((unsigned long long)rt * s * 16 * 64 > PARTIAL_FLOATS || rt > COUNTER_SLOTS)) s--;
             *out = crow_dims{rt, 1, s, 256};
+            return CROW_OK;
+        }
+        if (name[15] == '_' && name[16] == 'w') {  // gemm_nvfp4_bf16_w<tokens per block>: eight row tiles per block
+            const uint32_t mtw = (uint32_t)atoi(name + 17);
+            *out = crow_dims{(rt + 7) / 8, (z + mtw - 1) / mtw, 1, 512};
             return CROW_OK;
         }
         const uint32_t mt = name[15] == '_' ? (uint32_t)atoi(name + 17) : 128;  // gemm_nvfp4_bf16_m<tokens per block>

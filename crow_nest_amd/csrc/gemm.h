@@ -311,6 +311,82 @@ __device__ __forceinline__ void gemm_pipe_body(const unsigned char* __restrict__
     gemm_store<TBK>(acc, gs_ptr[0], y, rt, m0, rows, m_total, lane);
 }
 
+// Wide shared-X body: a block is EIGHT waves - two per SIMD, so that one wave's operand reads, decode and barrier waits run
+// under the other's matrix instructions (with one wave per SIMD all of them are serial: a 256 x 128 x 256 unit takes 5.6 us
+// against 3.3 us of issue time) - wave w owns row tile 8 * blockIdx.x + w and all of the block's MT = 16 * TBK token rows,
+// staged once in LDS for the eight row tiles.  There is ONE weight register set per wave: the next panel's weights are
+// requested when the current panel's last instruction has read them, and the SIMD's other wave hides the latency; the next
+// X tile travels through registers into the other LDS buffer as in the body above.  One barrier per panel.
+template <int TBK>
+__device__ __forceinline__ void gemm_wide_body(const unsigned char* __restrict__ w, const unsigned short* __restrict__ x,
+                                               const float* __restrict__ gs_ptr, float* __restrict__ y, int k_dim, int rows, int m_total,
+                                               __bf16* xs2) {
+    constexpr int NW = 8;
+    constexpr int MT = 16 * TBK;
+    constexpr int NT = 64 * NW;
+    constexpr int XCH = MT * 32 / NT;  // 16-byte chunks of an X tile per thread
+    static_assert(MT * 32 % NT == 0, "whole chunks per thread");
+    constexpr int XBUF = MT * CROW_GEMM_XS_STRIDE;
+    const int lane = lane_id();
+    const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
+    const int row_tiles = (rows + CROW_TILE_ROWS - 1) / CROW_TILE_ROWS;
+    const int rt = (int)blockIdx.x * NW + wave;
+    const bool has_rows = rt < row_tiles;  // wave-uniform; idle waves still stage X and join the barriers
+    const int m0 = (int)blockIdx.y * MT;
+    const int panels = (k_dim + CROW_PANEL_COLS - 1) / CROW_PANEL_COLS;
+    f32x4 acc[TBK][4];
+#pragma unroll
+    for (int tb = 0; tb < TBK; tb++)
+#pragma unroll
+        for (int j = 0; j < 4; j++) acc[tb][j] = f32x4{0.f, 0.f, 0.f, 0.f};
+    const int strips = (rows + CROW_STRIP_ROWS - 1) / CROW_STRIP_ROWS;
+    // chunk c = i * 512 + thread: token row c / 32, 8 columns from 8 (c % 32); rows beyond M read row M - 1 (never stored)
+    const int xq = ((int)threadIdx.x & 31) * 8;
+    unsigned xoff[XCH];
+#pragma unroll
+    for (int i = 0; i < XCH; i++) {
+        const int m = m0 + ((i * NT + (int)threadIdx.x) >> 5);
+        xoff[i] = (unsigned)(m < m_total ? m : m_total - 1) * (unsigned)k_dim + (unsigned)xq;
+    }
+    auto load_x = [&](int p, uint4 (&xv)[XCH]) {
+        const int k0 = p * CROW_PANEL_COLS;
+        const bool full = k0 + CROW_PANEL_COLS <= k_dim;  // uniform
+#pragma unroll
+        for (int i = 0; i < XCH; i++) {
+            xv[i] = make_uint4(0, 0, 0, 0);  // (the last, partial panel: columns beyond K are zeros)
+            if (full || k0 + xq < k_dim) xv[i] = *(const uint4*)(x + (size_t)(xoff[i] + (unsigned)k0));
+        }
+    };
+    auto store_x = [&](__bf16* xs, const uint4 (&xv)[XCH]) {
+#pragma unroll
+        for (int i = 0; i < XCH; i++) {
+            const int c = i * NT + (int)threadIdx.x, r = c >> 5, q = c & 31;
+            *(uint4*)(xs + r * CROW_GEMM_XS_STRIDE + q * 8) = xv[i];
+        }
+    };
+    const int lane_off = (lane & 15) * CROW_GEMM_XS_STRIDE + (lane >> 4) * 8;
+    PanelRegs pr;
+    uint4 xv[XCH];
+    load_x(0, xv);
+    load_panel(w, has_rows ? rt : 0, strips, panels, 0, lane, pr);
+    store_x(xs2, xv);
+    __syncthreads();
+    int h = 0;
+    for (int p = 0; p < panels; p++) {
+        const bool more = p + 1 < panels;
+        if (more) load_x(p + 1, xv);
+        gemm_panel<TBK>(pr, xs2 + h * XBUF + lane_off, acc);
+        if (more) {
+            load_panel(w, has_rows ? rt : 0, strips, panels, p + 1, lane, pr);
+            store_x(xs2 + (h ^ 1) * XBUF, xv);
+        }
+        __syncthreads();  // the other buffer is written, and this one read, by every wave
+        h ^= 1;
+    }
+    if (!has_rows) return;
+    gemm_store<TBK>(acc, gs_ptr[0], y, rt, m0, rows, m_total, lane);
+}
+
 }  // namespace crow
 
 // Y[M][rows] f32 = X[M][k_dim] bf16 times the tiled NVFP4 tensor, times gs.  The argument list is
@@ -361,3 +437,20 @@ CROW_GEMM_PIPE_ENTRY(gemm_nvfp4_bf16_m48, 3, 2)
 CROW_GEMM_PIPE_ENTRY(gemm_nvfp4_bf16_m64, 4, 2)
 CROW_GEMM_PIPE_ENTRY(gemm_nvfp4_bf16_m96, 6, 1)
 CROW_GEMM_PIPE_ENTRY(gemm_nvfp4_bf16, 8, 1)
+// the wide shared-X body: grid (ceil(row_tiles / 8), ceil(M / MT)), block 512, MT = 16 TBK tokens; dynamic LDS = two X tiles
+#define CROW_GEMM_WIDE_ENTRY(NAME, TBK)                                                                                        \
+    extern "C" __global__ void __launch_bounds__(512, 1) NAME(const unsigned char* __restrict__ w, const unsigned short* __restrict__ x, \
+                                                         const float* __restrict__ gs_ptr, float* __restrict__ y,              \
+                                                         const int* __restrict__ k_dim_p, const int* __restrict__ rows_p,      \
+                                                         const int* __restrict__ m_p) {                                        \
+        /* 512 threads; X is addressed with 32-bit element offsets */                                                         \
+        if (block_threads() != 512 || *m_p < 1 || (unsigned long long)*m_p * (unsigned long long)*k_dim_p > 0xffffffffull) {   \
+            if (threadIdx.x == 0) atomicOr(crow::g_ws.status, crow::STATUS_BAD_SHAPE);                                         \
+            return;                                                                                                            \
+        }                                                                                                                      \
+        crow::gemm_wide_body<TBK>(w, x, gs_ptr, y, *k_dim_p, *rows_p, *m_p, (__bf16*)crow_dyn_lds);                            \
+    }
+CROW_GEMM_WIDE_ENTRY(gemm_nvfp4_bf16_w48, 3)
+CROW_GEMM_WIDE_ENTRY(gemm_nvfp4_bf16_w64, 4)
+CROW_GEMM_WIDE_ENTRY(gemm_nvfp4_bf16_w80, 5)
+CROW_GEMM_WIDE_ENTRY(gemm_nvfp4_bf16_w96, 6)

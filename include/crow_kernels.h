@@ -97,6 +97,12 @@ CROW_KERNEL(moe_down_grouped, 9)
  * the quantised-activation buffer: x is bf16).  gemm_nvfp4_bf16_m16 serves *m_p <= 16 only; the others take any m
  * and differ in tiling (32, 48, 64, 96, 128 tokens per block); crow_hip_gemm_kernel names the one to use. */
 CROW_KERNEL(gemm_nvfp4_bf16, 7)
+/* the same product in blocks of eight waves (two per SIMD) x 48 / 64 / 80 / 96 tokens: what crow_hip_gemm_kernel picks from a few
+ * hundred tokens on */
+CROW_KERNEL(gemm_nvfp4_bf16_w48, 7)
+CROW_KERNEL(gemm_nvfp4_bf16_w64, 7)
+CROW_KERNEL(gemm_nvfp4_bf16_w80, 7)
+CROW_KERNEL(gemm_nvfp4_bf16_w96, 7)
 CROW_KERNEL(gemm_nvfp4_bf16_m96, 7)
 CROW_KERNEL(gemm_nvfp4_bf16_m64, 7)
 CROW_KERNEL(gemm_nvfp4_bf16_m48, 7)

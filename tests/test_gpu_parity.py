@@ -725,7 +725,7 @@ def test_config3_full_size_head(eng):
 # ---------------------------------------------------------------- batched GEMM on the matrix cores (config 4)
 
 @pytest.mark.parametrize("kernel", ["gemm_nvfp4_bf16_m16", "gemm_nvfp4_bf16_m32", "gemm_nvfp4_bf16_m48", "gemm_nvfp4_bf16_m64", "gemm_nvfp4_bf16_m96",
-                                    "gemm_nvfp4_bf16"])
+                                    "gemm_nvfp4_bf16", "gemm_nvfp4_bf16_w48", "gemm_nvfp4_bf16_w64", "gemm_nvfp4_bf16_w80", "gemm_nvfp4_bf16_w96"])
 @pytest.mark.parametrize("m,rows,cols", [(16, 320, 1024), (5, 100, 320), (17, 100, 320), (33, 256, 512), (128, 512, 2048), (200, 192, 5120)])
 def test_gemm_bf16_against_the_cpu_path(eng, m, rows, cols, kernel):
     """Weights decode to exact bf16, X is bf16, products are exact in f32: only the summation order
@@ -737,7 +737,8 @@ def test_gemm_ragged_shapes_drawn_at_random(eng):
     """Sixteen (tokens, rows, columns) triples drawn with a fixed seed - partial row tiles, partial panels, partial token
     blocks - through the entry point the library picks and through one drawn at random."""
     g = np.random.default_rng(4242)
-    names = ["gemm_nvfp4_bf16_m32", "gemm_nvfp4_bf16_m48", "gemm_nvfp4_bf16_m64", "gemm_nvfp4_bf16_m96", "gemm_nvfp4_bf16"]
+    names = ["gemm_nvfp4_bf16_m32", "gemm_nvfp4_bf16_m48", "gemm_nvfp4_bf16_m64", "gemm_nvfp4_bf16_m96", "gemm_nvfp4_bf16", "gemm_nvfp4_bf16_w48",
+             "gemm_nvfp4_bf16_w64", "gemm_nvfp4_bf16_w80", "gemm_nvfp4_bf16_w96"]
     for case in range(16):
         m = int(g.integers(5, 300))
         rows = int(g.integers(1, 700))
@@ -780,7 +781,7 @@ def _gemm_case(eng, m, rows, cols, kernel):
     assert gamma_ratio(y[:4], w, rows, cols, gs, xw.reshape(m, cols)[:4]) <= 1.0
 
 
-@pytest.mark.parametrize("m", [512, 128])
+@pytest.mark.parametrize("m", [512, 128, 384])
 def test_gemm_full_size_sampled_rows(eng, m):
     """Benchmark config 4 (batched GEMM) at M = 512 and M = 128 on the full [17408, 5120] tensor; the CPU path checks 768 sampled rows."""
     rows, cols = 17408, 5120
