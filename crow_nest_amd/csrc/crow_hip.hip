@@ -31,7 +31,7 @@ struct FnEntry {
 // NR tensors per block, bodies for 1 .. MMAX activation rows, bf16 or f32 activations
 // (the bodies for several rows need more registers than a block of sixteen waves leaves each: they run in blocks of eight)
 #define CROW_GEMV(name, nargs, NR, MMAX, XBF16) \
-    {#name, (const void*)&name, nargs, 0u, NR, MMAX > 1 ? 8 : 16, crow::crow_gemv_lds_per_wave(MMAX, XBF16), MMAX > 1 ? CROW_MULTI_STRIPS : 1, true}
+    {#name, (const void*)&name, nargs, 0u, NR, MMAX > 1 ? 8 : 16, crow::crow_gemv_lds_per_wave(MMAX, XBF16), MMAX > 1 ? (XBF16 ? CROW_MULTI_STRIPS_BF16 : CROW_MULTI_STRIPS) : 1, true}
 const FnEntry g_table[] = {
     CROW_GEMV(gemv_nvfp4_w, 6, 1, 1, false),       CROW_GEMV(gemv_nvfp4_w_bf16, 6, 1, 1, true),  CROW_GEMV(gemv_nvfp4_w_argmax, 7, 1, 1, false),
     CROW_GEMV(gemv_nvfp4_gu, 8, 2, 1, false),      CROW_GEMV(gemv_nvfp4_gu_bf16, 8, 2, 1, true),

@@ -111,7 +111,12 @@ extern "C" __global__ void __launch_bounds__(1024) gemv_nvfp4_gu_bf16(const unsi
 #ifndef CROW_MULTI_STRIPS
 #define CROW_MULTI_STRIPS 2
 #endif
-template <int NR, bool XBF16, int EPI>
+// ... except the bf16 twins of the verify kernels: their rows ride in one operand set, the operand reads are a sixth of the
+// f32 kernels', and one strip per block (the one-row kernels' walk, four groups in flight) measured faster at two rows
+#ifndef CROW_MULTI_STRIPS_BF16
+#define CROW_MULTI_STRIPS_BF16 1
+#endif
+template <int NR, bool XBF16, int EPI, int NS = CROW_MULTI_STRIPS>
 __device__ __forceinline__ void gemv_m_dispatch(const GemvArgs& a, int m, unsigned z, lds_p lds, const Workspace& ws) {
     if (m < 1 || m > 4) {  // the reference's NVFP4_MMAX (engine/src/kernels_p2.rs:397-400); uniform over the launch
         if (threadIdx.x == 0) atomicOr(ws.status, STATUS_BAD_SHAPE);
@@ -119,10 +124,10 @@ __device__ __forceinline__ void gemv_m_dispatch(const GemvArgs& a, int m, unsign
     }
     // one body per M keeps each row's operation sequence identical to the one-row kernel
     switch (m) {
-        case 1: gemv_body<NR, 1, XBF16, EPI, 4, CROW_MULTI_STRIPS>(a, z, lds, ws); break;
-        case 2: gemv_body<NR, 2, XBF16, EPI, 4, CROW_MULTI_STRIPS>(a, z, lds, ws); break;
-        case 3: gemv_body<NR, 3, XBF16, EPI, 4, CROW_MULTI_STRIPS>(a, z, lds, ws); break;
-        default: gemv_body<NR, 4, XBF16, EPI, 4, CROW_MULTI_STRIPS>(a, z, lds, ws); break;
+        case 1: gemv_body<NR, 1, XBF16, EPI, 4, NS>(a, z, lds, ws); break;
+        case 2: gemv_body<NR, 2, XBF16, EPI, 4, NS>(a, z, lds, ws); break;
+        case 3: gemv_body<NR, 3, XBF16, EPI, 4, NS>(a, z, lds, ws); break;
+        default: gemv_body<NR, 4, XBF16, EPI, 4, NS>(a, z, lds, ws); break;
     }
 }
 // The activation row count of a verify launch: from the geometry word when the launcher put it there (then the word behind
@@ -164,7 +169,7 @@ extern "C" __global__ void __launch_bounds__(512) gemv_nvfp4_wm_bf16(const unsig
     ENTER(w, x, gs_ptr, y, k_dim_p, rows_p, m_p, geo);
     const int pairs = geo & 0xFFFFF;
     GemvArgs a = gemv_args(w, nullptr, gs_ptr, nullptr, x, (size_t)pairs * CROW_PAIR_COLS, y, 0, pairs, k_dim_p, rows_p);
-    gemv_m_dispatch<1, true, EPI_SCALE>(a, rows_of(a, geo, m_p), 0, LDS, ws);
+    gemv_m_dispatch<1, true, EPI_SCALE, CROW_MULTI_STRIPS_BF16>(a, rows_of(a, geo, m_p), 0, LDS, ws);
 }
 extern "C" __global__ void __launch_bounds__(512) gemv_nvfp4_gum_bf16(const unsigned char* __restrict__ wg, const unsigned char* __restrict__ wu,
                                                                        const unsigned short* __restrict__ x, const float* __restrict__ gs_g,
@@ -174,7 +179,7 @@ extern "C" __global__ void __launch_bounds__(512) gemv_nvfp4_gum_bf16(const unsi
     ENTER(wg, wu, x, gs_g, gs_u, y, k_dim_p, rows_p, m_p, geo);
     const int pairs = geo & 0xFFFFF;
     GemvArgs a = gemv_args(wg, wu, gs_g, gs_u, x, (size_t)pairs * CROW_PAIR_COLS, y, 0, pairs, k_dim_p, rows_p);
-    gemv_m_dispatch<2, true, EPI_SILU_GU>(a, rows_of(a, geo, m_p), 0, LDS, ws);
+    gemv_m_dispatch<2, true, EPI_SILU_GU, CROW_MULTI_STRIPS_BF16>(a, rows_of(a, geo, m_p), 0, LDS, ws);
 }
 
 // ------------------------------------------------------------------ batched over token rows
