@@ -25,6 +25,9 @@ struct FnEntry {
     int lds_per_wave;
     int ns;  // adjacent 16-row strips per block (kernels for several activation rows: CROW_MULTI_STRIPS), else 1
     bool takes_ws;  // the launcher appends the scratch descriptor (every kernel of the GEMV family)
+    // a twin of `stub` for strips of exactly two groups (K in 257 .. 512), started in its place when the launch dimensions say
+    // so; its dynamic LDS is the zero area and ONE staging area (per block, not per wave)
+    const void* short_k_stub;
 };
 
 #define CROW_FN(name, nargs) {#name, (const void*)&name, nargs, 0u, 0, 16, 0, 1, false}
@@ -39,7 +42,8 @@ const FnEntry g_table[] = {
     CROW_GEMV(gemv_nvfp4_wm_bf16, 7, 1, 4, true),  CROW_GEMV(gemv_nvfp4_gum_bf16, 9, 2, 4, true), CROW_GEMV(gemv_fp4, 6, 1, 1, false),
     CROW_GEMV(gemv_fp4_b, 7, 1, 4, false),         CROW_GEMV(gemv_fp4_b1k, 7, 1, 4, false),      CROW_GEMV(gemv_fp4_bs, 8, 1, 4, false),
     CROW_GEMV(gemv_fp4_ptrb, 8, 1, 1, false),      CROW_GEMV(moe_gate_up_silu, 8, 2, 1, false),  CROW_GEMV(moe_down_combine, 7, 1, 1, false),
-    CROW_GEMV(moe_route_gate_up_silu, 11, 2, 1, false), CROW_GEMV(moe_gate_up_silu_grouped, 11, 2, 4, false), CROW_GEMV(moe_down_grouped, 9, 1, 4, false),
+    CROW_GEMV(moe_route_gate_up_silu, 11, 2, 1, false), CROW_GEMV(moe_gate_up_silu_grouped, 11, 2, 4, false),
+    {"moe_down_grouped", (const void*)&moe_down_grouped, 9, 0u, 1, 8, crow::crow_gemv_lds_per_wave(4, false), CROW_MULTI_STRIPS, true, (const void*)&moe_down_grouped_short_k},
     CROW_FN(moe_group, 6),
     CROW_FN(router_top10, 10),     CROW_FN(silu_mul_combo, 3),      CROW_FN(acc_combo, 3),
     CROW_FN(argmax_k, 3),          CROW_FN(dequant_fp4_flat, 4),    CROW_FN(repack_nvfp4, 4),
@@ -140,10 +144,18 @@ int launch_entry(const FnEntry* e, dim3 grid, dim3 block, const uint64_t* vals, 
         args[na++] = (void*)&geo;
     }
     if (e->takes_ws) args[na++] = (void*)&ws_arg;
+    const void* stub = e->stub;
+    if (e->short_k_stub != nullptr) {
+        const unsigned pairs = (unsigned)geo & 0xFFFFFu;
+        if (pairs > CROW_GROUP_PAIRS && pairs <= 2 * CROW_GROUP_PAIRS && block.x <= 256) {
+            stub = e->short_k_stub;
+            lds = (size_t)CROW_GEMV_ZERO_BYTES + (size_t)e->lds_per_wave;
+        }
+    }
     const bool head = e->stub == (const void*)&gemv_nvfp4_w_argmax;
     // the fused head keeps one key per strip (the kernel checks again and reports through the status word)
     if (head && grid.x > ws.head_words) return CROW_ERR_WORKSPACE;
-    hipError_t rc = hipLaunchKernel(e->stub, grid, block, args, lds, s);
+    hipError_t rc = hipLaunchKernel(stub, grid, block, args, lds, s);
     if (rc == hipSuccess && head) {  // ... and its finishing kernel right behind it: the token out of the strips' keys
         unsigned strips = grid.x;
         void* fargs[3] = {(void*)&vals[6], (void*)&strips, (void*)&ws_arg};
@@ -384,6 +396,11 @@ int crow_hip_launch_dims_split(const char* name, uint32_t rows, uint32_t k_dim, 
         if (down_combine) {  // rows = hidden; one wave per picked expert, every wave all columns of its strip
             if (g.geo_topk < 1 || g.geo_topk > 16) return CROW_ERR_GEO;
             *out = crow_dims{strips, pairs | (1u << 24), z, 64u * (uint32_t)g.geo_topk};
+            return CROW_OK;
+        }
+        if (strcmp(name, "moe_down_grouped") == 0 && groups == 2) {  // short K: 4 waves per block, each a run of CROW_SHORTK_STRIPS strips
+            const uint32_t per_block = 4u * CROW_SHORTK_STRIPS;
+            *out = crow_dims{(strips + per_block - 1) / per_block, pairs | (1u << 24), z, 256};
             return CROW_OK;
         }
         if (verify && z > 4) return CROW_ERR_SHAPE;

@@ -543,6 +543,130 @@ struct MultiWalk {
     }
 };
 
+// The walk of a wave over MANY strips of FEW groups (short K: the routed experts' down slabs, K = 512 -> two groups per strip).
+// Walking such strips one block each means tens of thousands of blocks that each stage the same activations, fill a pipeline
+// of two groups and drain it again.  Here the block stages the tile's activations ONCE (all G groups of all M rows; they never
+// change along the walk) and every wave streams a run of consecutive strips - whose groups are one contiguous run of
+// 2304-byte records in memory - through the ring of four, with no activation traffic and no staging inside the loop.  Per
+// strip and activation row the operation sequence is StripWalk's for a strip walked by one wave, so the sums are the same bits.
+//   G   groups per strip, a power of two <= the ring (ring slot J always holds a group J % G)
+template <int M, int G>
+struct ShortKWalk {
+    static_assert(G == 1 || G == 2 || G == 4, "a ring slot's group index is static");
+    static constexpr int XR = 3 * M, NSET = (3 * M + 3) / 4, SLOT = XR * CROW_GEMV_XROW_BYTES;
+    unsigned sc[CROW_GEMV_RING][1];
+    u32x4 cd[CROW_GEMV_RING][1][2];
+    lds_p a1[G][NSET], a2[G][NSET];  // this lane's operand addresses in group g's staged rows (or in the zero area)
+    const unsigned char* wl;         // the lane's view of the wave's first record
+    int lane;
+    float acc[1][M];
+
+    // f32 activations of one group of one row -> three bf16 rows (hi, mid, lo) of the group's staged area; lane = 4 columns
+    static __device__ __forceinline__ void stage_row(lds_p staged, int g, int t, f32x4 v, int lane_) {
+        unsigned h[4], m[4], l[4];
+        split3(v.x, h[0], m[0], l[0]);
+        split3(v.y, h[1], m[1], l[1]);
+        split3(v.z, h[2], m[2], l[2]);
+        split3(v.w, h[3], m[3], l[3]);
+        lds_p row = staged + g * SLOT + (3 * t) * CROW_GEMV_XROW_BYTES + 8 * lane_;
+        lds_store8(row, __builtin_amdgcn_perm(h[1], h[0], 0x07060302u), __builtin_amdgcn_perm(h[3], h[2], 0x07060302u));
+        lds_store8(row + CROW_GEMV_XROW_BYTES, __builtin_amdgcn_perm(m[1], m[0], 0x07060302u), __builtin_amdgcn_perm(m[3], m[2], 0x07060302u));
+        lds_store8(row + 2 * CROW_GEMV_XROW_BYTES, __builtin_amdgcn_perm(l[1], l[0], 0x07060302u), __builtin_amdgcn_perm(l[3], l[2], 0x07060302u));
+    }
+    __device__ __forceinline__ void init(const unsigned char* first_record, lds_p staged, lds_p zero) {
+        lane = lane_id();
+        wl = first_record;
+#pragma unroll
+        for (int m = 0; m < M; m++) acc[0][m] = 0.0f;
+        // (the operand addressing of StripWalk::init, one staged area per group)
+        const int g = lane >> 4, i = lane & 15, r4 = i & 3;
+        const bool half_ok = (g >> 1) == (i >> 3);
+        const bool second = ((i >> 2) & 1) != 0;
+#pragma unroll
+        for (int s = 0; s < G; s++)
+#pragma unroll
+            for (int q = 0; q < NSET; q++) {
+                const int row = 4 * q + r4;
+                const bool live = half_ok && row < XR;
+                lds_p data = staged + s * SLOT + row * CROW_GEMV_XROW_BYTES + 16 * g;
+                a1[s][q] = (live && !second) ? data : zero + 16 * g;
+                a2[s][q] = (live && second) ? data + 64 : zero + 16 * g;
+            }
+    }
+    template <int J>
+    __device__ __forceinline__ void issue_w(int i) {
+        const unsigned char* p = wl + (size_t)i * CROW_GROUP_BYTES;
+        sc[J][0] = stream_load_u32((const unsigned*)p + lane);
+        cd[J][0][0] = stream_load_v((const uint4*)(p + CROW_GROUP_SCALE_BYTES) + lane);
+        cd[J][0][1] = stream_load_v((const uint4*)(p + CROW_GROUP_SCALE_BYTES + 1024) + lane);
+    }
+    // record i sits in slot J: multiply it by its group's staged rows; behind a strip's last group hand the strip's sums to
+    // `emit(strip index within the run, v)` - v in lane l = the dot product of strip row l % 16 with activation row l / 16
+    template <int J, class Emit>
+    __device__ __forceinline__ void multiply(int i, Emit& emit) {
+        group_multiply<M, false, 1>(sc[J], cd[J], a1[J % G], a2[J % G], acc);
+        __builtin_amdgcn_sched_barrier(0);
+        if (J % G == G - 1) {
+            float v = 0.0f;
+#pragma unroll
+            for (int m = 0; m < M; m++) {  // (StripWalk::finish)
+                const unsigned a = __float_as_uint(acc[0][m]);
+                const u32x2 sw = __builtin_amdgcn_permlane32_swap(a, a, false, false);
+                const unsigned b = __float_as_uint(__fadd_rn(__uint_as_float(sw.x), __uint_as_float(sw.y)));
+                const u32x2 sq = __builtin_amdgcn_permlane16_swap(b, b, false, false);
+                const float o = __fadd_rn(__uint_as_float(sq.x), __uint_as_float(sq.y));
+                v = (lane >> 4) == m ? o : v;
+                acc[0][m] = 0.0f;
+            }
+            emit(i / G, v);
+        }
+    }
+    // `count` records (a multiple of G) from the wave's first one; `mid` runs once, after the first loads have left: the
+    // block's staging and its barrier
+    template <class Mid, class Emit>
+    __device__ __forceinline__ void go(int count, Mid mid, Emit emit) {
+        const int nq = count >> 2, r = count & 3;
+        if (nq > 0) {
+            issue_w<0>(0);
+            issue_w<1>(1);
+            issue_w<2>(2);
+            issue_w<3>(3);
+            mid();
+            int q = 0;
+            for (; q + 1 < nq; q++) {
+                const int i0 = 4 * q;
+                multiply<0>(i0, emit);
+                issue_w<0>(i0 + 4);
+                multiply<1>(i0 + 1, emit);
+                issue_w<1>(i0 + 5);
+                multiply<2>(i0 + 2, emit);
+                issue_w<2>(i0 + 6);
+                multiply<3>(i0 + 3, emit);
+                issue_w<3>(i0 + 7);
+            }
+            const int i0 = 4 * q;
+            multiply<0>(i0, emit);
+            if (r > 0) issue_w<0>(i0 + 4);
+            multiply<1>(i0 + 1, emit);
+            if (r > 1) issue_w<1>(i0 + 5);
+            multiply<2>(i0 + 2, emit);
+            if (r > 2) issue_w<2>(i0 + 6);
+            multiply<3>(i0 + 3, emit);
+            if (r > 0) multiply<0>(i0 + 4, emit);
+            if (r > 1) multiply<1>(i0 + 5, emit);
+            if (r > 2) multiply<2>(i0 + 6, emit);
+        } else {
+            if (r > 0) issue_w<0>(0);
+            if (r > 1) issue_w<1>(1);
+            if (r > 2) issue_w<2>(2);
+            mid();
+            if (r > 0) multiply<0>(0, emit);
+            if (r > 1) multiply<1>(1, emit);
+            if (r > 2) multiply<2>(2, emit);
+        }
+    }
+};
+
 // Ordering point of the cross-block hand-over.  Every access to the shared partials and counters is an agent-scope atomic:
 // on gfx950 such a store / load / read-modify-write carries the coherence bit that makes it bypass the per-die L2 for
 // data other dies may touch, so each one is performed at the level all compute dies share.  What is left to guarantee is
@@ -744,6 +868,74 @@ __device__ __forceinline__ void gemv_body(const GemvArgs& a, unsigned z, lds_p l
             a.y[yo + row] = silu_mul(v[s] * a.gs[0][0], v[(NR - 1) * NS + s] * a.gs[NR - 1][0]);
         }
     }
+}
+
+// The body of a short-K product (ShortKWalk): grid.x blocks of W waves, every wave a run of CROW_SHORTK_STRIPS consecutive
+// strips of the tensor, all M activation rows staged once per block.  `lds`: the zero area, then G x 3 M staged rows.
+#ifndef CROW_SHORTK_STRIPS
+#define CROW_SHORTK_STRIPS 8
+#endif
+template <int M, int G>
+__device__ __forceinline__ void short_k_body(const GemvArgs& a, lds_p lds, const Workspace& ws) {
+    typedef ShortKWalk<M, G> Walk;
+    const int lane = lane_id();
+    const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6)), waves = block_threads() >> 6;
+    const int k_dim = a.pairs * CROW_PAIR_COLS;
+    const int strip0 = ((int)blockIdx.x * waves + wave) * CROW_SHORTK_STRIPS;
+    size_t xoff[M];
+    int yrow[M];
+#pragma unroll
+    for (int m = 0; m < M; m++) {
+        if (a.row_map != nullptr) {
+            const int c = a.row_map[m];
+            xoff[m] = (size_t)(c / a.x_div) * a.x_stride;
+            yrow[m] = c;
+        } else {
+            xoff[m] = (size_t)m * a.x_stride;
+            yrow[m] = a.y_row0 + m;
+        }
+    }
+    // the row count bounds every wave's run (its word arrives with the caller's other words: no round trip of its own), and
+    // a grid that does not cover the tensor is refused
+    const int strips = (*a.rows_p + CROW_STRIP_ROWS - 1) / CROW_STRIP_ROWS;
+    const int left = strips - strip0;
+    const int n_strips = left < 0 ? 0 : (left < CROW_SHORTK_STRIPS ? left : CROW_SHORTK_STRIPS);
+    const bool covered = (long long)gridDim.x * waves * CROW_SHORTK_STRIPS >= (long long)strips;
+    lds_p zero = lds, staged = lds + CROW_GEMV_ZERO_BYTES;
+    Walk walk;
+    walk.init(a.w[0] + (size_t)strip0 * G * CROW_GROUP_BYTES, staged, zero);
+    int rows = 0;
+    float gs = 0.0f;
+    bool ok = true;
+    auto mid = [&]() {
+        for (int o = 16 * (int)threadIdx.x; o < CROW_GEMV_ZERO_BYTES; o += 16 * (waves << 6)) lds_store16(zero + o, 0, 0, 0, 0);
+        // (group, row) pairs dealt to the waves; a lane whose four columns lie beyond K stages zeros
+#pragma unroll
+        for (int t = 0; t < M; t++)
+#pragma unroll
+            for (int g = 0; g < G; g++) {
+                if ((t * G + g) % waves != wave) continue;  // wave-uniform
+                const int col = g * CROW_GROUP_COLS + 4 * lane;
+                f32x4 v = {0.f, 0.f, 0.f, 0.f};
+                if (col < k_dim) v = *(const f32x4*)((const float*)a.x + xoff[t] + col);
+                Walk::stage_row(staged, g, t, v, lane);
+            }
+        rows = *a.rows_p;
+        gs = a.gs[0][0];
+        ok = covered && *a.k_dim_p == k_dim && (a.count_p == nullptr || *a.count_p == a.count_expect);
+        __syncthreads();
+    };
+    const int mo = lane >> 4, n = lane & 15;
+    int yr = yrow[0];
+#pragma unroll
+    for (int m = 1; m < M; m++)
+        if (mo == m) yr = yrow[m];
+    auto emit = [&](int s, float v) {
+        const int row = (strip0 + s) * CROW_STRIP_ROWS + n;
+        if (ok && mo < M && row < rows) a.y[(size_t)yr * (a.y_stride != 0 ? a.y_stride : (size_t)rows) + row] = v * gs;
+    };
+    walk.go(n_strips * G, mid, emit);
+    if (!ok && threadIdx.x == 0) atomicOr(ws.status, STATUS_BAD_SHAPE);
 }
 
 }  // namespace crow

@@ -385,3 +385,31 @@ extern "C" __global__ void __launch_bounds__(512) moe_down_grouped(const int4* _
     a.row_map = perm + tl.y, a.x_div = 1;
     gemv_m_dispatch<1, false, EPI_SCALE>(a, tl.z, blockIdx.z, LDS, ws);
 }
+// The same for strips of two groups (K in 257 .. 512: this model's down slabs), which the launcher starts in place of the
+// kernel above whenever the launch dimensions say so (one table entry, one name): every wave streams a run of strips against
+// activations staged once per block (gemv.h: ShortKWalk); crow_hip_launch_dims sizes grid.x for it.  Same bits.
+extern "C" __global__ void __launch_bounds__(256) moe_down_grouped_short_k(const int4* __restrict__ tiles, const int* __restrict__ n_tiles_p,
+                                                                            const int* __restrict__ perm, const unsigned long long* __restrict__ table,
+                                                                            const float* __restrict__ h, const float* __restrict__ gs_ptr,
+                                                                            float* __restrict__ eo, const int* __restrict__ k_dim_p,
+                                                                            const int* __restrict__ rows_p, int geo, const Workspace ws) {
+    ENTER(tiles, n_tiles_p, perm, table, h, gs_ptr, eo, k_dim_p, rows_p, geo);
+    const int pairs = geo & 0xFFFFF;
+    const int z = (int)blockIdx.z;
+    if (z >= *n_tiles_p) return;
+    const int4 tl = tiles[z];
+    const unsigned char* w = (const unsigned char*)table[2 * tl.x + 1];
+    CROW_REFUSE_NULL_SLAB(w);
+    if (pairs <= CROW_GROUP_PAIRS || pairs > 2 * CROW_GROUP_PAIRS || tl.z < 1 || tl.z > 4) {
+        if (threadIdx.x == 0) atomicOr(ws.status, STATUS_BAD_SHAPE);
+        return;
+    }
+    GemvArgs a = gemv_args(w, nullptr, gs_ptr, nullptr, h, (size_t)pairs * CROW_PAIR_COLS, eo, 0, pairs, k_dim_p, rows_p);
+    a.row_map = perm + tl.y, a.x_div = 1;
+    switch (tl.z) {
+        case 1: short_k_body<1, 2>(a, LDS, ws); break;
+        case 2: short_k_body<2, 2>(a, LDS, ws); break;
+        case 3: short_k_body<3, 2>(a, LDS, ws); break;
+        default: short_k_body<4, 2>(a, LDS, ws); break;
+    }
+}

@@ -628,6 +628,55 @@ def test_moe_layer_grouped_by_expert(eng, t):
     eng.check()
 
 
+@pytest.mark.parametrize("inter,hdim", [(512, 2048), (448, 200), (320, 1000)])
+def test_grouped_down_on_strips_of_two_groups_gives_the_bits_of_one_row_launches(eng, inter, hdim):
+    """K in 257 .. 512 (the down slabs of this model: K = 512): moe_down_grouped runs its twin that stages a tile's activation
+    rows once per block and streams runs of strips.  Every output row must be, bit for bit, what a one-row launch (gemv_nvfp4_w)
+    gives on that combo's slab and activation row - the contract of every kernel for several rows - also with a partial last
+    group (K = 448, 320), a row count that is no multiple of 16 or of a block's strips, and tiles of 1 .. 4 rows."""
+    from crow_nest_amd.kernels import launch_dims, launch_v
+    from crow_nest_amd.weights import load_expert_slabs
+    E = 8
+    print(f"case grouped down inter={inter} hdim={hdim}", flush=True)
+    dn = random_nvfp4(910 + inter, E * hdim, inter, scale_lo=0x30, scale_hi=0x48, p7f=0)
+    slabs = load_expert_slabs(dn, E, hdim, inter, 3.0e-3)
+    ids = np.array([3, 1, 3, 0, 3, 7, 3, 1, 7, 3, 7, 5, 5, 5], dtype=np.int32)  # expert 3: five combos -> tiles of 4 + 1
+    combos = ids.size
+    perm = np.argsort(ids, kind="stable").astype(np.int32)
+    tiles, start = [], 0
+    for e in range(E):
+        c = int((ids == e).sum())
+        for q in range(0, c, 4):
+            tiles.append((e, start + q, min(4, c - q), 0))
+        start += c
+    max_tiles = len(tiles) + 3  # blocks of tiles beyond the count leave at once
+    tl = np.zeros((max_tiles, 4), dtype=np.int32)
+    tl[:len(tiles)] = np.array(tiles, dtype=np.int32)
+    table = torch.tensor([[0, slabs.ptr(e)] for e in range(E)], dtype=torch.int64, device=eng.dev)
+    h = normal_f32(12, inter + hdim, combos * inter).reshape(combos, inter)
+    hd = _dev(h)
+    eo = torch.full((combos, hdim), float("nan"), dtype=torch.float32, device=eng.dev)
+    p = eng.p
+    dims = launch_dims("moe_down_grouped", hdim, inter, max_tiles)
+    assert dims[3] == 256 and dims[0] == (hdim + 16 * 32 - 1) // (16 * 32)  # the twin's grid: 4 waves x 8 strips per block
+    tl_d, nt_d, perm_d = _dev(tl), _dev(np.array([len(tiles)], dtype=np.int32)), _dev(perm)
+    launch_v(eng.k.f("moe_down_grouped"), *dims,
+             [tl_d.data_ptr(), nt_d.data_ptr(), perm_d.data_ptr(), table.data_ptr(), hd.data_ptr(), slabs.gs.data_ptr(), eo.data_ptr(), p.i32(inter),
+              p.i32(hdim)])
+    eng.check()
+    got = eo.cpu().numpy()
+    one = torch.empty((hdim,), dtype=torch.float32, device=eng.dev)
+    d1 = launch_dims("gemv_nvfp4_w", hdim, inter, 1)
+    rb = inter // 64 * 36
+    for c in range(combos):
+        e = int(ids[c])
+        launch_v(eng.k.f("gemv_nvfp4_w"), *d1, [slabs.ptr(e), hd[c].data_ptr(), slabs.gs.data_ptr(), one.data_ptr(), p.i32(inter), p.i32(hdim)])
+        eng.check()
+        assert np.array_equal(one.cpu().numpy().view(np.uint32), got[c].view(np.uint32)), c
+    ref = orc.gemv(dn[3 * hdim * rb:4 * hdim * rb], hdim, inter, 3.0e-3, h[2])[0]  # combo 2 picked expert 3
+    assert rel_err(got[2], ref) <= TOL
+
+
 # ---------------------------------------------------------------- benchmark config 0 (dense GEMV [17408, 5120], f32 x) at full size
 
 def test_config0_full_size(eng):
