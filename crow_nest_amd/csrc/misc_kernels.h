@@ -391,17 +391,35 @@ extern "C" __global__ void __launch_bounds__(1024) moe_group(const int* __restri
         }
     }
     const int tc = (cnt + 3) >> 2;
-    s_off[t] = cnt;
-    s_tile[t] = tc;
-    __syncthreads();
-    for (int d = 1; d < 1024; d <<= 1) {  // inclusive scans over the experts: combos, and tiles of four
-        const int a = t >= d ? s_off[t - d] : 0, b = t >= d ? s_tile[t - d] : 0;
-        __syncthreads();
-        s_off[t] += a;
-        s_tile[t] += b;
-        __syncthreads();
+    // inclusive scans over the experts - combos, and tiles of four - inside each wavefront by lane shifts, then over the
+    // sixteen wavefronts' totals: two block barriers instead of two per doubling step
+    const int ln = lane_id(), wv = t >> 6;
+    int so = cnt, st = tc;
+#pragma unroll
+    for (int d = 1; d < 64; d <<= 1) {
+        const int a = __shfl_up(so, d), b = __shfl_up(st, d);
+        if (ln >= d) {
+            so += a;
+            st += b;
+        }
     }
-    const int first = s_off[t] - cnt, first_tile = s_tile[t] - tc, total_tiles = s_tile[1023];
+    if (ln == 63) {
+        s_off[wv] = so;
+        s_tile[wv] = st;
+    }
+    __syncthreads();
+    int base_o = 0, base_t = 0, total_tiles = 0;
+#pragma unroll
+    for (int q = 0; q < 16; q++) {
+        const int a = s_off[q], b = s_tile[q];
+        if (q < wv) {
+            base_o += a;
+            base_t += b;
+        }
+        total_tiles += b;
+    }
+    __syncthreads();  // the totals are read before s_off is reused below
+    const int first = base_o + so - cnt, first_tile = base_t + st - tc;
     if (total_tiles > max_tiles) {  // uniform: every thread reads the same total
         if (t == 0) {
             atomicOr(g_ws.status, STATUS_WORKSPACE_TOO_SMALL);
