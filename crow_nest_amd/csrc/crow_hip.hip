@@ -28,24 +28,28 @@ struct FnEntry {
     // a twin of `stub` for strips of exactly two groups (K in 257 .. 512), started in its place when the launch dimensions say
     // so; its dynamic LDS is the zero area and ONE staging area (per block, not per wave)
     const void* short_k_stub;
+    bool takes_geo;  // the launcher appends the model geometry (crow_hip_set_geo) by value, last
 };
 
-#define CROW_FN(name, nargs) {#name, (const void*)&name, nargs, 0u, 0, 16, 0, 1, false}
+#define CROW_FN(name, nargs) {#name, (const void*)&name, nargs, 0u, 0, 16, 0, 1, false, nullptr, false}
+#define CROW_FN_GEO(name, nargs) {#name, (const void*)&name, nargs, 0u, 0, 16, 0, 1, false, nullptr, true}
 // NR tensors per block, bodies for 1 .. MMAX activation rows, bf16 or f32 activations
 // (the bodies for several rows need more registers than a block of sixteen waves leaves each: they run in blocks of eight)
 #define CROW_GEMV(name, nargs, NR, MMAX, XBF16) \
-    {#name, (const void*)&name, nargs, 0u, NR, MMAX > 1 ? 8 : 16, crow::crow_gemv_lds_per_wave(MMAX, XBF16), MMAX > 1 ? (XBF16 ? CROW_MULTI_STRIPS_BF16 : CROW_MULTI_STRIPS) : 1, true}
+    {#name, (const void*)&name, nargs, 0u, NR, MMAX > 1 ? 8 : 16, crow::crow_gemv_lds_per_wave(MMAX, XBF16), MMAX > 1 ? (XBF16 ? CROW_MULTI_STRIPS_BF16 : CROW_MULTI_STRIPS) : 1, true, nullptr, false}
+#define CROW_GEMV_GEO(name, nargs, NR, MMAX, XBF16) \
+    {#name, (const void*)&name, nargs, 0u, NR, 16, crow::crow_gemv_lds_per_wave(MMAX, XBF16), 1, true, nullptr, true}
 const FnEntry g_table[] = {
     CROW_GEMV(gemv_nvfp4_w, 6, 1, 1, false),       CROW_GEMV(gemv_nvfp4_w_bf16, 6, 1, 1, true),  CROW_GEMV(gemv_nvfp4_w_argmax, 7, 1, 1, false),
     CROW_GEMV(gemv_nvfp4_gu, 8, 2, 1, false),      CROW_GEMV(gemv_nvfp4_gu_bf16, 8, 2, 1, true),
     CROW_GEMV(gemv_nvfp4_wm, 7, 1, 4, false),      CROW_GEMV(gemv_nvfp4_gum, 9, 2, 4, false),
     CROW_GEMV(gemv_nvfp4_wm_bf16, 7, 1, 4, true),  CROW_GEMV(gemv_nvfp4_gum_bf16, 9, 2, 4, true), CROW_GEMV(gemv_fp4, 6, 1, 1, false),
     CROW_GEMV(gemv_fp4_b, 7, 1, 4, false),         CROW_GEMV(gemv_fp4_b1k, 7, 1, 4, false),      CROW_GEMV(gemv_fp4_bs, 8, 1, 4, false),
-    CROW_GEMV(gemv_fp4_ptrb, 8, 1, 1, false),      CROW_GEMV(moe_gate_up_silu, 8, 2, 1, false),  CROW_GEMV(moe_down_combine, 7, 1, 1, false),
-    CROW_GEMV(moe_route_gate_up_silu, 11, 2, 1, false), CROW_GEMV(moe_gate_up_silu_grouped, 11, 2, 4, false),
-    {"moe_down_grouped", (const void*)&moe_down_grouped, 9, 0u, 1, 8, crow::crow_gemv_lds_per_wave(4, false), CROW_MULTI_STRIPS, true, (const void*)&moe_down_grouped_short_k},
-    CROW_FN(moe_group, 6),
-    CROW_FN(router_top10, 10),     CROW_FN(silu_mul_combo, 3),      CROW_FN(acc_combo, 3),
+    CROW_GEMV(gemv_fp4_ptrb, 8, 1, 1, false),      CROW_GEMV(moe_gate_up_silu, 8, 2, 1, false),  CROW_GEMV_GEO(moe_down_combine, 7, 1, 1, false),
+    CROW_GEMV_GEO(moe_route_gate_up_silu, 11, 2, 1, false), CROW_GEMV(moe_gate_up_silu_grouped, 11, 2, 4, false),
+    {"moe_down_grouped", (const void*)&moe_down_grouped, 9, 0u, 1, 8, crow::crow_gemv_lds_per_wave(4, false), CROW_MULTI_STRIPS, true, (const void*)&moe_down_grouped_short_k, false},
+    CROW_FN_GEO(moe_group, 6),
+    CROW_FN_GEO(router_top10, 10), CROW_FN_GEO(silu_mul_combo, 3),  CROW_FN_GEO(acc_combo, 3),
     CROW_FN(argmax_k, 3),          CROW_FN(dequant_fp4_flat, 4),    CROW_FN(repack_nvfp4, 4),
     CROW_FN(unpack_nvfp4, 4),      CROW_FN(dequant_nvfp4_tiled, 5),
     // shared-X GEMM blocks: two staged X tiles of MT rows x 528 bytes
@@ -72,7 +76,7 @@ struct State {
     crow::Workspace ws_static{};  // the same roles inside `scratch`, through the device address crow_hip_init asked for
     int* scalars = nullptr;  // two device words for the library's own launches (rows, k_dim)
     char name[256] = {0};
-    int geo_topk = 0;  // host copy of the routed geometry (crow_hip_set_geo), for launch shapes
+    crow::Geo model{0, 0, 0, 0};  // the routed geometry (crow_hip_set_geo): appended by value to the kernels that take it
     size_t lds_cap = 64u * 1024u;  // most LDS one workgroup may take on this device
 } g;
 
@@ -144,6 +148,8 @@ int launch_entry(const FnEntry* e, dim3 grid, dim3 block, const uint64_t* vals, 
         args[na++] = (void*)&geo;
     }
     if (e->takes_ws) args[na++] = (void*)&ws_arg;
+    crow::Geo model_arg = g.model;
+    if (e->takes_geo) args[na++] = (void*)&model_arg;
     const void* stub = e->stub;
     if (e->short_k_stub != nullptr) {
         const unsigned pairs = (unsigned)geo & 0xFFFFFu;
@@ -203,8 +209,6 @@ int crow_hip_init(int device) {
     if ((e = hipMemset(ws.counters, 0, COUNTER_WORDS * sizeof(unsigned))) != hipSuccess) return fail(e);
     ws.status = ws.counters + COUNTER_SLOTS;
     if ((e = hipMemcpyToSymbol(HIP_SYMBOL(crow::g_ws), &ws, sizeof ws)) != hipSuccess) return fail(e);
-    crow::Geo geo{0, 0, 0, 0};
-    if ((e = hipMemcpyToSymbol(HIP_SYMBOL(crow::g_geo), &geo, sizeof geo)) != hipSuccess) return fail(e);
     // a GEMV block of 16 waves, and the GEMM's two staged X tiles, need more dynamic LDS than the default per-block limit
     for (int i = 0; i < g_table_n; i++) {
         size_t most = g_table[i].lds_fixed;
@@ -307,11 +311,8 @@ int crow_hip_set_geo(int experts, int topk, int hidden, int inter) {
     if (experts < 0 || topk < 0 || hidden < 0 || inter < 0) return CROW_ERR_BAD_ARGUMENT;
     // what the routing kernels take: no routed experts at all, or a power of two of them in 64..1024 with 1..16 picks
     if (experts != 0 && (experts < 64 || experts > 1024 || (experts & (experts - 1)) != 0 || topk < 1 || topk > 16)) return CROW_ERR_GEO;
-    crow::Geo geo{experts, topk, hidden, inter};
-    hipError_t e = hipMemcpyToSymbolAsync(HIP_SYMBOL(crow::g_geo), &geo, sizeof geo, 0, hipMemcpyHostToDevice, g.stream);
-    if (e != hipSuccess) return (int)e;
-    if ((e = hipStreamSynchronize(g.stream)) != hipSuccess) return (int)e;
-    g.geo_topk = topk;
+    // host state only: launches started from now on carry it by value (nothing is copied, nothing waits)
+    g.model = crow::Geo{experts, topk, hidden, inter};
     return CROW_OK;
 }
 
@@ -394,8 +395,8 @@ int crow_hip_launch_dims_split(const char* name, uint32_t rows, uint32_t k_dim, 
         const bool verify = strcmp(name, "gemv_nvfp4_wm") == 0 || strcmp(name, "gemv_nvfp4_gum") == 0 || strcmp(name, "gemv_nvfp4_wm_bf16") == 0 ||
                             strcmp(name, "gemv_nvfp4_gum_bf16") == 0;
         if (down_combine) {  // rows = hidden; one wave per picked expert, every wave all columns of its strip
-            if (g.geo_topk < 1 || g.geo_topk > 16) return CROW_ERR_GEO;
-            *out = crow_dims{strips, pairs | (1u << 24), z, 64u * (uint32_t)g.geo_topk};
+            if (g.model.topk < 1 || g.model.topk > 16) return CROW_ERR_GEO;
+            *out = crow_dims{strips, pairs | (1u << 24), z, 64u * (uint32_t)g.model.topk};
             return CROW_OK;
         }
         if (strcmp(name, "moe_down_grouped") == 0 && groups == 2) {  // short K: 4 waves per block, each a run of CROW_SHORTK_STRIPS strips

@@ -54,12 +54,13 @@ struct Workspace {
 };
 __device__ Workspace g_ws;
 
-// Model geometry the reference bakes into its kernel text as CN_* defines
-// (engine/src/kernels.rs:5040-5125); here it is a device struct written by crow_hip_set_geo.
+// Model geometry the reference bakes into its kernel text as CN_* defines (engine/src/kernels.rs:5040-5125).  Here the
+// kernels that need it take it BY VALUE as their last argument, which callers never pass: the launcher appends what
+// crow_hip_set_geo last recorded on the host.  No device-side state, so setting it needs no copy and no synchronisation, and
+// a launch captured into a graph keeps the geometry it was captured with.
 struct Geo {
     int experts, topk, hidden, inter;
 };
-__device__ Geo g_geo;
 
 enum StatusBits : unsigned { STATUS_WORKSPACE_TOO_SMALL = 1u, STATUS_BAD_SHAPE = 2u, STATUS_BAD_GEO = 4u };
 

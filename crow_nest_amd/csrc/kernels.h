@@ -289,12 +289,12 @@ extern "C" __global__ void __launch_bounds__(1024) moe_gate_up_silu(const unsign
 extern "C" __global__ void __launch_bounds__(1024) moe_down_combine(const unsigned long long* __restrict__ ptrs, const float* __restrict__ h,
                                                                     const float* __restrict__ gs_ptr, const float* __restrict__ rw,
                                                                     float* __restrict__ y, const int* __restrict__ k_dim_p,
-                                                                    const int* __restrict__ rows_p, int geo, const Workspace ws) {
+                                                                    const int* __restrict__ rows_p, int geo, const Workspace ws, const Geo model) {
     ENTER(ptrs, h, gs_ptr, rw, y, k_dim_p, rows_p, geo);
     const int pairs = geo & 0xFFFFF;
     constexpr int AREA = crow_gemv_lds_per_wave(1, false);
     const int topk = block_threads() >> 6;
-    if (topk != g_geo.topk || topk > 16) {
+    if (topk != model.topk || topk > 16) {
         if (threadIdx.x == 0) atomicOr(ws.status, STATUS_BAD_GEO);
         return;
     }

@@ -264,14 +264,15 @@ __device__ __forceinline__ void router_dispatch(int E, const float* __restrict__
 // reference: router_top10, engine/src/kernels.rs:3109-3184.  grid (T), block 64: one wavefront per
 // token.  The softmax denominator is added in the reference's halving-tree order (slots first, then
 // lanes), so weights match an E-thread tree.  Ties go to the lowest expert id.
-// E = g_geo.experts (power of two, 64..1024), K = g_geo.topk <= 16.
+// E = model.experts (power of two, 64..1024), K = model.topk <= 16 (the geometry the launcher appends).
 // bitmap / cold_mask / counters / sel_counts / table / *_ptrs may be null (skipped).
 extern "C" __global__ void __launch_bounds__(64) router_top10(const float* __restrict__ logits, const unsigned int* __restrict__ bitmap,
                                                               int* __restrict__ ids, float* __restrict__ wts,
                                                               unsigned long long* __restrict__ gu_ptrs, unsigned long long* __restrict__ dn_ptrs,
                                                               const unsigned long long* __restrict__ table, unsigned int* __restrict__ cold_mask,
-                                                              unsigned long long* __restrict__ counters, unsigned long long* __restrict__ sel_counts) {
-    const int E = g_geo.experts, K = g_geo.topk;
+                                                              unsigned long long* __restrict__ counters, unsigned long long* __restrict__ sel_counts,
+                                                              const Geo model) {
+    const int E = model.experts, K = model.topk;
     if (E < 64 || E > 1024 || (E & (E - 1)) != 0 || K < 1 || K > 16 || K > E || block_threads() != 64) {
         if (threadIdx.x == 0) atomicOr(g_ws.status, STATUS_BAD_GEO);
         return;
@@ -288,11 +289,12 @@ extern "C" __global__ void __launch_bounds__(1024) moe_route_gate_up_silu(const 
                                                                           const float* __restrict__ x, const float* __restrict__ gs_ptr,
                                                                           float* __restrict__ h, int* __restrict__ ids, float* __restrict__ wts,
                                                                           unsigned long long* __restrict__ dn_ptrs, const int* __restrict__ k_dim_p,
-                                                                          const int* __restrict__ x_stride_p, const int* __restrict__ inter_p, int geo, const Workspace ws) {
+                                                                          const int* __restrict__ x_stride_p, const int* __restrict__ inter_p, int geo, const Workspace ws,
+                                                                          const Geo model) {
     ENTER(logits, table, x, gs_ptr, h, ids, wts, dn_ptrs, k_dim_p, x_stride_p, inter_p, geo);
     const int pairs = geo & 0xFFFFF;
     __shared__ unsigned long long s_slab;
-    const int E = g_geo.experts, K = g_geo.topk;
+    const int E = model.experts, K = model.topk;
     if (E < 64 || E > 1024 || (E & (E - 1)) != 0 || K < 1 || K > 16 || K > E || table == nullptr) {
         if (threadIdx.x == 0) atomicOr(ws.status, STATUS_BAD_GEO);
         return;
@@ -344,15 +346,16 @@ extern "C" __global__ void __launch_bounds__(1024) moe_route_gate_up_silu(const 
 // tiles[t] = (expert, first position in perm, combos, 0), experts ascending; *n_tiles.
 // A counting sort over chunks of 64 combos (one wavefront pass each): per-chunk histograms, a running sum per expert
 // over the chunks, a block scan over the experts, then every chunk ranks its combos among equal experts with ballots.
-// n <= 4096, E = g_geo.experts <= 1024, E * ceil(n / 64) <= 16384.  grid 1, block 1024.
+// n <= 4096, E = model.experts <= 1024, E * ceil(n / 64) <= 16384.  grid 1, block 1024.
 #define CROW_MOE_GROUP_MAX_COMBOS 4096
 #define CROW_MOE_GROUP_HIST 16384
 extern "C" __global__ void __launch_bounds__(1024) moe_group(const int* __restrict__ ids, const int* __restrict__ n_p, int* __restrict__ perm,
-                                                             int4* __restrict__ tiles, int* __restrict__ n_tiles, const int* __restrict__ max_tiles_p) {
+                                                             int4* __restrict__ tiles, int* __restrict__ n_tiles, const int* __restrict__ max_tiles_p,
+                                                             const Geo model) {
     __shared__ unsigned short s_hist[CROW_MOE_GROUP_HIST];  // [chunk][expert]: count, then the count in earlier chunks
     __shared__ int s_off[1024], s_tile[1024];
     __shared__ int s_bad;
-    const int n = *n_p, E = g_geo.experts, max_tiles = *max_tiles_p, t = (int)threadIdx.x;
+    const int n = *n_p, E = model.experts, max_tiles = *max_tiles_p, t = (int)threadIdx.x;
     const int chunks = (n + 63) >> 6;
     if (block_threads() != 1024 || n < 0 || n > CROW_MOE_GROUP_MAX_COMBOS || E < 1 || E > 1024 || E * chunks > CROW_MOE_GROUP_HIST) {
         if (t == 0) {
@@ -449,19 +452,19 @@ extern "C" __global__ void __launch_bounds__(1024) moe_group(const int* __restri
     }
 }
 
-// reference: silu_mul_combo, engine/src/kernels.rs:1562-1570: [C][2 I] -> [C][I], I = g_geo.inter
-extern "C" __global__ void silu_mul_combo(const float* __restrict__ h1, float* __restrict__ h2, const int* __restrict__ n_p) {
+// reference: silu_mul_combo, engine/src/kernels.rs:1562-1570: [C][2 I] -> [C][I], I = model.inter
+extern "C" __global__ void silu_mul_combo(const float* __restrict__ h1, float* __restrict__ h2, const int* __restrict__ n_p, const Geo model) {
     const int i = (int)(blockIdx.x * blockDim.x + threadIdx.x);
     if (i >= *n_p) return;
-    const int inter = g_geo.inter;
+    const int inter = model.inter;
     const int c = i / inter, j = i % inter;
     h2[i] = silu_mul(h1[(size_t)c * 2 * inter + j], h1[(size_t)c * 2 * inter + inter + j]);
 }
 
 // reference: acc_combo, engine/src/kernels.rs:1583-1592: y[t][c] += sum_j rw[t][j] * x[t K + j][c],
 // j ascending, one rounding per multiply and per add.  grid (ceil(H / 256), T), block 256.
-extern "C" __global__ void acc_combo(const float* __restrict__ x, const float* __restrict__ rw, float* __restrict__ y) {
-    const int H = g_geo.hidden, K = g_geo.topk;
+extern "C" __global__ void acc_combo(const float* __restrict__ x, const float* __restrict__ rw, float* __restrict__ y, const Geo model) {
+    const int H = model.hidden, K = model.topk;
     const int c = (int)(blockIdx.x * blockDim.x + threadIdx.x), t = (int)blockIdx.y;
     if (c >= H) return;
     float acc = 0.0f;

@@ -69,7 +69,11 @@ int crow_hip_function_count(void);
 const char* crow_hip_function_name(int index);
 int crow_hip_function_arg_count(crow_fn_t f);
 
-/* ---- geometry the reference compiles into its kernel text ---- */
+/* ---- geometry the reference compiles into its kernel text ----
+ * Host state only: the launcher hands it BY VALUE to the kernels that need it (router_top10, moe_route_gate_up_silu,
+ * moe_down_combine, moe_group, silu_mul_combo, acc_combo), so the call copies nothing to the device and waits for nothing,
+ * launches already queued keep the geometry they were started with, and a launch captured into a graph keeps the
+ * geometry it was captured with.  A process that serves two geometries sets the one it needs before each group of launches. */
 int crow_hip_set_geo(int experts, int topk, int hidden, int inter);
 
 /* ---- launch ---- */

@@ -484,6 +484,33 @@ def test_router_other_geometries_and_ties(eng, experts, topk):
     assert ids_ref[2].tolist() == list(range(topk))
 
 
+def test_two_geometries_interleaved_without_a_wait(eng):
+    """The geometry rides on every launch by value: routing launches of two geometries queued alternately on one stream,
+    with nothing waited for in between, each use their own."""
+    from crow_nest_amd.kernels import KernelGeo, launch_v, set_geo
+    geos = [KernelGeo(experts=64, topk=4, hidden=2048, inter=512), KernelGeo(experts=512, topk=10, hidden=2048, inter=512)]
+    g = np.random.default_rng(99)
+    logits = [g.standard_normal((5, ge.experts)).astype(np.float32) for ge in geos for _ in range(3)]
+    devs = [_dev(l) for l in logits]
+    outs = []
+    try:
+        order = [0, 3, 1, 4, 2, 5]  # the data is A, A, A, B, B, B; launched A, B, A, B, A, B
+        for i in order:
+            ge = geos[i // 3]
+            set_geo(ge)
+            ids = torch.empty((5, ge.topk), dtype=torch.int32, device="cuda")
+            wts = torch.empty((5, ge.topk), dtype=torch.float32, device="cuda")
+            launch_v(eng.k.f("router_top10"), 5, 1, 1, 64, [devs[i].data_ptr(), 0, ids.data_ptr(), wts.data_ptr(), 0, 0, 0, 0, 0, 0])
+            outs.append((i, ids, wts))
+        eng.check()
+    finally:
+        set_geo(eng.geo)
+    for i, ids, wts in outs:
+        ids_ref, w_ref = orc.router_topk(logits[i], geos[i // 3].topk)
+        assert np.array_equal(ids.cpu().numpy(), ids_ref), i
+        assert np.allclose(wts.cpu().numpy(), w_ref, rtol=2e-6, atol=0), i
+
+
 @pytest.mark.parametrize("t", [1, 4])
 def test_moe_layer_both_launch_sequences(eng, t):
     from crow_nest_amd.engine import MoeW, expert_table
