@@ -25,9 +25,9 @@ struct FnEntry {
     int lds_per_wave;
     int ns;  // adjacent 16-row strips per block (kernels for several activation rows: CROW_MULTI_STRIPS), else 1
     bool takes_ws;  // the launcher appends the scratch descriptor (every kernel of the GEMV family)
-    // a twin of `stub` for strips of exactly two groups (K in 257 .. 512), started in its place when the launch dimensions say
-    // so; its dynamic LDS is the zero area and ONE staging area (per block, not per wave)
-    const void* short_k_stub;
+    // a twin of `stub` for strips of two to eight groups that one wave walks alone, started in its place when the launch
+    // dimensions say so; its dynamic LDS is the zero area and one staging area of twelve rows per GROUP (per block, not per wave)
+    const void* tile_stub;
     bool takes_geo;  // the launcher appends the model geometry (crow_hip_set_geo) by value, last
 };
 
@@ -46,8 +46,9 @@ const FnEntry g_table[] = {
     CROW_GEMV(gemv_nvfp4_wm_bf16, 7, 1, 4, true),  CROW_GEMV(gemv_nvfp4_gum_bf16, 9, 2, 4, true), CROW_GEMV(gemv_fp4, 6, 1, 1, false),
     CROW_GEMV(gemv_fp4_b, 7, 1, 4, false),         CROW_GEMV(gemv_fp4_b1k, 7, 1, 4, false),      CROW_GEMV(gemv_fp4_bs, 8, 1, 4, false),
     CROW_GEMV(gemv_fp4_ptrb, 8, 1, 1, false),      CROW_GEMV(moe_gate_up_silu, 8, 2, 1, false),  CROW_GEMV_GEO(moe_down_combine, 7, 1, 1, false),
-    CROW_GEMV_GEO(moe_route_gate_up_silu, 11, 2, 1, false), CROW_GEMV(moe_gate_up_silu_grouped, 11, 2, 4, false),
-    {"moe_down_grouped", (const void*)&moe_down_grouped, 9, 0u, 1, 8, crow::crow_gemv_lds_per_wave(4, false), CROW_MULTI_STRIPS, true, (const void*)&moe_down_grouped_short_k, false},
+    CROW_GEMV_GEO(moe_route_gate_up_silu, 11, 2, 1, false),
+    {"moe_gate_up_silu_grouped", (const void*)&moe_gate_up_silu_grouped, 11, 0u, 2, 8, crow::crow_gemv_lds_per_wave(4, false), CROW_MULTI_STRIPS, true, (const void*)&moe_gate_up_silu_grouped_tile, false},
+    {"moe_down_grouped", (const void*)&moe_down_grouped, 9, 0u, 1, 8, crow::crow_gemv_lds_per_wave(4, false), CROW_MULTI_STRIPS, true, (const void*)&moe_down_grouped_tile, false},
     CROW_FN_GEO(moe_group, 6),
     CROW_FN_GEO(router_top10, 10), CROW_FN_GEO(silu_mul_combo, 3),  CROW_FN_GEO(acc_combo, 3),
     CROW_FN(argmax_k, 3),          CROW_FN(dequant_fp4_flat, 4),    CROW_FN(repack_nvfp4, 4),
@@ -116,6 +117,13 @@ const FnEntry* entry_of(crow_fn_t f) {
 }
 
 
+// Groups per strip if the grouped expert kernels take their twin for K / 64 = pairs (strips of two to eight groups that one
+// wave walks alone in the launch shapes chosen below: up to 7 groups for one tensor, 10 - here 8 - per tensor for two), else 0.
+unsigned tile_groups(int nr, unsigned pairs) {
+    const unsigned groups = (pairs + CROW_GROUP_PAIRS - 1) / CROW_GROUP_PAIRS;
+    return groups >= 2 && groups <= (nr == 2 ? (unsigned)CROW_TILE_MAX_GROUPS : 7u) ? groups : 0u;
+}
+
 // The launch dimensions of the GEMV family carry the problem in `gy` (crow_hip_launch_dims writes it, callers pass it on
 // unchanged): bits 0..19 = K / 64, bits 20..23 = activation rows of the last token group (0 = not given), bits 24..31 = S, the
 // number of column slices per strip.  The real grid is (gx, S, gz); the low 24 bits reach the kernel by value.
@@ -132,32 +140,36 @@ int launch_entry(const FnEntry* e, dim3 grid, dim3 block, const uint64_t* vals, 
     size_t lds = e->lds_fixed;
     int geo = 0;
     crow::Workspace ws_arg = ws;
+    const void* stub = e->stub;
     if (e->nr != 0) {
         const unsigned word = grid.y;
-        const int pairs = (int)(word & 0xFFFFFu), slices = (int)(word >> 24) == 0 ? 1 : (int)(word >> 24);
+        const int pairs = (int)(word & 0xFFFFFu);
         const int waves = (int)(block.x / 64), wpt = waves / e->nr;
         if (pairs == 0 || wpt == 0) return CROW_ERR_BAD_ARGUMENT;
-        lds = (size_t)CROW_GEMV_ZERO_BYTES + (size_t)waves * (size_t)e->lds_per_wave;
+        if (e->tile_stub != nullptr && tile_groups(e->nr, (unsigned)pairs) != 0 && block.x <= 512) {
+            // the twin for strips that one wave walks alone: strips per wave ride where S sits (such a strip is never cut into
+            // slices), and the kernel takes the whole word; one staging area per group and block
+            if ((word >> 24) == 0) return CROW_ERR_BAD_ARGUMENT;
+            stub = e->tile_stub;
+            geo = (int)word;
+            grid.y = 1;
+            lds = (size_t)CROW_GEMV_ZERO_BYTES + (size_t)tile_groups(e->nr, (unsigned)pairs) * (size_t)(e->lds_per_wave / 2);
+        } else {
+            const int slices = (int)(word >> 24) == 0 ? 1 : (int)(word >> 24);
+            lds = (size_t)CROW_GEMV_ZERO_BYTES + (size_t)waves * (size_t)e->lds_per_wave;
+            // a split launch must fit the scratch memory it is given (the kernels check again and report through the status word)
+            if (slices > 1 && ((unsigned long long)grid.x * grid.z * (unsigned)slices * (unsigned)(e->nr * e->ns) * 64ull > ws.partial_floats ||
+                               (unsigned long long)grid.x * grid.z > ws.counter_slots))
+                return CROW_ERR_WORKSPACE;
+            geo = (int)(word & 0xFFFFFFu);
+            grid.y = (unsigned)slices;
+        }
         if (lds > g.lds_cap) return CROW_ERR_SHAPE;
-        // a split launch must fit the scratch memory it is given (the kernels check again and report through the status word)
-        if (slices > 1 && ((unsigned long long)grid.x * grid.z * (unsigned)slices * (unsigned)(e->nr * e->ns) * 64ull > ws.partial_floats ||
-                           (unsigned long long)grid.x * grid.z > ws.counter_slots))
-            return CROW_ERR_WORKSPACE;
-        geo = (int)(word & 0xFFFFFFu);
-        grid.y = (unsigned)slices;
         args[na++] = (void*)&geo;
     }
     if (e->takes_ws) args[na++] = (void*)&ws_arg;
     crow::Geo model_arg = g.model;
     if (e->takes_geo) args[na++] = (void*)&model_arg;
-    const void* stub = e->stub;
-    if (e->short_k_stub != nullptr) {
-        const unsigned pairs = (unsigned)geo & 0xFFFFFu;
-        if (pairs > CROW_GROUP_PAIRS && pairs <= 2 * CROW_GROUP_PAIRS && block.x <= 256) {
-            stub = e->short_k_stub;
-            lds = (size_t)CROW_GEMV_ZERO_BYTES + (size_t)e->lds_per_wave;
-        }
-    }
     const bool head = e->stub == (const void*)&gemv_nvfp4_w_argmax;
     // the fused head keeps one key per strip (the kernel checks again and reports through the status word)
     if (head && grid.x > ws.head_words) return CROW_ERR_WORKSPACE;
@@ -218,6 +230,11 @@ int crow_hip_init(int device) {
         }
         if (most > 48 * 1024 &&
             (e = hipFuncSetAttribute(g_table[i].stub, hipFuncAttributeMaxDynamicSharedMemorySize, (int)most)) != hipSuccess)
+            return fail(e);
+        // the twin for short strips stages up to eight groups of twelve rows per block
+        const size_t tile_most = (size_t)CROW_GEMV_ZERO_BYTES + (size_t)CROW_TILE_MAX_GROUPS * (size_t)(g_table[i].lds_per_wave / 2);
+        if (g_table[i].tile_stub != nullptr && tile_most > 48 * 1024 &&
+            (e = hipFuncSetAttribute(g_table[i].tile_stub, hipFuncAttributeMaxDynamicSharedMemorySize, (int)tile_most)) != hipSuccess)
             return fail(e);
     }
     // `scratch` in host code is a stand-in, not a device address: ask for this device's copy once, and use only that
@@ -399,9 +416,14 @@ int crow_hip_launch_dims_split(const char* name, uint32_t rows, uint32_t k_dim, 
             *out = crow_dims{strips, pairs | (1u << 24), z, 64u * (uint32_t)g.model.topk};
             return CROW_OK;
         }
-        if (strcmp(name, "moe_down_grouped") == 0 && groups == 2) {  // short K: 4 waves per block, each a run of CROW_SHORTK_STRIPS strips
-            const uint32_t per_block = 4u * CROW_SHORTK_STRIPS;
-            *out = crow_dims{(strips + per_block - 1) / per_block, pairs | (1u << 24), z, 256};
+        if (e->tile_stub != nullptr && tile_groups(e->nr, pairs) != 0) {
+            // about sixteen records per wave; eight waves per block where the staged rows are large (two blocks per compute unit)
+            // (force_s / force_w: strips per wave / waves per block, for measurements)
+            uint32_t spw = 16u / ((uint32_t)e->nr * groups);
+            if (spw < 1) spw = 1;
+            if (force_s > 0) spw = force_s > 255 ? 255 : force_s;
+            const uint32_t wb = force_w > 0 ? (force_w > 8 ? 8 : force_w) : (groups > 4 ? 8u : 4u), per_block = wb * spw;
+            *out = crow_dims{(strips + per_block - 1) / per_block, pairs | (spw << 24), z, 64u * wb};
             return CROW_OK;
         }
         if (verify && z > 4) return CROW_ERR_SHAPE;

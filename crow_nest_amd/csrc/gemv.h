@@ -543,25 +543,29 @@ struct MultiWalk {
     }
 };
 
-// The walk of a wave over MANY strips of FEW groups (short K: the routed experts' down slabs, K = 512 -> two groups per strip).
-// Walking such strips one block each means tens of thousands of blocks that each stage the same activations, fill a pipeline
-// of two groups and drain it again.  Here the block stages the tile's activations ONCE (all G groups of all M rows; they never
-// change along the walk) and every wave streams a run of consecutive strips - whose groups are one contiguous run of
-// 2304-byte records in memory - through the ring of four, with no activation traffic and no staging inside the loop.  Per
-// strip and activation row the operation sequence is StripWalk's for a strip walked by one wave, so the sums are the same bits.
-//   G   groups per strip, a power of two <= the ring (ring slot J always holds a group J % G)
-template <int M, int G>
-struct ShortKWalk {
-    static_assert(G == 1 || G == 2 || G == 4, "a ring slot's group index is static");
+// The walk of a wave over MANY strips of FEW groups (short K: the routed experts' slabs, K = 2048 / 512 -> eight / two groups
+// per strip).  Walking such strips one block each means tens of thousands of blocks that each stage the same activation rows,
+// fill a pipeline of a few groups and drain it again.  Here the block stages the tile's activation rows ONCE (all groups of all
+// M rows; they never change along the walk) and every wave streams a run of consecutive strips - whose groups are one
+// contiguous run of 2304-byte records in memory - through the ring of four, with no activation traffic, no staging and no
+// register slots for activations inside the loop.  NR = 2: a strip of `gate` is followed by the same strip of `up` (the
+// tensor `up_off` bytes further on) and the two sums leave together.  A strip is walked by this one wave from its first group
+// to its last, which is the operation sequence of StripWalk for a strip that one wave walks alone: the same bits.
+template <int M, int NR>
+struct TileWalk {
     static constexpr int XR = 3 * M, NSET = (3 * M + 3) / 4, SLOT = XR * CROW_GEMV_XROW_BYTES;
     unsigned sc[CROW_GEMV_RING][1];
     u32x4 cd[CROW_GEMV_RING][1][2];
-    lds_p a1[G][NSET], a2[G][NSET];  // this lane's operand addresses in group g's staged rows (or in the zero area)
-    const unsigned char* wl;         // the lane's view of the wave's first record
-    int lane;
+    lds_p a1b[NSET], a2b[NSET];  // this lane's operand addresses in group 0's staged rows (or in the zero area) ...
+    int st1[NSET], st2[NSET];    // ... and what a group further on adds to them (0 for the zero area)
+    // the request side: the next record, its group and its tensor; the multiply side: the same for the next record to multiply
+    const unsigned char* p_next;
+    ptrdiff_t up_off;
+    int groups, gi_req, t_req, gi, t_mul, done, lane;
+    float first_sum;
     float acc[1][M];
 
-    // f32 activations of one group of one row -> three bf16 rows (hi, mid, lo) of the group's staged area; lane = 4 columns
+    // f32 activations of one group of one row -> three bf16 rows (hi, mid, lo) of the group's staged area; a lane = 4 columns
     static __device__ __forceinline__ void stage_row(lds_p staged, int g, int t, f32x4 v, int lane_) {
         unsigned h[4], m[4], l[4];
         split3(v.x, h[0], m[0], l[0]);
@@ -573,9 +577,12 @@ struct ShortKWalk {
         lds_store8(row + CROW_GEMV_XROW_BYTES, __builtin_amdgcn_perm(m[1], m[0], 0x07060302u), __builtin_amdgcn_perm(m[3], m[2], 0x07060302u));
         lds_store8(row + 2 * CROW_GEMV_XROW_BYTES, __builtin_amdgcn_perm(l[1], l[0], 0x07060302u), __builtin_amdgcn_perm(l[3], l[2], 0x07060302u));
     }
-    __device__ __forceinline__ void init(const unsigned char* first_record, lds_p staged, lds_p zero) {
+    __device__ __forceinline__ void init(const unsigned char* first_record, ptrdiff_t up_off_, int groups_, lds_p staged, lds_p zero) {
         lane = lane_id();
-        wl = first_record;
+        p_next = first_record;
+        up_off = up_off_;
+        groups = groups_;
+        gi_req = 0, t_req = 0, gi = 0, t_mul = 0, done = 0, first_sum = 0.0f;
 #pragma unroll
         for (int m = 0; m < M; m++) acc[0][m] = 0.0f;
         // (the operand addressing of StripWalk::init, one staged area per group)
@@ -583,30 +590,47 @@ struct ShortKWalk {
         const bool half_ok = (g >> 1) == (i >> 3);
         const bool second = ((i >> 2) & 1) != 0;
 #pragma unroll
-        for (int s = 0; s < G; s++)
-#pragma unroll
-            for (int q = 0; q < NSET; q++) {
-                const int row = 4 * q + r4;
-                const bool live = half_ok && row < XR;
-                lds_p data = staged + s * SLOT + row * CROW_GEMV_XROW_BYTES + 16 * g;
-                a1[s][q] = (live && !second) ? data : zero + 16 * g;
-                a2[s][q] = (live && second) ? data + 64 : zero + 16 * g;
-            }
+        for (int q = 0; q < NSET; q++) {
+            const int row = 4 * q + r4;
+            const bool live = half_ok && row < XR;
+            lds_p data = staged + row * CROW_GEMV_XROW_BYTES + 16 * g;
+            a1b[q] = (live && !second) ? data : zero + 16 * g;
+            st1[q] = (live && !second) ? SLOT : 0;
+            a2b[q] = (live && second) ? data + 64 : zero + 16 * g;
+            st2[q] = (live && second) ? SLOT : 0;
+        }
     }
+    // requests the wave's next record into slot J
     template <int J>
-    __device__ __forceinline__ void issue_w(int i) {
-        const unsigned char* p = wl + (size_t)i * CROW_GROUP_BYTES;
+    __device__ __forceinline__ void issue_w() {
+        const unsigned char* p = p_next;
         sc[J][0] = stream_load_u32((const unsigned*)p + lane);
         cd[J][0][0] = stream_load_v((const uint4*)(p + CROW_GROUP_SCALE_BYTES) + lane);
         cd[J][0][1] = stream_load_v((const uint4*)(p + CROW_GROUP_SCALE_BYTES + 1024) + lane);
+        p_next += CROW_GROUP_BYTES;
+        if (++gi_req == groups) {  // wave-uniform
+            gi_req = 0;
+            if (NR == 2) {  // gate strip s -> up strip s -> gate strip s + 1
+                p_next += t_req == 0 ? up_off - (ptrdiff_t)groups * CROW_GROUP_BYTES : -up_off;
+                t_req ^= 1;
+            }
+        }
     }
-    // record i sits in slot J: multiply it by its group's staged rows; behind a strip's last group hand the strip's sums to
-    // `emit(strip index within the run, v)` - v in lane l = the dot product of strip row l % 16 with activation row l / 16
+    // the next record sits in slot J: multiply it by its group's staged rows; behind a strip's last group the strip's sums are
+    // closed, and behind the last tensor's `emit(strips finished before, first, last)` - in lane l the dot products of strip
+    // row l % 16 with activation row l / 16, of the first tensor and of the last (one tensor: `last` only)
     template <int J, class Emit>
-    __device__ __forceinline__ void multiply(int i, Emit& emit) {
-        group_multiply<M, false, 1>(sc[J], cd[J], a1[J % G], a2[J % G], acc);
+    __device__ __forceinline__ void multiply(Emit& emit) {
+        lds_p a1[NSET], a2[NSET];
+#pragma unroll
+        for (int q = 0; q < NSET; q++) {
+            a1[q] = a1b[q] + gi * st1[q];
+            a2[q] = a2b[q] + gi * st2[q];
+        }
+        group_multiply<M, false, 1>(sc[J], cd[J], a1, a2, acc);
         __builtin_amdgcn_sched_barrier(0);
-        if (J % G == G - 1) {
+        if (++gi == groups) {  // wave-uniform
+            gi = 0;
             float v = 0.0f;
 #pragma unroll
             for (int m = 0; m < M; m++) {  // (StripWalk::finish)
@@ -618,51 +642,55 @@ struct ShortKWalk {
                 v = (lane >> 4) == m ? o : v;
                 acc[0][m] = 0.0f;
             }
-            emit(i / G, v);
+            if (NR == 2 && t_mul == 0) {
+                first_sum = v;
+                t_mul = 1;
+            } else {
+                emit(done, first_sum, v);
+                done++;
+                t_mul = 0;
+            }
         }
     }
-    // `count` records (a multiple of G) from the wave's first one; `mid` runs once, after the first loads have left: the
-    // block's staging and its barrier
+    // `count` records (whole strips of every tensor) from the wave's first one; `mid` runs once, after the first loads have
+    // left: the block's staging and its barrier
     template <class Mid, class Emit>
     __device__ __forceinline__ void go(int count, Mid mid, Emit emit) {
         const int nq = count >> 2, r = count & 3;
         if (nq > 0) {
-            issue_w<0>(0);
-            issue_w<1>(1);
-            issue_w<2>(2);
-            issue_w<3>(3);
+            issue_w<0>();
+            issue_w<1>();
+            issue_w<2>();
+            issue_w<3>();
             mid();
-            int q = 0;
-            for (; q + 1 < nq; q++) {
-                const int i0 = 4 * q;
-                multiply<0>(i0, emit);
-                issue_w<0>(i0 + 4);
-                multiply<1>(i0 + 1, emit);
-                issue_w<1>(i0 + 5);
-                multiply<2>(i0 + 2, emit);
-                issue_w<2>(i0 + 6);
-                multiply<3>(i0 + 3, emit);
-                issue_w<3>(i0 + 7);
+            for (int q = 0; q + 1 < nq; q++) {
+                multiply<0>(emit);
+                issue_w<0>();
+                multiply<1>(emit);
+                issue_w<1>();
+                multiply<2>(emit);
+                issue_w<2>();
+                multiply<3>(emit);
+                issue_w<3>();
             }
-            const int i0 = 4 * q;
-            multiply<0>(i0, emit);
-            if (r > 0) issue_w<0>(i0 + 4);
-            multiply<1>(i0 + 1, emit);
-            if (r > 1) issue_w<1>(i0 + 5);
-            multiply<2>(i0 + 2, emit);
-            if (r > 2) issue_w<2>(i0 + 6);
-            multiply<3>(i0 + 3, emit);
-            if (r > 0) multiply<0>(i0 + 4, emit);
-            if (r > 1) multiply<1>(i0 + 5, emit);
-            if (r > 2) multiply<2>(i0 + 6, emit);
+            multiply<0>(emit);
+            if (r > 0) issue_w<0>();
+            multiply<1>(emit);
+            if (r > 1) issue_w<1>();
+            multiply<2>(emit);
+            if (r > 2) issue_w<2>();
+            multiply<3>(emit);
+            if (r > 0) multiply<0>(emit);
+            if (r > 1) multiply<1>(emit);
+            if (r > 2) multiply<2>(emit);
         } else {
-            if (r > 0) issue_w<0>(0);
-            if (r > 1) issue_w<1>(1);
-            if (r > 2) issue_w<2>(2);
+            if (r > 0) issue_w<0>();
+            if (r > 1) issue_w<1>();
+            if (r > 2) issue_w<2>();
             mid();
-            if (r > 0) multiply<0>(0, emit);
-            if (r > 1) multiply<1>(1, emit);
-            if (r > 2) multiply<2>(2, emit);
+            if (r > 0) multiply<0>(emit);
+            if (r > 1) multiply<1>(emit);
+            if (r > 2) multiply<2>(emit);
         }
     }
 };
@@ -870,18 +898,18 @@ __device__ __forceinline__ void gemv_body(const GemvArgs& a, unsigned z, lds_p l
     }
 }
 
-// The body of a short-K product (ShortKWalk): grid.x blocks of W waves, every wave a run of CROW_SHORTK_STRIPS consecutive
-// strips of the tensor, all M activation rows staged once per block.  `lds`: the zero area, then G x 3 M staged rows.
-#ifndef CROW_SHORTK_STRIPS
-#define CROW_SHORTK_STRIPS 8
-#endif
-template <int M, int G>
-__device__ __forceinline__ void short_k_body(const GemvArgs& a, lds_p lds, const Workspace& ws) {
-    typedef ShortKWalk<M, G> Walk;
+// The body of a product over strips of few groups (TileWalk): grid.x blocks of W waves, every wave a run of `spw` consecutive
+// strips (of each of the NR tensors), all M activation rows staged once per block.  `lds`: the zero area, then one area of
+// 3 M staged rows per group.  Strips of at most CROW_TILE_MAX_GROUPS groups.
+#define CROW_TILE_MAX_GROUPS 8
+template <int M, int NR, int EPI>
+__device__ __forceinline__ void tile_body(const GemvArgs& a, int spw, lds_p lds, const Workspace& ws) {
+    typedef TileWalk<M, NR> Walk;
     const int lane = lane_id();
     const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6)), waves = block_threads() >> 6;
     const int k_dim = a.pairs * CROW_PAIR_COLS;
-    const int strip0 = ((int)blockIdx.x * waves + wave) * CROW_SHORTK_STRIPS;
+    const int groups = (a.pairs + CROW_GROUP_PAIRS - 1) / CROW_GROUP_PAIRS;
+    const int strip0 = ((int)blockIdx.x * waves + wave) * spw;
     size_t xoff[M];
     int yrow[M];
 #pragma unroll
@@ -899,13 +927,13 @@ __device__ __forceinline__ void short_k_body(const GemvArgs& a, lds_p lds, const
     // a grid that does not cover the tensor is refused
     const int strips = (*a.rows_p + CROW_STRIP_ROWS - 1) / CROW_STRIP_ROWS;
     const int left = strips - strip0;
-    const int n_strips = left < 0 ? 0 : (left < CROW_SHORTK_STRIPS ? left : CROW_SHORTK_STRIPS);
-    const bool covered = (long long)gridDim.x * waves * CROW_SHORTK_STRIPS >= (long long)strips;
+    const int n_strips = left < 0 ? 0 : (left < spw ? left : spw);
+    const bool covered = (long long)gridDim.x * waves * spw >= (long long)strips && groups <= CROW_TILE_MAX_GROUPS && spw >= 1;
     lds_p zero = lds, staged = lds + CROW_GEMV_ZERO_BYTES;
     Walk walk;
-    walk.init(a.w[0] + (size_t)strip0 * G * CROW_GROUP_BYTES, staged, zero);
+    walk.init(a.w[0] + (size_t)strip0 * groups * CROW_GROUP_BYTES, NR == 2 ? a.w[1] - a.w[0] : 0, groups, staged, zero);
     int rows = 0;
-    float gs = 0.0f;
+    float gs0 = 0.0f, gs1 = 0.0f;
     bool ok = true;
     auto mid = [&]() {
         for (int o = 16 * (int)threadIdx.x; o < CROW_GEMV_ZERO_BYTES; o += 16 * (waves << 6)) lds_store16(zero + o, 0, 0, 0, 0);
@@ -913,15 +941,16 @@ __device__ __forceinline__ void short_k_body(const GemvArgs& a, lds_p lds, const
 #pragma unroll
         for (int t = 0; t < M; t++)
 #pragma unroll
-            for (int g = 0; g < G; g++) {
-                if ((t * G + g) % waves != wave) continue;  // wave-uniform
+            for (int g = 0; g < CROW_TILE_MAX_GROUPS; g++) {
+                if (g >= groups || (t * CROW_TILE_MAX_GROUPS + g) % waves != wave) continue;  // wave-uniform
                 const int col = g * CROW_GROUP_COLS + 4 * lane;
                 f32x4 v = {0.f, 0.f, 0.f, 0.f};
                 if (col < k_dim) v = *(const f32x4*)((const float*)a.x + xoff[t] + col);
                 Walk::stage_row(staged, g, t, v, lane);
             }
         rows = *a.rows_p;
-        gs = a.gs[0][0];
+        gs0 = a.gs[0][0];
+        gs1 = a.gs[NR - 1][0];
         ok = covered && *a.k_dim_p == k_dim && (a.count_p == nullptr || *a.count_p == a.count_expect);
         __syncthreads();
     };
@@ -930,11 +959,15 @@ __device__ __forceinline__ void short_k_body(const GemvArgs& a, lds_p lds, const
 #pragma unroll
     for (int m = 1; m < M; m++)
         if (mo == m) yr = yrow[m];
-    auto emit = [&](int s, float v) {
+    auto emit = [&](int s, float first, float last) {
         const int row = (strip0 + s) * CROW_STRIP_ROWS + n;
-        if (ok && mo < M && row < rows) a.y[(size_t)yr * (a.y_stride != 0 ? a.y_stride : (size_t)rows) + row] = v * gs;
+        if (ok && mo < M && row < rows) {
+            const size_t o = (size_t)yr * (a.y_stride != 0 ? a.y_stride : (size_t)rows) + row;
+            if (EPI == EPI_SCALE) a.y[o] = last * gs0;
+            else a.y[o] = silu_mul(first * gs0, last * gs1);
+        }
     };
-    walk.go(n_strips * G, mid, emit);
+    walk.go(covered ? n_strips * NR * groups : 0, mid, emit);
     if (!ok && threadIdx.x == 0) atomicOr(ws.status, STATUS_BAD_SHAPE);
 }
 

@@ -385,14 +385,46 @@ extern "C" __global__ void __launch_bounds__(512) moe_down_grouped(const int4* _
     a.row_map = perm + tl.y, a.x_div = 1;
     gemv_m_dispatch<1, false, EPI_SCALE>(a, tl.z, blockIdx.z, LDS, ws);
 }
-// The same for strips of two groups (K in 257 .. 512: this model's down slabs), which the launcher starts in place of the
-// kernel above whenever the launch dimensions say so (one table entry, one name): every wave streams a run of strips against
-// activations staged once per block (gemv.h: ShortKWalk); crow_hip_launch_dims sizes grid.x for it.  Same bits.
-extern "C" __global__ void __launch_bounds__(256) moe_down_grouped_short_k(const int4* __restrict__ tiles, const int* __restrict__ n_tiles_p,
-                                                                            const int* __restrict__ perm, const unsigned long long* __restrict__ table,
-                                                                            const float* __restrict__ h, const float* __restrict__ gs_ptr,
-                                                                            float* __restrict__ eo, const int* __restrict__ k_dim_p,
-                                                                            const int* __restrict__ rows_p, int geo, const Workspace ws) {
+// The two kernels above for strips of two to eight groups that one wave walks alone (K in 257 .. 2048 for gate|up, .. 1792 for
+// down: this model's slabs), which the launcher starts in their place whenever the launch dimensions say so (one table entry,
+// one name each): a block stages the tile's activation rows once and every wave streams runs of strips (gemv.h: TileWalk);
+// crow_hip_launch_dims sizes the grid for it.  Here bits 24..31 of the geometry word = strips per wave.  Same bits.
+#define CROW_TILE_DISPATCH(NR, EPI)                                      \
+    switch (tl.z) {                                                      \
+        case 1: tile_body<1, NR, EPI>(a, (geo >> 24) & 0xFF, LDS, ws); break; \
+        case 2: tile_body<2, NR, EPI>(a, (geo >> 24) & 0xFF, LDS, ws); break; \
+        case 3: tile_body<3, NR, EPI>(a, (geo >> 24) & 0xFF, LDS, ws); break; \
+        case 4: tile_body<4, NR, EPI>(a, (geo >> 24) & 0xFF, LDS, ws); break; \
+        default:                                                         \
+            if (threadIdx.x == 0) atomicOr(ws.status, STATUS_BAD_SHAPE); \
+    }
+extern "C" __global__ void __launch_bounds__(512) moe_gate_up_silu_grouped_tile(const int4* __restrict__ tiles, const int* __restrict__ n_tiles_p,
+                                                                                  const int* __restrict__ perm, const unsigned long long* __restrict__ table,
+                                                                                  const float* __restrict__ x, const float* __restrict__ gs_ptr,
+                                                                                  float* __restrict__ h, const int* __restrict__ k_dim_p,
+                                                                                  const int* __restrict__ x_div_p, const int* __restrict__ x_stride_p,
+                                                                                  const int* __restrict__ inter_p, int geo, const Workspace ws) {
+    ENTER(tiles, n_tiles_p, perm, table, x, gs_ptr, h, k_dim_p, x_div_p, x_stride_p, inter_p, geo);
+    const int pairs = geo & 0xFFFFF;
+    const int z = (int)blockIdx.z;
+    if (z >= *n_tiles_p) return;
+    const int4 tl = tiles[z];
+    const int inter = *inter_p;
+    const unsigned char* w = (const unsigned char*)table[2 * tl.x];
+    CROW_REFUSE_NULL_SLAB(w);
+    if (inter % CROW_STRIP_ROWS != 0) {
+        if (threadIdx.x == 0) atomicOr(ws.status, STATUS_BAD_SHAPE);
+        return;
+    }
+    GemvArgs a = gemv_args(w, w + up_offset(inter, pairs), gs_ptr, gs_ptr, x, (size_t)*x_stride_p, h, 0, pairs, k_dim_p, inter_p);
+    a.row_map = perm + tl.y, a.x_div = *x_div_p;
+    CROW_TILE_DISPATCH(2, EPI_SILU_GU)
+}
+extern "C" __global__ void __launch_bounds__(512) moe_down_grouped_tile(const int4* __restrict__ tiles, const int* __restrict__ n_tiles_p,
+                                                                         const int* __restrict__ perm, const unsigned long long* __restrict__ table,
+                                                                         const float* __restrict__ h, const float* __restrict__ gs_ptr,
+                                                                         float* __restrict__ eo, const int* __restrict__ k_dim_p,
+                                                                         const int* __restrict__ rows_p, int geo, const Workspace ws) {
     ENTER(tiles, n_tiles_p, perm, table, h, gs_ptr, eo, k_dim_p, rows_p, geo);
     const int pairs = geo & 0xFFFFF;
     const int z = (int)blockIdx.z;
@@ -400,16 +432,8 @@ extern "C" __global__ void __launch_bounds__(256) moe_down_grouped_short_k(const
     const int4 tl = tiles[z];
     const unsigned char* w = (const unsigned char*)table[2 * tl.x + 1];
     CROW_REFUSE_NULL_SLAB(w);
-    if (pairs <= CROW_GROUP_PAIRS || pairs > 2 * CROW_GROUP_PAIRS || tl.z < 1 || tl.z > 4) {
-        if (threadIdx.x == 0) atomicOr(ws.status, STATUS_BAD_SHAPE);
-        return;
-    }
     GemvArgs a = gemv_args(w, nullptr, gs_ptr, nullptr, h, (size_t)pairs * CROW_PAIR_COLS, eo, 0, pairs, k_dim_p, rows_p);
     a.row_map = perm + tl.y, a.x_div = 1;
-    switch (tl.z) {
-        case 1: short_k_body<1, 2>(a, LDS, ws); break;
-        case 2: short_k_body<2, 2>(a, LDS, ws); break;
-        case 3: short_k_body<3, 2>(a, LDS, ws); break;
-        default: short_k_body<4, 2>(a, LDS, ws); break;
-    }
+    CROW_TILE_DISPATCH(1, EPI_SCALE)
 }
+#undef CROW_TILE_DISPATCH

@@ -165,11 +165,11 @@ class Engine:
 
     def moe_layer(self, moe: MoeW, x: torch.Tensor, logits: torch.Tensor, y: torch.Tensor | None = None):
         """The routed part of one MoE layer with the launch sequence that is faster for this batch, as measured on MI355X at
-        256 experts, top-8: up to 4 tokens the router rides inside the gate|up launch (two launches: 1 token 16.0 us against
-        17.5 us for three, 4 tokens 18.8 / 20.4; at 8 tokens 29.4 / 29.0, every block repeating its token's routing no longer
-        pays); 5 to 23 tokens per combo in three launches; from 24 grouped by expert (five launches, every expert slab read
-        once per four combos: 16 tokens 47 / 53 us per combo / grouped, 24 tokens 65 / 63, 64 tokens 134 / 92)."""
-        if x.shape[0] >= 24:
+        256 experts, top-8: up to 4 tokens the router rides inside the gate|up launch (two launches: 1 token 12.5 us against
+        14.1 us for three, 4 tokens 17.8 / 19.8; at 8 tokens every block repeating its token's routing no longer pays); 5 to
+        27 tokens per combo in three launches; from 28 grouped by expert (five launches, every expert slab read once per four
+        combos: 16 tokens 50 / 57 us per combo / grouped, 24 tokens 69 / 72, 32 tokens 86 / 78, 64 tokens 158 / 101)."""
+        if x.shape[0] >= 28:
             return self.moe_run_grouped(moe, x, logits, y)[:3]
         return self.moe_run(moe, x, logits, "route" if x.shape[0] <= 4 else True, y)
 

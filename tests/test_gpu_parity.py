@@ -685,7 +685,7 @@ def test_grouped_down_on_strips_of_two_groups_gives_the_bits_of_one_row_launches
     eo = torch.full((combos, hdim), float("nan"), dtype=torch.float32, device=eng.dev)
     p = eng.p
     dims = launch_dims("moe_down_grouped", hdim, inter, max_tiles)
-    assert dims[3] == 256 and dims[0] == (hdim + 16 * 32 - 1) // (16 * 32)  # the twin's grid: 4 waves x 8 strips per block
+    assert dims[3] == 256 and dims[0] == (hdim + 16 * 32 - 1) // (16 * 32) and dims[1] >> 24 == 8  # the twin's grid: 4 waves x 8 strips per block
     tl_d, nt_d, perm_d = _dev(tl), _dev(np.array([len(tiles)], dtype=np.int32)), _dev(perm)
     launch_v(eng.k.f("moe_down_grouped"), *dims,
              [tl_d.data_ptr(), nt_d.data_ptr(), perm_d.data_ptr(), table.data_ptr(), hd.data_ptr(), slabs.gs.data_ptr(), eo.data_ptr(), p.i32(inter),
@@ -702,6 +702,50 @@ def test_grouped_down_on_strips_of_two_groups_gives_the_bits_of_one_row_launches
         assert np.array_equal(one.cpu().numpy().view(np.uint32), got[c].view(np.uint32)), c
     ref = orc.gemv(dn[3 * hdim * rb:4 * hdim * rb], hdim, inter, 3.0e-3, h[2])[0]  # combo 2 picked expert 3
     assert rel_err(got[2], ref) <= TOL
+
+
+@pytest.mark.parametrize("inter,hdim", [(512, 2048), (96, 1600), (48, 320)])
+def test_grouped_gate_up_on_short_strips_gives_the_bits_of_per_combo_launches(eng, inter, hdim):
+    """K up to 2048 (this model's gate|up slabs: K = 2048, eight groups per strip): moe_gate_up_silu_grouped runs its twin that
+    stages a tile's activation rows once per block and streams gate strip, up strip, gate strip ... per wave.  Every row of h
+    must be, bit for bit, what the per-combo kernel (moe_gate_up_silu) gives for that combo - also with a partial last group
+    (K = 1600, 320), few rows, and tiles of 1 .. 4 rows."""
+    from crow_nest_amd.kernels import launch_dims, launch_v
+    from crow_nest_amd.weights import load_expert_slabs
+    E, topk = 8, 2
+    print(f"case grouped gate|up inter={inter} hdim={hdim}", flush=True)
+    gu = random_nvfp4(930 + inter, E * 2 * inter, hdim, scale_lo=0x30, scale_hi=0x48, p7f=0)
+    slabs = load_expert_slabs(gu, E, 2 * inter, hdim, 2.0e-3)
+    ids = np.array([3, 1, 3, 0, 3, 7, 3, 1, 7, 3, 7, 5, 5, 5], dtype=np.int32)  # combo c belongs to token c // topk
+    combos, t = ids.size, ids.size // topk
+    perm = np.argsort(ids, kind="stable").astype(np.int32)
+    tiles, start = [], 0
+    for e in range(E):
+        c = int((ids == e).sum())
+        for q in range(0, c, 4):
+            tiles.append((e, start + q, min(4, c - q), 0))
+        start += c
+    max_tiles = len(tiles) + 2
+    tl = np.zeros((max_tiles, 4), dtype=np.int32)
+    tl[:len(tiles)] = np.array(tiles, dtype=np.int32)
+    table = torch.tensor([[slabs.ptr(e), 0] for e in range(E)], dtype=torch.int64, device=eng.dev)
+    x = _dev((normal_f32(13, inter + hdim, t * hdim) * np.float32(0.3)).reshape(t, hdim))
+    p = eng.p
+    tl_d, nt_d, perm_d = _dev(tl), _dev(np.array([len(tiles)], dtype=np.int32)), _dev(perm)
+    h = torch.full((combos, inter), float("nan"), dtype=torch.float32, device=eng.dev)
+    dims = launch_dims("moe_gate_up_silu_grouped", inter, hdim, max_tiles)
+    assert dims[1] >> 24 >= 1 and dims[3] in (256, 512)  # the twin's launch shape: strips per wave in the top byte
+    launch_v(eng.k.f("moe_gate_up_silu_grouped"), *dims,
+             [tl_d.data_ptr(), nt_d.data_ptr(), perm_d.data_ptr(), table.data_ptr(), x.data_ptr(), slabs.gs.data_ptr(), h.data_ptr(), p.i32(hdim),
+              p.i32(topk), p.i32(hdim), p.i32(inter)])
+    eng.check()
+    ptrs = torch.tensor([slabs.ptr(int(e)) for e in ids], dtype=torch.int64, device=eng.dev)
+    h1 = torch.full((combos, inter), float("nan"), dtype=torch.float32, device=eng.dev)
+    launch_v(eng.k.f("moe_gate_up_silu"), *launch_dims("moe_gate_up_silu", inter, hdim, combos),
+             [ptrs.data_ptr(), x.data_ptr(), slabs.gs.data_ptr(), h1.data_ptr(), p.i32(hdim), p.i32(topk), p.i32(hdim), p.i32(inter)])
+    eng.check()
+    assert np.array_equal(h.cpu().numpy().view(np.uint32), h1.cpu().numpy().view(np.uint32))
+    assert np.isfinite(h.cpu().numpy()).all()
 
 
 # ---------------------------------------------------------------- benchmark config 0 (dense GEMV [17408, 5120], f32 x) at full size
