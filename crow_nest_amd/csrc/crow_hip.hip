@@ -31,14 +31,31 @@ struct FnEntry {
     bool takes_geo;  // the launcher appends the model geometry (crow_hip_set_geo) by value, last
 };
 
-#define CROW_FN(name, nargs) {#name, (const void*)&name, nargs, 0u, 0, 16, 0, 1, false, nullptr, false}
-#define CROW_FN_GEO(name, nargs) {#name, (const void*)&name, nargs, 0u, 0, 16, 0, 1, false, nullptr, true}
+// The launcher builds a kernel's argument array from the fields of its table entry: the caller's `nargs` values, then the
+// geometry word (GEMV family), the scratch descriptor (takes_ws), the model geometry (takes_geo).  A kernel that gains a
+// parameter its entry does not append would make HIP read an argument slot nobody wrote; the table is therefore checked
+// against the kernels' own signatures when this file is compiled.
+#define CROW_MAX_LAUNCH_ARGS 18
+template <typename F>
+struct arity;
+template <typename... A>
+struct arity<void (*)(A...)> {
+    static constexpr int value = (int)sizeof...(A);
+};
+template <int NARGS, int APPENDED, typename F>
+constexpr int checked_nargs(F) {
+    static_assert(arity<F>::value == NARGS + APPENDED, "a kernel's parameter list and its table entry disagree");
+    static_assert(NARGS + APPENDED <= CROW_MAX_LAUNCH_ARGS, "the launcher's argument array is too short for this kernel");
+    return NARGS;
+}
+#define CROW_FN(name, nargs) {#name, (const void*)&name, checked_nargs<nargs, 0>(&name), 0u, 0, 16, 0, 1, false, nullptr, false}
+#define CROW_FN_GEO(name, nargs) {#name, (const void*)&name, checked_nargs<nargs, 1>(&name), 0u, 0, 16, 0, 1, false, nullptr, true}
 // NR tensors per block, bodies for 1 .. MMAX activation rows, bf16 or f32 activations
 // (the bodies for several rows need more registers than a block of sixteen waves leaves each: they run in blocks of eight)
 #define CROW_GEMV(name, nargs, NR, MMAX, XBF16) \
-    {#name, (const void*)&name, nargs, 0u, NR, MMAX > 1 ? 8 : 16, crow::crow_gemv_lds_per_wave(MMAX, XBF16), MMAX > 1 ? (XBF16 ? CROW_MULTI_STRIPS_BF16 : CROW_MULTI_STRIPS) : 1, true, nullptr, false}
+    {#name, (const void*)&name, checked_nargs<nargs, 2>(&name), 0u, NR, MMAX > 1 ? 8 : 16, crow::crow_gemv_lds_per_wave(MMAX, XBF16), MMAX > 1 ? (XBF16 ? CROW_MULTI_STRIPS_BF16 : CROW_MULTI_STRIPS) : 1, true, nullptr, false}
 #define CROW_GEMV_GEO(name, nargs, NR, MMAX, XBF16) \
-    {#name, (const void*)&name, nargs, 0u, NR, 16, crow::crow_gemv_lds_per_wave(MMAX, XBF16), 1, true, nullptr, true}
+    {#name, (const void*)&name, checked_nargs<nargs, 3>(&name), 0u, NR, 16, crow::crow_gemv_lds_per_wave(MMAX, XBF16), 1, true, nullptr, true}
 const FnEntry g_table[] = {
     CROW_GEMV(gemv_nvfp4_w, 6, 1, 1, false),       CROW_GEMV(gemv_nvfp4_w_bf16, 6, 1, 1, true),  CROW_GEMV(gemv_nvfp4_w_argmax, 7, 1, 1, false),
     CROW_GEMV(gemv_nvfp4_gu, 8, 2, 1, false),      CROW_GEMV(gemv_nvfp4_gu_bf16, 8, 2, 1, true),
@@ -47,21 +64,21 @@ const FnEntry g_table[] = {
     CROW_GEMV(gemv_fp4_b, 7, 1, 4, false),         CROW_GEMV(gemv_fp4_b1k, 7, 1, 4, false),      CROW_GEMV(gemv_fp4_bs, 8, 1, 4, false),
     CROW_GEMV(gemv_fp4_ptrb, 8, 1, 1, false),      CROW_GEMV(moe_gate_up_silu, 8, 2, 1, false),  CROW_GEMV_GEO(moe_down_combine, 7, 1, 1, false),
     CROW_GEMV_GEO(moe_route_gate_up_silu, 11, 2, 1, false),
-    {"moe_gate_up_silu_grouped", (const void*)&moe_gate_up_silu_grouped, 11, 0u, 2, 8, crow::crow_gemv_lds_per_wave(4, false), CROW_MULTI_STRIPS, true, (const void*)&moe_gate_up_silu_grouped_tile, false},
-    {"moe_down_grouped", (const void*)&moe_down_grouped, 9, 0u, 1, 8, crow::crow_gemv_lds_per_wave(4, false), CROW_MULTI_STRIPS, true, (const void*)&moe_down_grouped_tile, false},
+    {"moe_gate_up_silu_grouped", (const void*)&moe_gate_up_silu_grouped, checked_nargs<11, 2>(&moe_gate_up_silu_grouped) + 0 * checked_nargs<11, 2>(&moe_gate_up_silu_grouped_tile), 0u, 2, 8, crow::crow_gemv_lds_per_wave(4, false), CROW_MULTI_STRIPS, true, (const void*)&moe_gate_up_silu_grouped_tile, false},
+    {"moe_down_grouped", (const void*)&moe_down_grouped, checked_nargs<9, 2>(&moe_down_grouped) + 0 * checked_nargs<9, 2>(&moe_down_grouped_tile), 0u, 1, 8, crow::crow_gemv_lds_per_wave(4, false), CROW_MULTI_STRIPS, true, (const void*)&moe_down_grouped_tile, false},
     CROW_FN_GEO(moe_group, 6),
     CROW_FN_GEO(router_top10, 10), CROW_FN_GEO(silu_mul_combo, 3),  CROW_FN_GEO(acc_combo, 3),
     CROW_FN(argmax_k, 3),          CROW_FN(dequant_fp4_flat, 4),    CROW_FN(repack_nvfp4, 4),
     CROW_FN(unpack_nvfp4, 4),      CROW_FN(dequant_nvfp4_tiled, 5),
     // shared-X GEMM blocks: two staged X tiles of MT rows x 528 bytes
-    {"gemm_nvfp4_bf16", (const void*)&gemm_nvfp4_bf16, 7, 2u * 128u * 528u, 0, 16, 0, 1, false},
-    {"gemm_nvfp4_bf16_m64", (const void*)&gemm_nvfp4_bf16_m64, 7, 2u * 64u * 528u, 0, 16, 0, 1, false},
-    {"gemm_nvfp4_bf16_m48", (const void*)&gemm_nvfp4_bf16_m48, 7, 2u * 48u * 528u, 0, 16, 0, 1, false},
-    {"gemm_nvfp4_bf16_m96", (const void*)&gemm_nvfp4_bf16_m96, 7, 2u * 96u * 528u, 0, 16, 0, 1, false},
-    {"gemm_nvfp4_bf16_w48", (const void*)&gemm_nvfp4_bf16_w48, 7, 2u * 48u * 528u, 0, 8, 0, 1, false},
-    {"gemm_nvfp4_bf16_w64", (const void*)&gemm_nvfp4_bf16_w64, 7, 2u * 64u * 528u, 0, 8, 0, 1, false},
-    {"gemm_nvfp4_bf16_w80", (const void*)&gemm_nvfp4_bf16_w80, 7, 2u * 80u * 528u, 0, 8, 0, 1, false},
-    {"gemm_nvfp4_bf16_w96", (const void*)&gemm_nvfp4_bf16_w96, 7, 2u * 96u * 528u, 0, 8, 0, 1, false},
+    {"gemm_nvfp4_bf16", (const void*)&gemm_nvfp4_bf16, checked_nargs<7, 0>(&gemm_nvfp4_bf16), 2u * 128u * 528u, 0, 16, 0, 1, false},
+    {"gemm_nvfp4_bf16_m64", (const void*)&gemm_nvfp4_bf16_m64, checked_nargs<7, 0>(&gemm_nvfp4_bf16_m64), 2u * 64u * 528u, 0, 16, 0, 1, false},
+    {"gemm_nvfp4_bf16_m48", (const void*)&gemm_nvfp4_bf16_m48, checked_nargs<7, 0>(&gemm_nvfp4_bf16_m48), 2u * 48u * 528u, 0, 16, 0, 1, false},
+    {"gemm_nvfp4_bf16_m96", (const void*)&gemm_nvfp4_bf16_m96, checked_nargs<7, 0>(&gemm_nvfp4_bf16_m96), 2u * 96u * 528u, 0, 16, 0, 1, false},
+    {"gemm_nvfp4_bf16_w48", (const void*)&gemm_nvfp4_bf16_w48, checked_nargs<7, 0>(&gemm_nvfp4_bf16_w48), 2u * 48u * 528u, 0, 8, 0, 1, false},
+    {"gemm_nvfp4_bf16_w64", (const void*)&gemm_nvfp4_bf16_w64, checked_nargs<7, 0>(&gemm_nvfp4_bf16_w64), 2u * 64u * 528u, 0, 8, 0, 1, false},
+    {"gemm_nvfp4_bf16_w80", (const void*)&gemm_nvfp4_bf16_w80, checked_nargs<7, 0>(&gemm_nvfp4_bf16_w80), 2u * 80u * 528u, 0, 8, 0, 1, false},
+    {"gemm_nvfp4_bf16_w96", (const void*)&gemm_nvfp4_bf16_w96, checked_nargs<7, 0>(&gemm_nvfp4_bf16_w96), 2u * 96u * 528u, 0, 8, 0, 1, false},
     CROW_FN(gemm_nvfp4_bf16_m32, 7), CROW_FN(gemm_nvfp4_bf16_m16, 7), CROW_FN(gemv_bf16_w, 5),
     CROW_FN(gemv_bf16, 5), CROW_FN(gemv_bf16_b, 5), CROW_FN(gemv_b, 5), CROW_FN(gemv_bf16_ws, 5), CROW_FN(gemv_bf16_bs, 6),
     CROW_FN(gemv_nvfp4_w_valu1, 6), CROW_FN(gemv_nvfp4_w_valu2, 6), CROW_FN(gemv_nvfp4_w_valu4, 6),  // measurement only
@@ -134,7 +151,7 @@ int launch_entry(const FnEntry* e, dim3 grid, dim3 block, const uint64_t* vals, 
     if ((int)n != e->nargs) return CROW_ERR_ARG_COUNT;
     // whole wavefronts only: every kernel derives its wave count (and its LDS layout) from block.x / 64
     if (grid.x == 0 || grid.y == 0 || grid.z == 0 || block.x == 0 || block.x > 64u * (unsigned)e->max_waves || block.x % 64 != 0) return CROW_ERR_BAD_ARGUMENT;
-    void* args[18];
+    void* args[CROW_MAX_LAUNCH_ARGS];
     for (uint32_t i = 0; i < n; i++) args[i] = (void*)&vals[i];
     uint32_t na = n;
     size_t lds = e->lds_fixed;
@@ -384,9 +401,23 @@ const char* crow_hip_gemm_kernel(uint32_t rows, uint32_t m) {
 // to W waves of the block (combined in LDS) and, only when a strip has more groups than one block's waves can hold, to S
 // blocks (combined through the workspace).  The result depends on (rows, k_dim) only.
 int crow_hip_launch_dims_split(const char* name, uint32_t rows, uint32_t k_dim, uint32_t z, uint32_t force_s, uint32_t force_w, crow_dims* out) {
-    if (!out || !name || rows == 0 || z == 0) return CROW_ERR_BAD_ARGUMENT;
+    if (!out || !name || rows == 0) return CROW_ERR_BAD_ARGUMENT;
     const FnEntry* e = find(name);
     if (!e) return CROW_ERR_KERNEL_MISSING;
+    // CROW_DIMS_COUNT_FROM_MEMORY (verify and token-row kernels only): the launch reads its row count from the word behind
+    // m_p / t_p, as the reference's kernels do; the low bits are then the capacity the grid is sized for
+    const bool from_memory = (z & CROW_DIMS_COUNT_FROM_MEMORY) != 0 || z == 0;
+    z &= ~CROW_DIMS_COUNT_FROM_MEMORY;
+    {
+        const bool takes_count = strcmp(name, "gemv_nvfp4_wm") == 0 || strcmp(name, "gemv_nvfp4_gum") == 0 || strcmp(name, "gemv_nvfp4_wm_bf16") == 0 ||
+                                 strcmp(name, "gemv_nvfp4_gum_bf16") == 0 || strcmp(name, "gemv_fp4_b") == 0 || strcmp(name, "gemv_fp4_b1k") == 0 ||
+                                 strcmp(name, "gemv_fp4_bs") == 0;
+        if (from_memory && !takes_count) return CROW_ERR_BAD_ARGUMENT;
+        if (z == 0) {
+            if (strncmp(name, "gemv_nvfp4_", 11) != 0) return CROW_ERR_BAD_ARGUMENT;  // token rows: the capacity sizes the grid
+            z = 4;                                                                   // the verify kernels' most
+        }
+    }
     const uint32_t strips = (rows + CROW_STRIP_ROWS - 1) / CROW_STRIP_ROWS;
     const uint32_t groups = (k_dim + CROW_GROUP_COLS - 1) / CROW_GROUP_COLS;
     const uint32_t rt = (rows + CROW_TILE_ROWS - 1) / CROW_TILE_ROWS, panels = groups;  // the GEMM's 64-row tiles
@@ -453,7 +484,7 @@ int crow_hip_launch_dims_split(const char* name, uint32_t rows, uint32_t k_dim, 
             s = groups / w;
         }
         const uint32_t gz = routed ? z : (tokens ? (z + 3) / 4 : 1);
-        const uint32_t hint = verify ? z : (tokens ? (z - 1) % 4 + 1 : 0);
+        const uint32_t hint = from_memory ? 0 : (verify ? z : (tokens ? (z - 1) % 4 + 1 : 0));
         const uint32_t gx = (strips + (uint32_t)e->ns - 1) / (uint32_t)e->ns;
         *out = crow_dims{gx, pairs | (hint << 20) | (s << 24), gz, 64u * w * (uint32_t)e->nr};
         if (s > 1 && ((unsigned long long)gx * gz * s * (unsigned)(e->nr * e->ns) * 64 > PARTIAL_FLOATS || (unsigned long long)gx * gz > COUNTER_SLOTS)) return CROW_ERR_WORKSPACE;
@@ -534,7 +565,9 @@ int crow_hip_reset_workspace(void) {
     if (!g.ready) return CROW_ERR_NOT_INITIALIZED;
     hipError_t e = hipDeviceSynchronize();
     if (e != hipSuccess) return (int)e;
-    if ((e = hipMemset(g.ws_static.counters, 0, NOALLOC_COUNTER_SLOTS * sizeof(unsigned))) != hipSuccess) return (int)e;
+    // arrival counters and the status word of both scratch areas (the head's keys need no clearing: every launch overwrites
+    // the words it reads)
+    if ((e = hipMemset(g.ws_static.counters, 0, (NOALLOC_COUNTER_SLOTS + 32) * sizeof(unsigned))) != hipSuccess) return (int)e;
     return hip_rc(hipMemset(g.ws.counters, 0, COUNTER_WORDS * sizeof(unsigned)));
 }
 
@@ -698,6 +731,20 @@ int crow_hip_time_graph(void* graph_exec, void* stream, uint32_t iters, float* u
     *us_per_replay = ms * 1000.0f / (float)iters;
     return out;
 }
+
+#ifdef CROW_TRACE  // measurement builds only: the per-block timestamps of gemv.h
+int crow_hip_trace_read(unsigned long long* dst, size_t words, int clear) {
+    hipError_t e = hipDeviceSynchronize();
+    if (e != hipSuccess) return (int)e;
+    if ((e = hipMemcpyFromSymbol(dst, HIP_SYMBOL(crow::crow_trace), words * 8)) != hipSuccess) return (int)e;
+    if (clear) {
+        void* p = nullptr;
+        if ((e = hipGetSymbolAddress(&p, HIP_SYMBOL(crow::crow_trace))) != hipSuccess) return (int)e;
+        return hip_rc(hipMemset(p, 0, sizeof(unsigned long long) * 16384 * 8));
+    }
+    return CROW_OK;
+}
+#endif
 
 size_t crow_hip_container_bytes(uint32_t rows, uint32_t cols) { return crow_container_bytes(rows, cols); }
 size_t crow_hip_tiled_bytes(uint32_t rows, uint32_t cols) { return crow_tiled_bytes(rows, cols); }

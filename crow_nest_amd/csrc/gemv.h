@@ -62,6 +62,18 @@ namespace crow {
 
 enum Epilogue { EPI_SCALE = 0, EPI_SILU_GU = 1 };
 
+// Measurement builds only (-DCROW_TRACE): per-block timestamps (the 100 MHz wall clock) of the phases of a launch, read back
+// with crow_hip_trace_read.  Slot 0 = the block's first instruction, 1 = its first waves past their first requests and the
+// block barrier, 2 = the last wave done with its groups, 3 = the stores issued.
+#ifdef CROW_TRACE
+__device__ unsigned long long crow_trace[16384 * 8];
+#define CROW_STAMP(slot) do { if (threadIdx.x == 0 && blockIdx.y == 0 && blockIdx.x < 16384) crow_trace[blockIdx.x * 8 + (slot)] = wall_clock64(); } while (0)
+#define CROW_STAMP_LAST(slot) do { if ((threadIdx.x & 63) == 0 && blockIdx.y == 0 && blockIdx.x < 16384) atomicMax(&crow_trace[blockIdx.x * 8 + (slot)], (unsigned long long)wall_clock64()); } while (0)
+#else
+#define CROW_STAMP(slot) do { } while (0)
+#define CROW_STAMP_LAST(slot) do { } while (0)
+#endif
+
 struct GemvArgs {
     const unsigned char* w[2];  // tiled tensors (w[1] only for EPI_SILU_GU: the `up` matrix)
     const float* gs[2];
@@ -767,6 +779,7 @@ __device__ __forceinline__ void gemv_body(const GemvArgs& a, unsigned z, lds_p l
     static_assert(NS * M * 64 <= AREA, "a wave's sums fit its staging area");
     const int lane = lane_id();
     const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6)), waves = block_threads() >> 6;  // wave-uniform on purpose
+    CROW_STAMP(0);
     const int strip = (int)blockIdx.x * NS, strips = (int)gridDim.x * NS;
     const int slice = (int)blockIdx.y, slices = (int)gridDim.y;
     const int k_dim = a.pairs * CROW_PAIR_COLS;
@@ -801,6 +814,7 @@ __device__ __forceinline__ void gemv_body(const GemvArgs& a, unsigned z, lds_p l
         for (int o = 16 * (int)threadIdx.x; o < CROW_GEMV_ZERO_BYTES; o += 16 * (waves << 6)) lds_store16(zero + o, 0, 0, 0, 0);
         if (waves > 1) __syncthreads();
         else __builtin_amdgcn_wave_barrier();
+        CROW_STAMP(1);
     };
     float part[NS][M];
     if constexpr (NS == 1) {
@@ -808,6 +822,7 @@ __device__ __forceinline__ void gemv_body(const GemvArgs& a, unsigned z, lds_p l
         walk.init(wsel + (size_t)strip * groups * CROW_GROUP_BYTES, first, k_dim, a.x, xoff, areas + wave * AREA, zero);
         walk.go(count, mid);
         walk.finish(part[0]);
+        CROW_STAMP_LAST(2);
     } else {
         // Only the launch's last block can reach past the tensor's last strip: it alone reads the row count before its first
         // weight load, and reads an existing strip instead (the sums of a strip beyond the tensor are never stored).
@@ -896,6 +911,7 @@ __device__ __forceinline__ void gemv_body(const GemvArgs& a, unsigned z, lds_p l
             a.y[yo + row] = silu_mul(v[s] * a.gs[0][0], v[(NR - 1) * NS + s] * a.gs[NR - 1][0]);
         }
     }
+    CROW_STAMP(3);
 }
 
 // The body of a product over strips of few groups (TileWalk): grid.x blocks of W waves, every wave a run of `spw` consecutive

@@ -123,6 +123,22 @@ Nvfp4Matrix Nvfp4Matrix::make(const uint8_t* bytes, size_t len, int rows, int co
         throw Refused("cpu_nvfp4: [" + std::to_string(rows) + ", " + std::to_string(cols) + "] needs " + std::to_string(want) + " B, got " + std::to_string(len));
     return Nvfp4Matrix{bytes, len, rows, cols, global_scale};
 }
+ExpertBlock ExpertBlock::make(const Nvfp4Matrix& gate, const Nvfp4Matrix& up, const Nvfp4Matrix& down) {
+    const int inter = gate.rows, hidden = gate.cols;
+    if (up.rows != inter || up.cols != hidden || down.rows != hidden || down.cols != inter)
+        throw Refused("cpu_nvfp4: expert shapes gate [" + std::to_string(gate.rows) + ", " + std::to_string(gate.cols) + "], up [" +
+                      std::to_string(up.rows) + ", " + std::to_string(up.cols) + "], down [" + std::to_string(down.rows) + ", " +
+                      std::to_string(down.cols) + "] do not fit together");
+    return ExpertBlock{gate, up, down, hidden, inter};
+}
+ExpertBlock ExpertBlock::from_unit(const uint8_t* unit, size_t len, int hidden, int inter, const float (&global_scales)[3]) {
+    const size_t gu = Nvfp4Matrix::byte_len(inter, hidden), dn = Nvfp4Matrix::byte_len(hidden, inter);
+    if (len != 2 * gu + dn)
+        throw Refused("cpu_nvfp4: expert unit H " + std::to_string(hidden) + " I " + std::to_string(inter) + " needs " + std::to_string(2 * gu + dn) +
+                      " B, got " + std::to_string(len));
+    return make(Nvfp4Matrix::make(unit, gu, inter, hidden, global_scales[0]), Nvfp4Matrix::make(unit + gu, gu, inter, hidden, global_scales[1]),
+                Nvfp4Matrix::make(unit + 2 * gu, dn, hidden, inter, global_scales[2]));
+}
 static void repack_into(uint64_t raw_dev, int rows, int cols, uint64_t dst_dev) {
     ck(crow_hip_repack_nvfp4((const void*)(uintptr_t)raw_dev, (uint32_t)rows, (uint32_t)cols, (void*)(uintptr_t)dst_dev), "crow_hip_repack_nvfp4");
 }
@@ -139,6 +155,11 @@ Fp4 load_fp4(const Nvfp4Matrix& m) {
     sync();  // the raw copy is freed when this returns
     status();
     return out;
+}
+MlpW load_expert_block(const ExpertBlock& e) {
+    MlpW m;
+    m.gate = load_fp4(e.gate), m.up = load_fp4(e.up), m.down = load_fp4(e.down);
+    return m;
 }
 std::vector<float> dequant(const Fp4& w) {
     const size_t n = (size_t)w.rows * w.cols;

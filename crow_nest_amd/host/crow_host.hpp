@@ -119,6 +119,17 @@ struct Nvfp4Matrix {
     static Nvfp4Matrix make(const uint8_t* bytes, size_t len, int rows, int cols, float global_scale);
 };
 
+// one routed expert on the host (cpu_nvfp4::ExpertBlock, cpu_nvfp4.rs:143-179): gate [inter, hidden], up [inter, hidden],
+// down [hidden, inter].  Refused "cpu_nvfp4: expert shapes gate [..], up [..], down [..] do not fit together" /
+// "cpu_nvfp4: expert unit H {hidden} I {inter} needs {n} B, got {m}"
+struct ExpertBlock {
+    Nvfp4Matrix gate, up, down;
+    int hidden, inter;
+    static ExpertBlock make(const Nvfp4Matrix& gate, const Nvfp4Matrix& up, const Nvfp4Matrix& down);
+    // one expert unit as the GLM converter writes it: gate | up | down back to back, global scales in that order
+    static ExpertBlock from_unit(const uint8_t* unit, size_t len, int hidden, int inter, const float (&global_scales)[3]);
+};
+
 // PW::Fp4(w, gs): tiled weight bytes and the global scale, both on the device
 struct Fp4 {
     DevBuf w, gs;
@@ -130,6 +141,7 @@ std::vector<float> dequant(const Fp4& w);  // f32 [rows][cols], bit-exact with t
 struct MlpW {
     Fp4 gate, up, down;
 };
+MlpW load_expert_block(const ExpertBlock& e);  // the unit's three matrices on the device, each under its own global scale
 
 // an expert tensor [E][rows][cols] re-tiled per expert: slab e starts at e * slab_bytes (residency.rs:108-117)
 struct ExpertSlabs {

@@ -5,6 +5,8 @@ Mirrors, for the NVFP4 path only:
     rows / cols / global scale, with the same shape checks and error texts;
   * ``weights::load_fp4 -> Fp4 {w, gs}`` and ``PW::Fp4(w, gs)`` (engine/src/weights.rs:26-33,
     engine/src/gen.rs:234-237): device bytes + a one-float device scalar;
+  * ``cpu_nvfp4::ExpertBlock`` with ``new`` and ``from_unit`` (engine/src/cpu_nvfp4.rs:143-179): one routed expert as three
+    matrices, or cut out of a gate | up | down unit, same checks and texts;
   * the loader's scale rule 0x7F -> 0x7E (engine/src/gen.rs:2178-2187, residency.rs:126-137), which the
     library's repacker applies while it re-tiles (``crow_hip_repack_nvfp4``);
   * ``Params`` (engine/src/gen.rs:2913-2925): the 4-byte device words kernels read their scalars from.
@@ -45,6 +47,44 @@ class Nvfp4Matrix:
         if b.size != want:
             raise ValueError(f"cpu_nvfp4: [{rows}, {cols}] needs {want} B, got {b.size}")
         return Nvfp4Matrix(b, rows, cols, float(np.float32(global_scale)))
+
+
+@dataclass(frozen=True)
+class ExpertBlock:
+    """One routed expert on the host (``cpu_nvfp4::ExpertBlock``, engine/src/cpu_nvfp4.rs:143-179): gate [inter, hidden],
+    up [inter, hidden], down [hidden, inter], each with its own global scale."""
+    gate: Nvfp4Matrix
+    up: Nvfp4Matrix
+    down: Nvfp4Matrix
+    hidden: int
+    inter: int
+
+    @staticmethod
+    def new(gate: Nvfp4Matrix, up: Nvfp4Matrix, down: Nvfp4Matrix) -> "ExpertBlock":
+        inter, hidden = gate.rows, gate.cols
+        if (up.rows, up.cols) != (inter, hidden) or (down.rows, down.cols) != (hidden, inter):
+            raise ValueError(f"cpu_nvfp4: expert shapes gate [{gate.rows}, {gate.cols}], up [{up.rows}, {up.cols}], "
+                             f"down [{down.rows}, {down.cols}] do not fit together")
+        return ExpertBlock(gate, up, down, hidden, inter)
+
+    @staticmethod
+    def from_unit(unit, hidden: int, inter: int, global_scales) -> "ExpertBlock":
+        """One expert unit as the GLM converter writes it: gate | up | down back to back, global scales in that order
+        (``ExpertBlock::from_unit``, engine/src/cpu_nvfp4.rs:165-178)."""
+        b = np.ascontiguousarray(np.asarray(unit, dtype=np.uint8).reshape(-1))
+        gu, dn = Nvfp4Matrix.byte_len(inter, hidden), Nvfp4Matrix.byte_len(hidden, inter)
+        if b.size != 2 * gu + dn:
+            raise ValueError(f"cpu_nvfp4: expert unit H {hidden} I {inter} needs {2 * gu + dn} B, got {b.size}")
+        g0, g1, g2 = global_scales
+        return ExpertBlock.new(Nvfp4Matrix.new(b[:gu], inter, hidden, g0), Nvfp4Matrix.new(b[gu:2 * gu], inter, hidden, g1),
+                               Nvfp4Matrix.new(b[2 * gu:], hidden, inter, g2))
+
+
+def load_expert_block(e: ExpertBlock):
+    """The three matrices of one expert unit on the device, as an ``engine.MlpW`` (gate, up, down): the dense kernels
+    (gemv_nvfp4_gu + gemv_nvfp4_w) then run the expert's FFN, each matrix under its own global scale."""
+    from .engine import MlpW
+    return MlpW(load_fp4(e.gate), load_fp4(e.up), load_fp4(e.down))
 
 
 def _device() -> torch.device:

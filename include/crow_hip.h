@@ -88,8 +88,10 @@ int crow_hip_launch(crow_fn_t f, uint32_t gx, uint32_t gy, uint32_t gz, uint32_t
  * `gy`) with more than CROW_NOALLOC_MAX_PARTIAL_FLOATS partial sums (gx * gz * S * tensors * 64) or more than
  * CROW_NOALLOC_MAX_STRIPS strips (gx * gz), and a fused head (gemv_nvfp4_w_argmax) of more than CROW_NOALLOC_MAX_HEAD_STRIPS
  * strips, is refused with CROW_ERR_WORKSPACE before anything runs.  Every call on a device
- * shares the one array: calls that overlap on the device (two streams, two threads) race; order them on one stream.  crow_hip_status
- * reports both scratch areas. */
+ * shares the one array: calls that overlap on the device (two streams, two threads) race; order them on one stream.  (The
+ * library cannot check this for the caller: telling whether an earlier launch on another stream is still running takes a
+ * stream query, which is not legal while a stream is being captured in global mode - the very callers this entry point
+ * is for.)  crow_hip_status reports both scratch areas; crow_hip_reset_workspace clears the counters and status words of both. */
 #define CROW_NOALLOC_MAX_PARTIAL_FLOATS (1u << 20)
 #define CROW_NOALLOC_MAX_STRIPS 4096u
 #define CROW_NOALLOC_MAX_HEAD_STRIPS 16384u /* the fused head through this entry point: at most 262,144 rows */
@@ -97,7 +99,22 @@ int crow_hip_launch(crow_fn_t f, uint32_t gx, uint32_t gy, uint32_t gz, uint32_t
 int crow_hip_launch_noalloc(crow_fn_t f, uint32_t gx, uint32_t gy, uint32_t gz, uint32_t bx, const uint64_t* vals,
                             uint32_t n_vals, void* stream);
 /* grid/block for `name` on a [rows, k_dim] tensor with `z` token rows (batched and verify kernels: the value *t_p / *m_p
- * will hold) or combos (routed kernels); 1 otherwise.  The split of the work depends on (rows, k_dim) only, never on z. */
+ * will hold) or combos (routed kernels); 1 otherwise.  The split of the work depends on (rows, k_dim) only, never on z.
+ *
+ * Dimensions made for a row count are BOUND to it: the count rides in `gy`, the kernel works with it from its first
+ * instruction and stores nothing (CROW_ERR_SHAPE from crow_hip_status) if the word behind m_p / t_p says otherwise - so a
+ * launch captured into a graph with such dimensions serves that one count.  For the reference's own convention - a fixed
+ * grid, the count read from the device word by every launch (engine/src/kernels_p2.rs:472-497, gen.rs:5455-5466 rewrite
+ * *m_p per step) - pass z = CROW_DIMS_COUNT_FROM_MEMORY | capacity: the verify kernels (gemv_nvfp4_wm / _gum and their
+ * bf16 twins; capacity 1..4, or plain z = 0) then serve any 1 <= *m_p <= 4 with one set of dimensions and one captured
+ * graph, the token-row kernels (gemv_fp4_b / _b1k / _bs) any 1 <= *t_p <= capacity.  Row m of such a launch holds the same
+ * bits as under dimensions bound to the count; the only cost is one dependent read before the first weight request.
+ *
+ * Precondition of every launch of the NVFP4 GEMV family: the four words come from this call for the SAME (rows, k_dim) as
+ * the weight tensor handed to the kernel.  The kernels read their weights as the dimensions say before they compare K and
+ * the row count with the caller's device words (a disagreement stores nothing and raises CROW_ERR_SHAPE) - dimensions
+ * made for a larger tensor make them read beyond the allocation. */
+#define CROW_DIMS_COUNT_FROM_MEMORY 0x80000000u
 int crow_hip_launch_dims(const char* name, uint32_t rows, uint32_t k_dim, uint32_t z, crow_dims* out);
 /* the GEMM entry point (a name of the kernel table) that serves `m` token rows fastest on a tensor of `rows` rows: the
  * choice depends on how the blocks of each tiling fall on this device's compute units */

@@ -258,6 +258,26 @@ int main(int argc, char** argv) {
             printf("ok %d %d %zu\n", ok.rows, ok.cols, Nvfp4Matrix::byte_len(17408, 5120));
             return 0;
         }
+        if (cmd == "expert-checks") {  // ExpertBlock::new / from_unit refusals and an accepted unit (no GPU needed)
+            const size_t gu = Nvfp4Matrix::byte_len(64, 128), dn = Nvfp4Matrix::byte_len(128, 64);
+            std::vector<uint8_t> unit(2 * gu + dn, 0);
+            const float gsv[3] = {1.0f, 2.0f, 3.0f};
+            try {
+                ExpertBlock::from_unit(unit.data(), unit.size() - 1, 128, 64, gsv);
+            } catch (const Refused& e) {
+                printf("%s\n", e.what());
+            }
+            try {
+                ExpertBlock::make(Nvfp4Matrix::make(unit.data(), gu, 64, 128, 1.0f), Nvfp4Matrix::make(unit.data(), gu, 64, 128, 1.0f),
+                                  Nvfp4Matrix::make(unit.data(), gu, 64, 128, 1.0f));
+            } catch (const Refused& e) {
+                printf("%s\n", e.what());
+            }
+            const ExpertBlock ok = ExpertBlock::from_unit(unit.data(), unit.size(), 128, 64, gsv);
+            printf("ok H %d I %d gate %zu up %zu down %zu scales %g %g %g\n", ok.hidden, ok.inter, (size_t)(ok.gate.bytes - unit.data()),
+                   (size_t)(ok.up.bytes - unit.data()), (size_t)(ok.down.bytes - unit.data()), ok.gate.global_scale, ok.up.global_scale, ok.down.global_scale);
+            return 0;
+        }
         if (cmd == "cnq-list" && argc == 3) return cnq_list(argv[2]);
         if (cmd == "cnq-refuse" && argc == 3) {
             try {

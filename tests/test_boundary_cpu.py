@@ -104,6 +104,24 @@ def test_matrix_shapes_are_checked_like_the_reference():
         Nvfp4Matrix.new(b[1:], 3, 128, 1.0)
 
 
+def test_expert_block_is_cut_out_of_a_unit_like_the_reference():
+    """ExpertBlock::new / from_unit (engine/src/cpu_nvfp4.rs:153-178): gate | up | down back to back, the three global scales
+    in that order, the reference's refusal texts."""
+    from crow_nest_amd.weights import ExpertBlock
+    hidden, inter = 128, 64
+    gu, dn = Nvfp4Matrix.byte_len(inter, hidden), Nvfp4Matrix.byte_len(hidden, inter)
+    unit = (np.arange(2 * gu + dn) % 251).astype(np.uint8)
+    e = ExpertBlock.from_unit(unit, hidden, inter, (1.0, 2.0, 3.0))
+    assert (e.hidden, e.inter) == (hidden, inter)
+    assert np.array_equal(e.gate.bytes, unit[:gu]) and np.array_equal(e.up.bytes, unit[gu:2 * gu]) and np.array_equal(e.down.bytes, unit[2 * gu:])
+    assert (e.gate.global_scale, e.up.global_scale, e.down.global_scale) == (1.0, 2.0, 3.0)
+    assert (e.down.rows, e.down.cols) == (hidden, inter)
+    with pytest.raises(ValueError, match=f"expert unit H 128 I 64 needs {2 * gu + dn} B, got {2 * gu + dn - 1}"):
+        ExpertBlock.from_unit(unit[1:], hidden, inter, (1.0, 2.0, 3.0))
+    with pytest.raises(ValueError, match=r"expert shapes gate \[64, 128\], up \[64, 128\], down \[64, 128\] do not fit together"):
+        ExpertBlock.new(e.gate, e.up, e.gate)
+
+
 def test_no_cpu_fallback():
     import torch
     if torch.cuda.is_available():

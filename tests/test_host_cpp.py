@@ -44,6 +44,14 @@ def test_nvfp4_matrix_checks_and_their_texts():
     assert out == ["cpu_nvfp4: 96 columns are not whole 64-value NVFP4 blocks", "cpu_nvfp4: [2, 128] needs 144 B, got 72", "ok 2 64 50135040"]
 
 
+def test_expert_block_checks_and_their_texts():
+    out = run("expert-checks").splitlines()  # cpu_nvfp4.rs:153-178
+    gu, dn = 64 * 2 * 36, 128 * 36
+    assert out == [f"cpu_nvfp4: expert unit H 128 I 64 needs {2 * gu + dn} B, got {2 * gu + dn - 1}",
+                   "cpu_nvfp4: expert shapes gate [64, 128], up [64, 128], down [64, 128] do not fit together",
+                   f"ok H 128 I 64 gate 0 up {gu} down {2 * gu} scales 1 2 3"]
+
+
 def test_container_table_equals_the_python_reader():
     out = run("cnq-list", FIXTURE).splitlines()
     c = Cnq.open(FIXTURE)
