@@ -92,7 +92,7 @@ struct State {
     hipStream_t stream = nullptr;
     crow::Workspace ws{};
     crow::Workspace ws_static{};  // the same roles inside `scratch`, through the device address crow_hip_init asked for
-    int* scalars = nullptr;  // two device words for the library's own launches (rows, k_dim)
+    int* scalars = nullptr;  // device words for the library's own launches: (rows, k_dim) of the layout calls, the encoder's maxima
     char name[256] = {0};
     crow::Geo model{0, 0, 0, 0};  // the routed geometry (crow_hip_set_geo): appended by value to the kernels that take it
     size_t lds_cap = 64u * 1024u;  // most LDS one workgroup may take on this device
@@ -234,7 +234,7 @@ int crow_hip_init(int device) {
     if ((e = hipMalloc((void**)&ws.head, HEAD_WORDS * sizeof(unsigned long long))) != hipSuccess) return fail(e);
     if ((e = hipMemset(ws.head, 0, HEAD_WORDS * sizeof(unsigned long long))) != hipSuccess) return fail(e);
     ws.head_words = HEAD_WORDS;
-    if ((e = hipMalloc((void**)&scalars, 16 * sizeof(int))) != hipSuccess) return fail(e);
+    if ((e = hipMalloc((void**)&scalars, 32 * sizeof(int))) != hipSuccess) return fail(e);  // words 0..15: (rows, k_dim) of the layout calls, 16..23: the encoder's maxima
     if ((e = hipMemset(ws.counters, 0, COUNTER_WORDS * sizeof(unsigned))) != hipSuccess) return fail(e);
     ws.status = ws.counters + COUNTER_SLOTS;
     if ((e = hipMemcpyToSymbol(HIP_SYMBOL(crow::g_ws), &ws, sizeof ws)) != hipSuccess) return fail(e);
@@ -774,6 +774,29 @@ static int layout_launch(const char* name, const void* a, const void* b, const v
     rc = launch_entry(find(name), dim3(d.gx, d.gy, d.gz), dim3(d.bx), vals, n, g.stream, g.ws);
     if (rc != CROW_OK) return rc;
     return crow_hip_status();
+}
+
+int crow_hip_quantize_nvfp4(const float* values_dev, size_t n_values, void* blocks_dev, float* global_scale_dev) {
+    if (!g.ready) return CROW_ERR_NOT_INITIALIZED;
+    if (!values_dev || !blocks_dev || !global_scale_dev) return CROW_ERR_BAD_ARGUMENT;
+    if (n_values == 0 || n_values % CROW_BLOCK_VALUES != 0) return CROW_ERR_SHAPE;
+    // the tensor's largest raw scale meets in one device word (one of the library's own, taken in turn so that calls in a
+    // row do not share it)
+    static int slot = 0;
+    unsigned* max_bits = (unsigned*)(g.scalars + 16 + (slot++ & 7));
+    hipError_t e = hipMemsetAsync(max_bits, 0, sizeof(unsigned), g.stream);
+    if (e != hipSuccess) return (int)e;
+    unsigned long long n_sub = n_values / 16;
+    const unsigned long long want = (n_sub + 255) / 256;
+    const unsigned blocks1 = (unsigned)(want < 8192 ? want : 8192);
+    const float* vals = values_dev;
+    unsigned char* out = (unsigned char*)blocks_dev;
+    const unsigned* max_ro = max_bits;
+    void* a1[3] = {(void*)&vals, (void*)&n_sub, (void*)&max_bits};
+    if ((e = hipLaunchKernel((const void*)&quantize_nvfp4_amax, dim3(blocks1), dim3(256), a1, 0, g.stream)) != hipSuccess) return (int)e;
+    if (want > 0x7FFFFFFFull) return CROW_ERR_SHAPE;
+    void* a2[5] = {(void*)&vals, (void*)&n_sub, (void*)&max_ro, (void*)&out, (void*)&global_scale_dev};
+    return hip_rc(hipLaunchKernel((const void*)&quantize_nvfp4_encode, dim3((unsigned)want), dim3(256), a2, 0, g.stream));
 }
 
 int crow_hip_repack_nvfp4(const void* src_dev, uint32_t rows, uint32_t cols, void* dst_dev) {

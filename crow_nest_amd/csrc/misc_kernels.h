@@ -106,6 +106,87 @@ extern "C" __global__ void dequant_fp4_flat(const unsigned char* __restrict__ w,
     out[i] = v.x * s;
 }
 
+// ------------------------------------------------------------------ the NVFP4 encoder (ceiling scales)
+// reference: quantize_nvfp4 in ScalesMode::Ceil, converter/src/main.rs:550-664 with encode_ue4m3_ceil / encode_subblock_ceil
+// (:141-169, :404-410) and e2m1_index (:111-119): f32 values -> container blocks (4 scale bytes + 32 code bytes per 64
+// values) and the tensor's global scale.  Every division the converter makes with `/` is a correctly rounded IEEE division
+// here (raw = amax / 6, global = max raw / 448, r = raw / global, inv = 1 / dec); the codes are chosen against
+// |v| * inv, the reciprocal, exactly as the converter does.
+//
+// The scale byte: the converter's search (start from floor(log2 r) + 7, step through mantissas with ceil, carry, then bump
+// while the decoded byte is still below r) ends - whatever its log2 returns at a power of two - at the SMALLEST byte whose
+// value is >= r, or 0x7F when r is beyond 480.  With r >= 2^-6 that byte is r's own f32 pattern rounded UP to three mantissa
+// bits (exponent field e + 120, the mantissa's top three bits m); below, the subnormal ladder m = ceil(512 r).  r <= 0 gives
+// 0, and the one NaN the arithmetic can make (inf / inf) the 0x38 the converter's casts make of it.
+__device__ __forceinline__ unsigned ue4m3_ceil_byte(float r) {
+    if (!(r == r)) return 0x38u;
+    if (r <= 0.0f) return 0u;
+    if (r > 480.0f) return 0x7Fu;
+    if (r < 0x1p-6f) {
+        const unsigned m = (unsigned)ceilf(r * 512.0f);  // 1..8 (exact product)
+        return m;                                        // 8 = the first normal byte, 2^-6
+    }
+    unsigned u = __float_as_uint(r);
+    if (u & 0xFFFFFu) u = (u | 0xFFFFFu) + 1u;
+    return (((u >> 23) - 120u) << 3) | ((u >> 20) & 7u);
+}
+__device__ __forceinline__ float ue4m3_value(unsigned byte) {  // decode_ue4m3 (bytes 0..0x7F; 0x7F = 480)
+    return __uint_as_float((byte & 0x7Fu) << 20) * 0x1p120f;
+}
+// amax / 6 of the 16 values at `v` (f32::max ignores a NaN operand, like fmaxf)
+__device__ __forceinline__ float subblock_raw(const float4 (&q)[4]) {
+    float m = 0.0f;
+#pragma unroll
+    for (int i = 0; i < 4; i++) m = fmaxf(fmaxf(fmaxf(fmaxf(m, fabsf(q[i].x)), fabsf(q[i].y)), fabsf(q[i].z)), fabsf(q[i].w));
+    return __fdiv_rn(m, 6.0f);
+}
+// pass 1: the largest raw scale of the tensor, as the bit pattern of a non-negative f32 (they order like unsigned integers)
+// grid-stride over the n / 16 sub-blocks; *max_bits starts as 0
+extern "C" __global__ void __launch_bounds__(256) quantize_nvfp4_amax(const float* __restrict__ values, unsigned long long n_sub,
+                                                                       unsigned* __restrict__ max_bits) {
+    float best = 0.0f;
+    for (unsigned long long i = (unsigned long long)blockIdx.x * blockDim.x + threadIdx.x; i < n_sub; i += (unsigned long long)gridDim.x * blockDim.x) {
+        const float4* p = (const float4*)(values + 16 * i);
+        const float4 q[4] = {p[0], p[1], p[2], p[3]};
+        best = fmaxf(best, subblock_raw(q));
+    }
+    for (int o = 32; o > 0; o >>= 1) best = fmaxf(best, __shfl_xor(best, o));
+    if ((threadIdx.x & 63u) == 0 && best > 0.0f) atomicMax(max_bits, __float_as_uint(best));
+}
+// pass 2: one thread per sub-block: its scale byte and its sixteen codes; thread 0 also leaves the global scale
+extern "C" __global__ void __launch_bounds__(256) quantize_nvfp4_encode(const float* __restrict__ values, unsigned long long n_sub,
+                                                                         const unsigned* __restrict__ max_bits, unsigned char* __restrict__ blocks,
+                                                                         float* __restrict__ global_out) {
+    const float max_scale = __uint_as_float(*max_bits);
+    const float global = max_scale > 0.0f ? __fdiv_rn(max_scale, 448.0f) : 1.0f;
+    const unsigned long long i = (unsigned long long)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i == 0) global_out[0] = global;
+    if (i >= n_sub) return;
+    const float4* p = (const float4*)(values + 16 * i);
+    const float4 q[4] = {p[0], p[1], p[2], p[3]};
+    const unsigned byte = ue4m3_ceil_byte(__fdiv_rn(subblock_raw(q), global));
+    const float dec = ue4m3_value(byte) * global;
+    const float inv = __fdiv_rn(1.0f, dec);
+    auto code = [&](float v) -> unsigned {
+        const float m = fabsf(v) * inv;  // (0 * inf = NaN: every comparison false, code 0, as in the converter)
+        const unsigned idx = (unsigned)(m >= 0.25f) + (unsigned)(m >= 0.75f) + (unsigned)(m >= 1.25f) + (unsigned)(m >= 1.75f) + (unsigned)(m >= 2.5f) +
+                             (unsigned)(m >= 3.5f) + (unsigned)(m >= 5.0f);
+        return idx | ((v < 0.0f) ? 8u : 0u);
+    };
+    unsigned lo = 0, hi = 0;  // values 0..7 and 8..15 of the sub-block, four bits each, value j in bits 4 j
+#pragma unroll
+    for (int k = 0; k < 2; k++) {
+        lo |= (code(q[k].x) | (code(q[k].y) << 4) | (code(q[k].z) << 8) | (code(q[k].w) << 12)) << (16 * k);
+        hi |= (code(q[2 + k].x) | (code(q[2 + k].y) << 4) | (code(q[2 + k].z) << 8) | (code(q[2 + k].w) << 12)) << (16 * k);
+    }
+    unsigned char* blk = blocks + (i >> 2) * CROW_BLOCK_BYTES;
+    const unsigned sb = (unsigned)(i & 3);
+    blk[sb] = (unsigned char)byte;
+    unsigned* codes = (unsigned*)(blk + 4 + 8 * sb);  // (36-byte blocks: every code dword is four-byte aligned)
+    codes[0] = lo;
+    codes[1] = hi;
+}
+
 // ------------------------------------------------------------------ router
 // Wave-wide maximum of an unsigned key through the data-parallel lane moves (an inclusive scan along the rows of 16
 // lanes, then the two row broadcasts; lane 63 ends with the maximum): six dependent vector instructions where a

@@ -24,6 +24,11 @@ class KernelMissing(KeyError):
     pass
 
 
+# crow_hip.h: CROW_DIMS_COUNT_FROM_MEMORY - launch_dims(name, rows, k, COUNT_FROM_MEMORY | capacity): the launch reads its row
+# count from the device word behind m_p / t_p (the reference's convention: a fixed grid, the word rewritten per step)
+COUNT_FROM_MEMORY = 0x80000000
+
+
 @dataclass(frozen=True)
 class KernelGeo:
     """The geometry the reference bakes into its kernel source (kernels.rs:5040-5125, CN_* defines)."""

@@ -91,6 +91,7 @@ def lib():
         "crow_hip_repack_nvfp4": (C.c_int, [vp, u32, u32, vp]),
         "crow_hip_unpack_nvfp4": (C.c_int, [vp, u32, u32, vp]),
         "crow_hip_dequant_tiled": (C.c_int, [vp, vp, u32, u32, vp]),
+        "crow_hip_quantize_nvfp4": (C.c_int, [vp, sz, vp, vp]),
     }
     for name, (res, args) in sig.items():
         fn = getattr(L, name)  # AttributeError here = the library does not export what the header declares
@@ -112,7 +113,7 @@ EXPORTS = [
     "crow_hip_stream_create", "crow_hip_stream_destroy", "crow_hip_begin_capture", "crow_hip_end_capture_instantiate",
     "crow_hip_launch_graph", "crow_hip_graph_exec_destroy",
     "crow_hip_container_bytes", "crow_hip_tiled_bytes", "crow_hip_tile_code_offset", "crow_hip_tile_scale_offset", "crow_hip_repack_nvfp4", "crow_hip_unpack_nvfp4",
-    "crow_hip_dequant_tiled",
+    "crow_hip_dequant_tiled", "crow_hip_quantize_nvfp4",
 ]
 
 

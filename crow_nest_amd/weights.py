@@ -168,6 +168,29 @@ def load_expert_slabs_cnq(cnq, name: str, sec: str) -> ExpertSlabs:
     return load_expert_slabs(data, e, rows, cols, t.global_scale)
 
 
+def quantize_nvfp4(values: torch.Tensor) -> tuple[torch.Tensor, torch.Tensor]:
+    """``quantize_nvfp4`` with ceiling scales (converter/src/main.rs:550-664, ScalesMode::Ceil) on the device:
+    f32 values (a multiple of 64; sub-blocks are 16 consecutive values) -> (container blocks, uint8 [n / 64 * 36]; the
+    tensor's global scale, float32 [1]), byte for byte what the converter writes."""
+    _l.ensure_init()
+    v = values.reshape(-1)
+    if not (v.is_cuda and v.dtype == torch.float32 and v.is_contiguous()):
+        raise ValueError("quantize_nvfp4: f32 values on the device, contiguous")
+    if v.numel() == 0 or v.numel() % BLOCK_VALUES != 0:
+        raise ValueError(f"quantize_nvfp4: {v.numel()} values are not whole 64-value NVFP4 blocks")
+    blocks = torch.empty(v.numel() // BLOCK_VALUES * BLOCK_BYTES, dtype=torch.uint8, device=v.device)
+    gs = torch.empty(1, dtype=torch.float32, device=v.device)
+    _l.check(_l.lib().crow_hip_quantize_nvfp4(v.data_ptr(), v.numel(), blocks.data_ptr(), gs.data_ptr()), "crow_hip_quantize_nvfp4")
+    return blocks, gs
+
+
+def load_fp4_quantized(blocks: torch.Tensor, gs: torch.Tensor, rows: int, cols: int) -> Fp4:
+    """Container blocks already on the device (``quantize_nvfp4``'s) -> the tiled tensor the kernels read."""
+    w = torch.empty(tiled_bytes(rows, cols), dtype=torch.uint8, device=blocks.device)
+    repack_into(blocks, rows, cols, w)
+    return Fp4(w, gs, rows, cols)
+
+
 def unpack(w: Fp4) -> np.ndarray:
     """Tiled -> container bytes (scale bytes canonical); for round-trip checks."""
     out = torch.empty(Nvfp4Matrix.byte_len(w.rows, w.cols), dtype=torch.uint8, device=w.w.device)

@@ -160,6 +160,15 @@ size_t crow_hip_tiled_bytes(uint32_t rows, uint32_t cols);
  * (strip * ceil(cols / 256) + gi) * 2304.  UINT32_MAX for an argument out of range. */
 uint32_t crow_hip_tile_code_offset(uint32_t row, uint32_t wp);
 uint32_t crow_hip_tile_scale_offset(uint32_t row, uint32_t sb);
+/* ---- the NVFP4 encoder, ceiling scales: quantize_nvfp4 with ScalesMode::Ceil of converter/src/main.rs:550-664
+ * (encode_ue4m3_ceil :141-169, encode_subblock_ceil :404-410, e2m1_index :111-119), on the device.
+ * values_dev: n_values f32 (a multiple of 64; sub-blocks are 16 consecutive values); blocks_dev: n_values / 64 * 36 bytes of
+ * container blocks (4 scale bytes + 32 code bytes each); *global_scale_dev: max(amax / 6) / 448, or 1 for an all-zero
+ * tensor.  Byte for byte what the converter writes (every `/` of its arithmetic a correctly rounded division, the codes
+ * chosen against the reciprocal of the decoded scale), so the result loads through crow_hip_repack_nvfp4 like any
+ * container tensor.  Asynchronous on the current stream. ---- */
+int crow_hip_quantize_nvfp4(const float* values_dev, size_t n_values, void* blocks_dev, float* global_scale_dev);
+
 /* src_dev: container bytes [rows][cols/64][36] already on the device; dst_dev: crow_hip_tiled_bytes.
  * Applies the scale rule (0x7F -> 0x7E).  Expert tensors [E][rows][cols]: call once per expert
  * slab, the tiled slabs are then contiguous per expert. */
