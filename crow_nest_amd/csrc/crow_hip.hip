@@ -234,7 +234,7 @@ int crow_hip_init(int device) {
     if ((e = hipMalloc((void**)&ws.head, HEAD_WORDS * sizeof(unsigned long long))) != hipSuccess) return fail(e);
     if ((e = hipMemset(ws.head, 0, HEAD_WORDS * sizeof(unsigned long long))) != hipSuccess) return fail(e);
     ws.head_words = HEAD_WORDS;
-    if ((e = hipMalloc((void**)&scalars, 32 * sizeof(int))) != hipSuccess) return fail(e);  // words 0..15: (rows, k_dim) of the layout calls, 16..23: the encoder's maxima
+    if ((e = hipMalloc((void**)&scalars, 32 * sizeof(int))) != hipSuccess) return fail(e);  // words 0..15: (rows, k_dim) of the layout calls, 16..23: the encoder's maxima, 24: the read probe's sink
     if ((e = hipMemset(ws.counters, 0, COUNTER_WORDS * sizeof(unsigned))) != hipSuccess) return fail(e);
     ws.status = ws.counters + COUNTER_SLOTS;
     if ((e = hipMemcpyToSymbol(HIP_SYMBOL(crow::g_ws), &ws, sizeof ws)) != hipSuccess) return fail(e);
@@ -669,6 +669,32 @@ int crow_hip_time_sequence(uint32_t n_kernels, const crow_fn_t* fns, const crow_
     (void)hipEventDestroy(a);
     (void)hipEventDestroy(b);
     *us_per_iteration = ms * 1000.0f / (float)iters;
+    return out;
+}
+
+int crow_hip_time_pure_read(const uint64_t* bufs, uint32_t n_bufs, size_t bytes, uint32_t blocks, uint32_t threads, uint32_t iters, float* us_per_launch) {
+    if (!g.ready) return CROW_ERR_NOT_INITIALIZED;
+    if (!bufs || !us_per_launch || n_bufs == 0 || iters == 0 || blocks == 0 || threads == 0 || threads % 64 != 0 || threads > 1024) return CROW_ERR_BAD_ARGUMENT;
+    if (bytes == 0 || bytes % CROW_GROUP_BYTES != 0 || bytes / CROW_GROUP_BYTES > 0xFFFFFFFFull) return CROW_ERR_SHAPE;
+    unsigned units = (unsigned)(bytes / CROW_GROUP_BYTES);
+    unsigned* sink = (unsigned*)(g.scalars + 24);
+    hipEvent_t a, b;
+    hipError_t rc;
+    if ((rc = hipEventCreate(&a)) != hipSuccess) return (int)rc;
+    if ((rc = hipEventCreate(&b)) != hipSuccess) return (int)rc;
+    int out = hip_rc(hipEventRecord(a, g.stream));
+    for (uint32_t i = 0; i < iters && out == CROW_OK; i++) {
+        const unsigned char* w = (const unsigned char*)(uintptr_t)bufs[i % n_bufs];
+        void* args[3] = {(void*)&w, (void*)&units, (void*)&sink};
+        out = hip_rc(hipLaunchKernel((const void*)&pure_read_groups, dim3(blocks), dim3(threads), args, 0, g.stream));
+    }
+    if (out == CROW_OK) out = hip_rc(hipEventRecord(b, g.stream));
+    if (out == CROW_OK) out = hip_rc(hipEventSynchronize(b));
+    float ms = 0.0f;
+    if (out == CROW_OK) out = hip_rc(hipEventElapsedTime(&ms, a, b));
+    (void)hipEventDestroy(a);
+    (void)hipEventDestroy(b);
+    *us_per_launch = ms * 1000.0f / (float)iters;
     return out;
 }
 

@@ -106,6 +106,56 @@ extern "C" __global__ void dequant_fp4_flat(const unsigned char* __restrict__ w,
     out[i] = v.x * s;
 }
 
+// ------------------------------------------------------------------ measurement only: what a pure read of the same bytes takes
+// Reads `units` 2304-byte groups exactly as the GEMVs request them (one dword and two 16-byte non-temporal loads per lane and
+// group, four groups in flight per wave) and does nothing else: the chip's ceiling for this access pattern, measured beside
+// the kernels by the benchmark.  Group i goes to wave i % (all waves of the grid), so any grid covers any size.
+extern "C" __global__ void __launch_bounds__(1024) pure_read_groups(const unsigned char* __restrict__ w, unsigned units, unsigned* __restrict__ sink) {
+    const int lane = lane_id();
+    const unsigned waves = gridDim.x * (blockDim.x >> 6), wave = blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
+    const unsigned count = units > wave ? (units - wave + waves - 1) / waves : 0u;
+    const unsigned char* p = w + (size_t)wave * CROW_GROUP_BYTES;
+    const size_t step = (size_t)waves * CROW_GROUP_BYTES;
+    unsigned sc[4];
+    u32x4 c0[4], c1[4];
+    unsigned q = 0;
+    auto issue = [&](int j) {
+        sc[j] = stream_load_u32((const unsigned*)p + lane);
+        c0[j] = stream_load_v((const uint4*)(p + CROW_GROUP_SCALE_BYTES) + lane);
+        c1[j] = stream_load_v((const uint4*)(p + CROW_GROUP_SCALE_BYTES + 1024) + lane);
+        p += step;
+    };
+    auto use = [&](int j) { q ^= sc[j] ^ c0[j].x ^ c0[j].w ^ c1[j].y ^ c1[j].z; };
+    if (count >= 4) {
+#pragma unroll
+        for (int j = 0; j < 4; j++) issue(j);
+        unsigned left = count - 4;
+        for (; left >= 4; left -= 4) {
+#pragma unroll
+            for (int j = 0; j < 4; j++) {
+                use(j);
+                issue(j);
+            }
+        }
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            use(j);
+            if ((unsigned)j < left) issue(j);
+        }
+#pragma unroll
+        for (int j = 0; j < 4; j++)
+            if ((unsigned)j < left) use(j);
+    } else {
+#pragma unroll
+        for (int j = 0; j < 4; j++)
+            if ((unsigned)j < count) issue(j);
+#pragma unroll
+        for (int j = 0; j < 4; j++)
+            if ((unsigned)j < count) use(j);
+    }
+    if (q == 0x12345677u) sink[0] = q;  // (keeps the loads alive; practically never taken)
+}
+
 // ------------------------------------------------------------------ the NVFP4 encoder (ceiling scales)
 // reference: quantize_nvfp4 in ScalesMode::Ceil, converter/src/main.rs:550-664 with encode_ue4m3_ceil / encode_subblock_ceil
 // (:141-169, :404-410) and e2m1_index (:111-119): f32 values -> container blocks (4 scale bytes + 32 code bytes per 64

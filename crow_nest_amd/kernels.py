@@ -140,6 +140,15 @@ def time_launches(f: int, gx: int, gy: int, gz: int, bx: int, arg_sets, iters: i
     return float(us.value)
 
 
+def time_pure_read(buffers, nbytes: int, blocks: int, threads: int, iters: int) -> float:
+    """Mean microseconds per launch of a kernel that only READS `nbytes` (a multiple of 2304) of each of the device
+    `buffers` in turn, in the GEMVs' own access pattern: the chip's ceiling for that many bytes (measurement only)."""
+    arr = (C.c_uint64 * len(buffers))(*[int(b) for b in buffers])
+    us = C.c_float()
+    _l.check(_l.lib().crow_hip_time_pure_read(arr, len(buffers), nbytes, blocks, threads, iters, C.byref(us)), "crow_hip_time_pure_read")
+    return float(us.value)
+
+
 def time_sequence(kernels, n_sets: int, iters: int) -> float:
     """Mean microseconds per iteration of a launch SEQUENCE.  `kernels` = [(f, (gx, gy, gz, bx), arg_sets), ...];
     every kernel has `n_sets` argument sets (a kernel with one set repeats it); iteration i uses set i % n_sets."""

@@ -84,6 +84,7 @@ def lib():
         "crow_hip_launch_graph": (C.c_int, [vp, vp]),
         "crow_hip_graph_exec_destroy": (C.c_int, [vp]),
         "crow_hip_time_graph": (C.c_int, [vp, vp, u32, C.POINTER(C.c_float)]),
+        "crow_hip_time_pure_read": (C.c_int, [u64p, u32, sz, u32, u32, u32, C.POINTER(C.c_float)]),
         "crow_hip_container_bytes": (sz, [u32, u32]),
         "crow_hip_tiled_bytes": (sz, [u32, u32]),
         "crow_hip_tile_code_offset": (u32, [u32, u32]),
@@ -102,7 +103,7 @@ def lib():
 
 
 # include/crow_hip_bench.h: timing loops and the forced GEMV split, for bench.py and the tests (not part of the drop-in ABI)
-BENCH_EXPORTS = ["crow_hip_launch_dims_split", "crow_hip_time_launches", "crow_hip_time_sequence", "crow_hip_time_graph"]
+BENCH_EXPORTS = ["crow_hip_launch_dims_split", "crow_hip_time_launches", "crow_hip_time_sequence", "crow_hip_time_graph", "crow_hip_time_pure_read"]
 
 EXPORTS = [
     "crow_hip_init", "crow_hip_shutdown", "crow_hip_error_string", "crow_hip_device_name", "crow_hip_module_load",
