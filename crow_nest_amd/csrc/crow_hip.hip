@@ -471,6 +471,9 @@ int crow_hip_launch_dims_split(const char* name, uint32_t rows, uint32_t k_dim, 
             const uint32_t per_wave = e->nr == 2 ? 10 : 7;
             w = (groups + per_wave - 1) / per_wave;
             s = 1;
+            // (The split depends on the tensor's shape only, never on the number of tokens or experts in the launch: a token's
+            // bits are the same in every batch, and the grouped expert kernels reproduce them.  Four waves per tensor at
+            // batch 1 would take routed gate|up [1024, 2048] x 8 experts from 8.0 to 7.2 us and give that up.)
         } else {
             w = 4;
             s = (groups + 13) / 14;
