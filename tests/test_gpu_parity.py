@@ -1130,8 +1130,9 @@ def test_verify_kernels_refuse_more_than_four_rows(eng):
     with pytest.raises(CrowHipError) as ei:  # asked for by its own name, five rows are refused on the host
         launch_dims("gemv_nvfp4_wm", rows, cols, 5)
     assert ei.value.code == -7  # CROW_ERR_SHAPE
-    # dims made for four rows (or for an unknown count), the word behind m_p saying five: refused by the kernel
-    for z in (4, 1):
+    # dims bound to four rows or to one row, and dims that leave the count to the device word (z = 0), the word behind m_p
+    # saying five: a bound launch refuses because the word differs from its count, the unbound one because five is too many
+    for z in (4, 1, 0):
         launch_v(eng.k.f("gemv_nvfp4_wm"), *launch_dims("gemv_nvfp4_wm", rows, cols, z), [f.w_ptr, x.data_ptr(), f.gs_ptr, y.data_ptr(), p.i32(cols), p.i32(rows), p.i32(5)])
         with pytest.raises(CrowHipError) as ei:
             status()
