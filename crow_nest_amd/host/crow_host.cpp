@@ -156,6 +156,20 @@ Fp4 load_fp4(const Nvfp4Matrix& m) {
     status();
     return out;
 }
+QuantizedNvfp4 quantize_nvfp4(const float* values, size_t n_values) {
+    ensure_init();
+    if (n_values % 64 != 0) throw Panic("assertion failed: values.len() % 64 == 0");
+    QuantizedNvfp4 q;
+    q.blocks.resize(n_values / 64 * 36);
+    if (n_values == 0) return q;
+    DevBuf v(n_values * sizeof(float)), b(q.blocks.size()), g(sizeof(float));
+    v.upload(values, n_values * sizeof(float));
+    ck(crow_hip_quantize_nvfp4((const float*)(uintptr_t)v.ptr(), n_values, (void*)(uintptr_t)b.ptr(), (float*)(uintptr_t)g.ptr()), "crow_hip_quantize_nvfp4");
+    b.download(q.blocks.data(), q.blocks.size());
+    g.download(&q.global_scale, sizeof(float));
+    status();
+    return q;
+}
 MlpW load_expert_block(const ExpertBlock& e) {
     MlpW m;
     m.gate = load_fp4(e.gate), m.up = load_fp4(e.up), m.down = load_fp4(e.down);

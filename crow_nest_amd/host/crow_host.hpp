@@ -138,6 +138,15 @@ struct Fp4 {
 Fp4 load_fp4(const Nvfp4Matrix& m);  // upload, re-tile on the device (the 0x7F -> 0x7E scale rule is applied there)
 std::vector<float> dequant(const Fp4& w);  // f32 [rows][cols], bit-exact with the reference decode after the scale rule
 
+// quantize_nvfp4(values, Ceil) of the converter (converter/src/main.rs:534-664) on the device: container blocks (36 bytes per 64
+// values) and the tensor's global scale, byte for byte what the converter writes.  Panics, as the converter's assert does, when
+// the value count is not whole 64-value blocks.
+struct QuantizedNvfp4 {
+    std::vector<uint8_t> blocks;
+    float global_scale = 1.0f;
+};
+QuantizedNvfp4 quantize_nvfp4(const float* values, size_t n_values);
+
 struct MlpW {
     Fp4 gate, up, down;
 };

@@ -220,6 +220,20 @@ static int gemm(const std::string& dir) {
     return 0;
 }
 
+// values.bin (f32) -> blocks.bin, gs.bin through the host layer's encoder; a ragged count must panic with the converter's text
+static int quantize(const std::string& dir) {
+    const std::vector<uint8_t> raw = slurp(dir + "/values.bin");
+    const QuantizedNvfp4 q = quantize_nvfp4((const float*)raw.data(), raw.size() / 4);
+    spit(dir + "/blocks.bin", q.blocks.data(), q.blocks.size());
+    spit(dir + "/gs.bin", &q.global_scale, sizeof(float));
+    try {
+        quantize_nvfp4((const float*)raw.data(), 65);
+    } catch (const Panic& e) {
+        printf("ragged: %s\n", e.what());
+    }
+    return 0;
+}
+
 static int panics() {
     Engine eng;
     try {
@@ -295,8 +309,9 @@ int main(int argc, char** argv) {
         if (cmd == "gemm" && argc == 3) return gemm(argv[2]);
         if (cmd == "moe-grouped" && argc == 3) return moe_grouped(argv[2]);
         if (cmd == "keeps" && argc == 3) return keeps(argv[2]);
+        if (cmd == "quantize" && argc == 3) return quantize(argv[2]);
         if (cmd == "panics") return panics();
-        fprintf(stderr, "usage: host_parity missing | matrix-checks | cnq-list F | cnq-refuse F | cnq-dequant F DIR | dense DIR | head DIR | moe DIR | gemm DIR | panics\n");
+        fprintf(stderr, "usage: host_parity missing | matrix-checks | cnq-list F | cnq-refuse F | cnq-dequant F DIR | dense DIR | head DIR | moe DIR | gemm DIR | quantize DIR | panics\n");
         return 2;
     } catch (const std::exception& e) {
         fprintf(stderr, "host_parity %s: %s\n", cmd.c_str(), e.what());

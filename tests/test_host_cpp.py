@@ -278,6 +278,22 @@ def test_load_fp4_from_the_reference_container_dequantises_bit_exactly(tmp_path)
 
 
 @pytest.mark.gpu
+def test_quantize_nvfp4_through_the_host_layer(tmp_path):
+    """crow::quantize_nvfp4 (the converter's ceiling encoder, converter/src/main.rs:534-664): the blocks and the global scale
+    of the CPU restatement byte for byte, and the converter's assert text for a ragged value count."""
+    d = str(tmp_path)
+    v = normal_f32(77, 4096, 4096 * 64) * np.float32(0.02)
+    v[:64] = 0.0          # an all-zero block
+    v[64] = 3.0           # the tensor's maximum: its sub-block takes the top scale byte
+    _write(d, "values.bin", v)
+    out = run("quantize", d)
+    blocks, gs = orc.quantize_ceil(v)
+    assert np.array_equal(_read(d, "blocks.bin", np.uint8, (-1,)), np.asarray(blocks).reshape(-1))
+    assert _read(d, "gs.bin", np.float32, (1,))[0] == np.float32(gs)
+    assert "ragged: assertion failed: values.len() % 64 == 0" in out
+
+
+@pytest.mark.gpu
 def test_panics_carry_the_reference_texts():
     out = run("panics").splitlines()
     assert out == ["f: kernel missing: gemv_nvfp4_nope", "proj_m: proj_m: M = 5 is outside 1..=4"]
