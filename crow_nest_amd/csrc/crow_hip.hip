@@ -675,9 +675,9 @@ int crow_hip_time_sequence(uint32_t n_kernels, const crow_fn_t* fns, const crow_
     return out;
 }
 
-int crow_hip_time_pure_read(const uint64_t* bufs, uint32_t n_bufs, size_t bytes, uint32_t blocks, uint32_t threads, uint32_t iters, float* us_per_launch) {
+int crow_hip_time_pure_read(const uint64_t* bufs, uint32_t n_bufs, size_t bytes, uint32_t blocks, uint32_t threads, uint32_t pattern, uint32_t iters, float* us_per_launch) {
     if (!g.ready) return CROW_ERR_NOT_INITIALIZED;
-    if (!bufs || !us_per_launch || n_bufs == 0 || iters == 0 || blocks == 0 || threads == 0 || threads % 64 != 0 || threads > 1024) return CROW_ERR_BAD_ARGUMENT;
+    if (!bufs || !us_per_launch || n_bufs == 0 || iters == 0 || blocks == 0 || threads == 0 || threads % 64 != 0 || threads > 1024 || pattern > 2) return CROW_ERR_BAD_ARGUMENT;
     if (bytes == 0 || bytes % CROW_GROUP_BYTES != 0 || bytes / CROW_GROUP_BYTES > 0xFFFFFFFFull) return CROW_ERR_SHAPE;
     unsigned units = (unsigned)(bytes / CROW_GROUP_BYTES);
     unsigned* sink = (unsigned*)(g.scalars + 24);
@@ -688,8 +688,14 @@ int crow_hip_time_pure_read(const uint64_t* bufs, uint32_t n_bufs, size_t bytes,
     int out = hip_rc(hipEventRecord(a, g.stream));
     for (uint32_t i = 0; i < iters && out == CROW_OK; i++) {
         const unsigned char* w = (const unsigned char*)(uintptr_t)bufs[i % n_bufs];
-        void* args[3] = {(void*)&w, (void*)&units, (void*)&sink};
-        out = hip_rc(hipLaunchKernel((const void*)&pure_read_groups, dim3(blocks), dim3(threads), args, 0, g.stream));
+        if (pattern == 0) {
+            void* args[3] = {(void*)&w, (void*)&units, (void*)&sink};
+            out = hip_rc(hipLaunchKernel((const void*)&pure_read_groups, dim3(blocks), dim3(threads), args, 0, g.stream));
+        } else {
+            size_t n16 = bytes / 16;
+            void* args[3] = {(void*)&w, (void*)&n16, (void*)&sink};
+            out = hip_rc(hipLaunchKernel(pattern == 1 ? (const void*)&pure_read_flat_nt : (const void*)&pure_read_flat, dim3(blocks), dim3(threads), args, 0, g.stream));
+        }
     }
     if (out == CROW_OK) out = hip_rc(hipEventRecord(b, g.stream));
     if (out == CROW_OK) out = hip_rc(hipEventSynchronize(b));

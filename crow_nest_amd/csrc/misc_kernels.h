@@ -107,6 +107,33 @@ extern "C" __global__ void dequant_fp4_flat(const unsigned char* __restrict__ w,
 }
 
 // ------------------------------------------------------------------ measurement only: what a pure read of the same bytes takes
+// The textbook streaming read, for comparison with the pattern below: every lane 16 contiguous bytes per load (a wave 1 KB per
+// instruction), eight loads in flight per lane, the grid striding over the buffer; NT = non-temporal loads or plain ones.
+template <bool NT>
+__device__ __forceinline__ void pure_read_flat_body(const uint4* __restrict__ w, size_t n16, unsigned* __restrict__ sink) {
+    const size_t total = (size_t)gridDim.x * blockDim.x;
+    size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    unsigned q = 0;
+    for (; i + 7 * total < n16; i += 8 * total) {
+        u32x4 v[8];
+#pragma unroll
+        for (int j = 0; j < 8; j++) v[j] = NT ? stream_load_v(w + i + j * total) : *(const u32x4*)(w + i + j * total);
+#pragma unroll
+        for (int j = 0; j < 8; j++) q ^= v[j].x ^ v[j].y ^ v[j].z ^ v[j].w;
+    }
+    for (; i < n16; i += total) {
+        const u32x4 v = NT ? stream_load_v(w + i) : *(const u32x4*)(w + i);
+        q ^= v.x ^ v.y ^ v.z ^ v.w;
+    }
+    if (q == 0x9E3779B9u) *sink = q;  // keeps the loads alive; practically never taken
+}
+extern "C" __global__ void __launch_bounds__(1024) pure_read_flat_nt(const uint4* __restrict__ w, size_t n16, unsigned* __restrict__ sink) {
+    pure_read_flat_body<true>(w, n16, sink);
+}
+extern "C" __global__ void __launch_bounds__(1024) pure_read_flat(const uint4* __restrict__ w, size_t n16, unsigned* __restrict__ sink) {
+    pure_read_flat_body<false>(w, n16, sink);
+}
+
 // Reads `units` 2304-byte groups exactly as the GEMVs request them (one dword and two 16-byte non-temporal loads per lane and
 // group, four groups in flight per wave) and does nothing else: the chip's ceiling for this access pattern, measured beside
 // the kernels by the benchmark.  Group i goes to wave i % (all waves of the grid), so any grid covers any size.

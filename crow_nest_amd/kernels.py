@@ -140,12 +140,13 @@ def time_launches(f: int, gx: int, gy: int, gz: int, bx: int, arg_sets, iters: i
     return float(us.value)
 
 
-def time_pure_read(buffers, nbytes: int, blocks: int, threads: int, iters: int) -> float:
+def time_pure_read(buffers, nbytes: int, blocks: int, threads: int, iters: int, pattern: int = 0) -> float:
     """Mean microseconds per launch of a kernel that only READS `nbytes` (a multiple of 2304) of each of the device
-    `buffers` in turn, in the GEMVs' own access pattern: the chip's ceiling for that many bytes (measurement only)."""
+    `buffers` in turn: the chip's ceiling for that many bytes (measurement only).  pattern 0 = the GEMVs' own requests
+    (2304-byte groups, four in flight per wave), 1 = 16 contiguous bytes per lane, non-temporal, 2 = the same, plain loads."""
     arr = (C.c_uint64 * len(buffers))(*[int(b) for b in buffers])
     us = C.c_float()
-    _l.check(_l.lib().crow_hip_time_pure_read(arr, len(buffers), nbytes, blocks, threads, iters, C.byref(us)), "crow_hip_time_pure_read")
+    _l.check(_l.lib().crow_hip_time_pure_read(arr, len(buffers), nbytes, blocks, threads, pattern, iters, C.byref(us)), "crow_hip_time_pure_read")
     return float(us.value)
 
 

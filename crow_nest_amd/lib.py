@@ -84,7 +84,7 @@ def lib():
         "crow_hip_launch_graph": (C.c_int, [vp, vp]),
         "crow_hip_graph_exec_destroy": (C.c_int, [vp]),
         "crow_hip_time_graph": (C.c_int, [vp, vp, u32, C.POINTER(C.c_float)]),
-        "crow_hip_time_pure_read": (C.c_int, [u64p, u32, sz, u32, u32, u32, C.POINTER(C.c_float)]),
+        "crow_hip_time_pure_read": (C.c_int, [u64p, u32, sz, u32, u32, u32, u32, C.POINTER(C.c_float)]),
         "crow_hip_container_bytes": (sz, [u32, u32]),
         "crow_hip_tiled_bytes": (sz, [u32, u32]),
         "crow_hip_tile_code_offset": (u32, [u32, u32]),

@@ -28,12 +28,14 @@ int crow_hip_time_launches(crow_fn_t f, uint32_t gx, uint32_t gy, uint32_t gz, u
 int crow_hip_time_sequence(uint32_t n_kernels, const crow_fn_t* fns, const crow_dims* dims, const uint32_t* n_vals,
                            const uint64_t* vals, uint32_t n_sets, uint32_t iters, float* us_per_iteration);
 
-/* What a PURE READ of `bytes` (a multiple of 2304) takes on this device in the GEMVs' own access pattern - the same three
- * non-temporal loads per lane and 2304-byte group, four groups in flight per wave - with nothing else in the kernel: `iters`
- * back-to-back launches of (blocks x threads) between two events, launch i reading the device buffer bufs[i % n_bufs]
- * (rotating copies, as above).  The benchmark reports it beside each kernel as the chip's ceiling for that many bytes. */
-int crow_hip_time_pure_read(const uint64_t* bufs, uint32_t n_bufs, size_t bytes, uint32_t blocks, uint32_t threads, uint32_t iters,
-                            float* us_per_launch);
+/* What a PURE READ of `bytes` (a multiple of 2304) takes on this device with nothing else in the kernel: `iters` back-to-back
+ * launches of (blocks x threads) between two events, launch i reading the device buffer bufs[i % n_bufs] (rotating copies, as
+ * above).  pattern 0: the GEMVs' own access pattern - the same three non-temporal loads per lane and 2304-byte group, four groups
+ * in flight per wave; pattern 1: the textbook stream - 16 contiguous bytes per lane and load, eight loads in flight per lane,
+ * non-temporal; pattern 2: the same with plain loads.  The benchmark reports the best of them beside each kernel as the chip's
+ * ceiling for that many bytes. */
+int crow_hip_time_pure_read(const uint64_t* bufs, uint32_t n_bufs, size_t bytes, uint32_t blocks, uint32_t threads, uint32_t pattern,
+                            uint32_t iters, float* us_per_launch);
 
 /* `iters` back-to-back replays on `stream` between two events; mean microseconds per replay */
 int crow_hip_time_graph(void* graph_exec, void* stream, uint32_t iters, float* us_per_replay);
