@@ -819,11 +819,12 @@ int crow_hip_quantize_nvfp4(const float* values_dev, size_t n_values, void* bloc
     // row do not share it)
     static int slot = 0;
     unsigned* max_bits = (unsigned*)(g.scalars + 16 + (slot++ & 7));
-    hipError_t e = hipMemsetAsync(max_bits, 0, sizeof(unsigned), g.stream);
-    if (e != hipSuccess) return (int)e;
+    hipError_t e;
+    void* a0[1] = {(void*)&max_bits};
+    if ((e = hipLaunchKernel((const void*)&quantize_nvfp4_clear, dim3(1), dim3(1), a0, 0, g.stream)) != hipSuccess) return (int)e;
     unsigned long long n_sub = n_values / 16;
     const unsigned long long want = (n_sub + 255) / 256;
-    const unsigned blocks1 = (unsigned)(want < 8192 ? want : 8192);
+    const unsigned blocks1 = (unsigned)(want < 2048 ? want : 2048);
     const float* vals = values_dev;
     unsigned char* out = (unsigned char*)blocks_dev;
     const unsigned* max_ro = max_bits;

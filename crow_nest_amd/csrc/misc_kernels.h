@@ -210,31 +210,41 @@ __device__ __forceinline__ unsigned ue4m3_ceil_byte(float r) {
 __device__ __forceinline__ float ue4m3_value(unsigned byte) {  // decode_ue4m3 (bytes 0..0x7F; 0x7F = 480)
     return __uint_as_float((byte & 0x7Fu) << 20) * 0x1p120f;
 }
-// amax / 6 of the 16 values at `v` (f32::max ignores a NaN operand, like fmaxf)
-__device__ __forceinline__ float subblock_raw(const float4 (&q)[4]) {
+// the largest |v| of 16 values (f32::max ignores a NaN operand, like fmaxf), and the sub-block's raw scale: that over 6
+__device__ __forceinline__ float subblock_amax(const float4 (&q)[4]) {
     float m = 0.0f;
 #pragma unroll
     for (int i = 0; i < 4; i++) m = fmaxf(fmaxf(fmaxf(fmaxf(m, fabsf(q[i].x)), fabsf(q[i].y)), fabsf(q[i].z)), fabsf(q[i].w));
-    return __fdiv_rn(m, 6.0f);
+    return m;
 }
-// pass 1: the largest raw scale of the tensor, as the bit pattern of a non-negative f32 (they order like unsigned integers)
-// grid-stride over the n / 16 sub-blocks; *max_bits starts as 0
+__device__ __forceinline__ float subblock_raw(const float4 (&q)[4]) { return __fdiv_rn(subblock_amax(q), 6.0f); }
+// pass 1: the largest |value| of the tensor, as the bit pattern of a non-negative f32 (they order like unsigned integers).
+// The largest raw scale is that maximum over 6: a correctly rounded division is monotonic, so the maximum of the quotients is
+// the quotient of the maximum, bit for bit.  Grid-stride over the n / 16 sub-blocks, one atomic per block; *max_bits starts
+// as 0 (quantize_nvfp4_clear: a kernel rather than a memset, so that the three launches can be captured into a graph).
+extern "C" __global__ void quantize_nvfp4_clear(unsigned* __restrict__ max_bits) { *max_bits = 0u; }
 extern "C" __global__ void __launch_bounds__(256) quantize_nvfp4_amax(const float* __restrict__ values, unsigned long long n_sub,
                                                                        unsigned* __restrict__ max_bits) {
+    __shared__ float per_wave[4];
     float best = 0.0f;
     for (unsigned long long i = (unsigned long long)blockIdx.x * blockDim.x + threadIdx.x; i < n_sub; i += (unsigned long long)gridDim.x * blockDim.x) {
         const float4* p = (const float4*)(values + 16 * i);
         const float4 q[4] = {p[0], p[1], p[2], p[3]};
-        best = fmaxf(best, subblock_raw(q));
+        best = fmaxf(best, subblock_amax(q));
     }
     for (int o = 32; o > 0; o >>= 1) best = fmaxf(best, __shfl_xor(best, o));
-    if ((threadIdx.x & 63u) == 0 && best > 0.0f) atomicMax(max_bits, __float_as_uint(best));
+    if ((threadIdx.x & 63u) == 0) per_wave[threadIdx.x >> 6] = best;
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        best = fmaxf(fmaxf(per_wave[0], per_wave[1]), fmaxf(per_wave[2], per_wave[3]));
+        if (best > 0.0f) atomicMax(max_bits, __float_as_uint(best));
+    }
 }
 // pass 2: one thread per sub-block: its scale byte and its sixteen codes; thread 0 also leaves the global scale
 extern "C" __global__ void __launch_bounds__(256) quantize_nvfp4_encode(const float* __restrict__ values, unsigned long long n_sub,
                                                                          const unsigned* __restrict__ max_bits, unsigned char* __restrict__ blocks,
                                                                          float* __restrict__ global_out) {
-    const float max_scale = __uint_as_float(*max_bits);
+    const float max_scale = __fdiv_rn(__uint_as_float(*max_bits), 6.0f);  // the largest raw scale (see pass 1)
     const float global = max_scale > 0.0f ? __fdiv_rn(max_scale, 448.0f) : 1.0f;
     const unsigned long long i = (unsigned long long)blockIdx.x * blockDim.x + threadIdx.x;
     if (i == 0) global_out[0] = global;
