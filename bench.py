@@ -89,6 +89,11 @@ def med_min(ts):
     return ts[len(ts) // 2], ts[0]
 
 
+# sha256 (first 16 hex digits) of the three container byte strings and of the bf16 activations, recorded from runs in which the
+# CPU restatement of the converter's ceiling encoder built the inputs (same generator, same seeds)
+CPU_ENCODER_SHA256_16 = {"gate": "fac61cbbd89ba7f6", "up": "c5cddfd1cd12470a", "down": "140d0096e7183bfa", "x_bf16": "efb063872d27b714"}
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -294,6 +299,9 @@ def main() -> int:
                    "config0": config0,
                    "inputs": {"generator": "splitmix64 + Box-Muller, seed 0, one stream per tensor; W ~ N(0, 0.02^2) through the library's ceiling "
                                            "encoder on the device (crow_hip_quantize_nvfp4), x ~ N(0, 1) rounded to bf16", "sha256_16": input_sha256,
+                              # what the CPU restatement of the converter's encoder (and torch's bf16 rounding) gave for the same
+                              # streams when it still built these inputs: the device encoder's bytes must be the same bytes
+                              "equal_to_the_cpu_encoder_s_bytes": input_sha256 == CPU_ENCODER_SHA256_16,
                               "global_scales": {nm: float(np.float32(host[nm][1])) for nm in host}},
                    "device": name_buf.value.decode(), "input_generation_s": round(gen_s, 1)},
         "roofline": roof,
