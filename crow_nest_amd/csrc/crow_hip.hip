@@ -1,6 +1,7 @@
 // libcrow_hip.so: gfx950 code objects (built ahead of time from the headers below) and the C ABI
 // declared in include/crow_hip.h.  One translation unit, so the device globals are shared.
 #include <hip/hip_runtime.h>
+#include <atomic>
 #include <cstdio>
 #include <cstdlib>
 #include <cstring>
@@ -817,8 +818,8 @@ int crow_hip_quantize_nvfp4(const float* values_dev, size_t n_values, void* bloc
     if (n_values == 0 || n_values % CROW_BLOCK_VALUES != 0) return CROW_ERR_SHAPE;
     // the tensor's largest raw scale meets in one device word (one of the library's own, taken in turn so that calls in a
     // row do not share it)
-    static int slot = 0;
-    unsigned* max_bits = (unsigned*)(g.scalars + 16 + (slot++ & 7));
+    static std::atomic<unsigned> slot{0};
+    unsigned* max_bits = (unsigned*)(g.scalars + 16 + (slot.fetch_add(1) & 7u));
     hipError_t e;
     void* a0[1] = {(void*)&max_bits};
     if ((e = hipLaunchKernel((const void*)&quantize_nvfp4_clear, dim3(1), dim3(1), a0, 0, g.stream)) != hipSuccess) return (int)e;
