@@ -398,6 +398,171 @@ struct StripWalk {
     }
 };
 
+// StripWalk for bf16 activations with the activation traffic halved: a lane asks for 8 columns (16 bytes) of a PAIR of groups
+// at once - lanes 0..31 cover the pair's first group, lanes 32..63 its second - and one 16-byte LDS store per row stages both
+// groups' rows (the staged bytes, the operand reads and every sum are StripWalk's: same bits).  Per group that is 3.5 vector
+// memory instructions instead of 4 and half an LDS store instead of one.  The activation rows must be 16-byte aligned.
+#ifndef CROW_BF16_XPAIRS
+#define CROW_BF16_XPAIRS 1
+#endif
+template <int M>
+struct StripWalkPairs {
+    typedef Staging<M, true> St;
+    unsigned sc[CROW_GEMV_RING][1];
+    u32x4 cd[CROW_GEMV_RING][1][2];
+    u32x4 xp[2][M];           // pair slot P holds groups 4 q + 2 P, 4 q + 2 P + 1
+    lds_p a1[2][1], a2[2][1];
+    lds_p xw;
+    const unsigned char* wl;
+    const unsigned char* xl;
+    size_t xoff[M];
+    int col_lane, k_dim, lane;
+    float acc[1][M];
+
+    __device__ __forceinline__ void init(const unsigned char* strip, int first, int k_dim_, const void* x, const size_t (&xoff_elems)[M], lds_p xw_,
+                                         lds_p zero) {
+        lane = lane_id();
+        xw = xw_;
+        k_dim = k_dim_;
+        wl = strip + (size_t)first * CROW_GROUP_BYTES;
+        col_lane = first * CROW_GROUP_COLS + 8 * lane;
+        xl = (const unsigned char*)x;
+#pragma unroll
+        for (int m = 0; m < M; m++) {
+            xoff[m] = xoff_elems[m] * 2;
+            acc[0][m] = 0.0f;
+        }
+        const int g = lane >> 4, i = lane & 15, r4 = i & 3;
+        const bool half_ok = (g >> 1) == (i >> 3);
+        const bool second = ((i >> 2) & 1) != 0;
+#pragma unroll
+        for (int s = 0; s < 2; s++) {
+            const bool live = half_ok && r4 < St::XR;
+            lds_p data = xw + s * St::SLOT + r4 * CROW_GEMV_XROW_BYTES + 16 * g;
+            a1[s][0] = (live && !second) ? data : zero + 16 * g;
+            a2[s][0] = (live && second) ? data + 64 : zero + 16 * g;
+        }
+    }
+    // activations of groups g, g + 1 (g even in the wave's own count) into pair slot P
+    template <int P>
+    __device__ __forceinline__ void issue_xp(int g) {
+        const int col = col_lane + g * CROW_GROUP_COLS;
+        const size_t o = (size_t)(col < k_dim ? col : k_dim - 8) * 2;
+#pragma unroll
+        for (int t = 0; t < M; t++) xp[P][t] = *(const __attribute__((address_space(1))) u32x4*)(xl + xoff[t] + o);
+    }
+    template <int J>
+    __device__ __forceinline__ void issue_w(int g) {
+        const unsigned char* p = wl + (size_t)g * CROW_GROUP_BYTES;
+        sc[J][0] = stream_load_u32((const unsigned*)p + lane);
+        cd[J][0][0] = stream_load_v((const uint4*)(p + CROW_GROUP_SCALE_BYTES) + lane);
+        cd[J][0][1] = stream_load_v((const uint4*)(p + CROW_GROUP_SCALE_BYTES + 1024) + lane);
+    }
+    // pair slot P -> the two LDS staging slots (group g into slot 0, group g + 1 into slot 1)
+    template <int P>
+    __device__ __forceinline__ void stage_pair(int g) {
+        const bool in = col_lane + g * CROW_GROUP_COLS < k_dim;
+        lds_p dst = xw + (lane >> 5) * St::SLOT + 16 * (lane & 31);
+#pragma unroll
+        for (int t = 0; t < M; t++)
+            lds_store16(dst + t * CROW_GEMV_XROW_BYTES, in ? xp[P][t].x : 0u, in ? xp[P][t].y : 0u, in ? xp[P][t].z : 0u, in ? xp[P][t].w : 0u);
+        __builtin_amdgcn_wave_barrier();
+    }
+    template <int J>
+    __device__ __forceinline__ void multiply() {
+        group_multiply<M, true, 1>(sc[J], cd[J], a1[J & 1], a2[J & 1], acc);
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_sched_barrier(0);
+    }
+    template <int N>
+    __device__ __forceinline__ void start(int g) {
+        if (N > 0) issue_xp<0>(g);
+        if (N > 2) issue_xp<1>(g + 2);
+        if (N > 0) issue_w<0>(g);
+        if (N > 1) issue_w<1>(g + 1);
+        if (N > 2) issue_w<2>(g + 2);
+        if (N > 3) issue_w<3>(g + 3);
+    }
+    // On entry: the weights of g0 .. g0 + 3 are in (or on their way to) slots 0..3, the pair (g0, g0 + 1) is staged, pair slot 1
+    // holds (or awaits) g0 + 2, g0 + 3 and pair slot 0 g0 + 4, g0 + 5.  Requests beyond the wave's run read columns that exist
+    // (or the row's last eight) and are never used.  On return the pair (g0 + 4, g0 + 5) is staged if REFILL.
+    template <bool REFILL>
+    __device__ __forceinline__ void quad(int g0) {
+        multiply<0>();
+        if (REFILL) issue_w<0>(g0 + 4);
+        multiply<1>();
+        if (REFILL) issue_w<1>(g0 + 5);
+        stage_pair<1>(g0 + 2);
+        issue_xp<1>(g0 + 6);
+        multiply<2>();
+        if (REFILL) issue_w<2>(g0 + 6);
+        multiply<3>();
+        if (REFILL) {
+            issue_w<3>(g0 + 7);
+            stage_pair<0>(g0 + 4);
+            issue_xp<0>(g0 + 8);
+        }
+    }
+    template <int N>
+    __device__ __forceinline__ void rest(int g0) {
+        if (N > 0) multiply<0>();
+        if (N > 1) multiply<1>();
+        if (N > 2) {
+            stage_pair<1>(g0 + 2);
+            multiply<2>();
+        }
+    }
+    template <int N>
+    __device__ __forceinline__ void remainder(int g) {
+        start<N>(g);
+        stage_pair<0>(g);
+        rest<N>(g);
+    }
+    template <class Mid>
+    __device__ __forceinline__ void go(int count, Mid mid) {
+        const int nq = count >> 2, r = count & 3;
+        if (nq > 0) {
+            start<4>(0);
+            mid();
+            stage_pair<0>(0);
+            issue_xp<0>(4);
+            int q = 0;
+            for (; q + 1 < nq; q++) quad<true>(4 * q);
+            quad<false>(4 * q);
+            if (r == 3) remainder<3>(4 * nq);
+            else if (r == 2) remainder<2>(4 * nq);
+            else if (r == 1) remainder<1>(4 * nq);
+        } else if (r == 3) {
+            start<3>(0);
+            mid();
+            stage_pair<0>(0);
+            rest<3>(0);
+        } else if (r == 2) {
+            start<2>(0);
+            mid();
+            stage_pair<0>(0);
+            rest<2>(0);
+        } else if (r == 1) {
+            start<1>(0);
+            mid();
+            stage_pair<0>(0);
+            rest<1>(0);
+        } else {
+            mid();
+        }
+    }
+    __device__ __forceinline__ void finish(float (&out)[M]) const {
+#pragma unroll
+        for (int m = 0; m < M; m++) {
+            const unsigned a = __float_as_uint(acc[0][m]);
+            const u32x2 sw = __builtin_amdgcn_permlane32_swap(a, a, false, false);
+            const unsigned b = __float_as_uint(__fadd_rn(__uint_as_float(sw.x), __uint_as_float(sw.y)));
+            const u32x2 sq = __builtin_amdgcn_permlane16_swap(b, b, false, false);
+            out[m] = __fadd_rn(__uint_as_float(sq.x), __uint_as_float(sq.y));
+        }
+    }
+};
+
 // The walk of a wave that takes NS adjacent strips at once (the kernels for several activation rows): per group the staged
 // activations and the operand reads from LDS serve NS x 16 weight rows, which is what bounds those kernels - at four f32 rows a
 // group's operand reads are ten times its weight bytes.  Two groups (NS x 2304 bytes each) in flight; per strip and
@@ -819,7 +984,7 @@ __device__ __forceinline__ void gemv_body(const GemvArgs& a, unsigned z, lds_p l
     };
     float part[NS][M];
     if constexpr (NS == 1) {
-        StripWalk<M, XBF16> walk;
+        typename std::conditional<XBF16 && CROW_BF16_XPAIRS != 0, StripWalkPairs<M>, StripWalk<M, XBF16>>::type walk;
         walk.init(wsel + (size_t)strip * groups * CROW_GROUP_BYTES, first, k_dim, a.x, xoff, areas + wave * AREA, zero);
         walk.go(count, mid);
         walk.finish(part[0]);

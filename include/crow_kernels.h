@@ -13,7 +13,7 @@
  * Conventions shared by all entries:
  *   w, wg, wu   NVFP4 tensors in the library's tiled layout (crow_hip_repack_nvfp4), never raw container bytes
  *   gs, gs_*    one f32 per tensor: the global scale (PW::Fp4's second word, engine/src/gen.rs:234-237)
- *   x           activations, row-major [tokens][k_dim]: f32 unless the entry is a *_bf16 twin (then bf16)
+ *   x           activations, row-major [tokens][k_dim]: f32 unless the entry is a *_bf16 twin (then bf16); 16-byte aligned
  *   y           f32 outputs, row-major [tokens][rows]
  *   A shape a kernel cannot serve sets a bit of the device status word (read by crow_hip_status) and the launch
  *   writes nothing; no kernel traps.
