@@ -875,7 +875,9 @@ struct TileWalk {
 // Ordering point of the cross-block hand-over.  Every access to the shared partials and counters is an agent-scope atomic:
 // the partials are only written by atomic stores and read by atomic loads, which on gfx950 carry the coherence bit that
 // makes them bypass the per-die L2 for data other dies may touch; the counters are only touched by read-modify-write
-// atomics, which are coherent among themselves (never read a counter with a load: that pairing has no evidence here).  What is left to guarantee is
+// atomics, which are coherent among themselves.  Never read a counter with a load, atomic or not: it does not see the other
+// dies' updates (measured: a polling loop of atomic loads never saw them) - and the compiler turns a read-modify-write with a
+// constant identity operand (fetch_add(p, 0)) into exactly such a load.  What is left to guarantee is
 // program order between them, which a wait for this wave's outstanding memory operations gives: the partial stores are
 // acknowledged before the arrival counter is bumped, and the counter's value is back before any partial is read.  An
 // agent-scope fence would add a write-back (release) or an invalidate (acquire) of the whole L2 to exactly this wait;
